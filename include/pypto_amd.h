@@ -1,0 +1,133 @@
+/*
+ * pypto_amd.h - C ABI of the MI355X-native DeepSeek-V3.2 sparse decode-attention operators.
+ *
+ * The library (libpypto_amd.so, built from pypto_amd/csrc with hipcc for gfx950) is the drop-in
+ * boundary for three operator families of the reference's models/deepseek_v32_exp directory.  Each
+ * operator is a workspace-query / launch pair over one flat tensor list, the calling convention of the
+ * reference's ahead-of-time kernel bundle ABI (framework/include/tile_fwk_bundle/pypto_bundle_api.h:30-51):
+ * the tensor list holds every operand, outputs included, in the positional order of the Python entry
+ * point it replaces; the launch is asynchronous on the caller's HIP stream; 0 means success.
+ *
+ * Tensor descriptors use the reference's layout (pypto_bundle_api.h:30-35) and its DataType numbering
+ * (framework/include/tilefwk/data_type.h:33-65).  All tensors are dense row-major device memory on the
+ * current device.  No entry point synchronises the stream; none allocates device memory: scratch comes
+ * from the caller through `workspace` (reference: python/src/bindings/runtime.cpp:697-702, where the
+ * workspace is a torch allocation made by the caller's side of the binding).
+ */
+#ifndef PYPTO_AMD_H
+#define PYPTO_AMD_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* framework/include/tile_fwk_bundle/pypto_bundle_api.h:30-35 */
+typedef struct {
+    void* addr;       /* device address */
+    int32_t dataType; /* PtoDataType */
+    int32_t rank;
+    int64_t shape[8];
+} PtoTensorDesc;
+
+/* framework/include/tilefwk/data_type.h:33-65 (positions in the DataType enum) */
+enum PtoDataType { PTO_DT_INT8 = 1, PTO_DT_INT32 = 3, PTO_DT_FP16 = 6, PTO_DT_FP32 = 7, PTO_DT_BF16 = 8 };
+
+/* Error codes (negative).  pto_last_error() gives the message of the calling thread's last failure. */
+enum PtoStatus {
+    PTO_OK = 0,
+    PTO_ERR_ARG_COUNT = -1, /* wrong number of tensors */
+    PTO_ERR_DTYPE = -2,     /* a tensor has the wrong dtype */
+    PTO_ERR_SHAPE = -3,     /* rank/shape mismatch between operands or with the parameters */
+    PTO_ERR_PARAM = -4,     /* unsupported scalar parameter */
+    PTO_ERR_WORKSPACE = -5, /* workspace missing or too small */
+    PTO_ERR_NULL = -6,      /* null device address */
+    PTO_ERR_HIP = -7        /* the HIP runtime reported an error on launch */
+};
+
+/* Scalar arguments of sparse_flash_attention_quant_* / sparse_attention_antiquant_*
+ * (models/deepseek_v32_exp/sparse_flash_attention_quant_impl.py:655-674: nq, n_kv, softmax_scale, topk,
+ * block_size, max_blocknum_perbatch; the trailing tile_config holds Ascend tiling knobs and has no
+ * counterpart here). */
+typedef struct {
+    int32_t nq;
+    int32_t n_kv;
+    float softmax_scale;
+    int32_t topk;
+    int32_t block_size;
+    int32_t max_blocknum_perbatch;
+    int32_t kv_splits; /* 0 = choose from the problem size; >0 forces the number of KV splits per query token */
+} PtoSfaParams;
+
+/* Scalar arguments of lightning_indexer_decode
+ * (models/deepseek_v32_exp/lightning_indexer_quant_impl.py:226-238: selected_count; unroll_list and
+ * configs are Ascend tiling knobs - the only semantic field, extend_param scale = 1/2048 with ReLU,
+ * models/deepseek_v32_exp/deepseekv32_lightning_indexer_quant.py:43, is fixed in the kernels). */
+typedef struct {
+    int32_t selected_count;
+} PtoIndexerParams;
+
+/*
+ * sparse_flash_attention_quant_d / _p / _d_950
+ * (models/deepseek_v32_exp/sparse_flash_attention_quant_impl.py:572-591,655-674,734-753).
+ * tensors[9], in order:
+ *   0 query_nope    [t*nq, 512]      BF16
+ *   1 query_rope    [t*nq, 64]       BF16
+ *   2 key_nope_2d   [N, 512]         INT8 (quantised cache) or BF16
+ *   3 key_rope_2d   [N, 64]          BF16
+ *   4 k_nope_scales [N, 4]           FP32 (one scale per 128 nope columns; ignored for a BF16 cache)
+ *   5 topk_indices  [t, n_kv*topk]   INT32 (entries past a token's valid length are ignored)
+ *   6 block_table   [b, max_blocknum_perbatch] INT32 (-1 = unused)
+ *   7 kv_act_seqs   [b]              INT32
+ *   8 attention_out [b, s1, nq, 512] BF16 (output)
+ */
+uint64_t pto_sfa_quant_workspace(const PtoTensorDesc* tensors, uint32_t n_tensors, const PtoSfaParams* params);
+int pto_sfa_quant_launch(const PtoTensorDesc* tensors, uint32_t n_tensors, const PtoSfaParams* params,
+                         void* workspace, uint64_t workspace_bytes, void* hip_stream);
+
+/*
+ * sparse_attention_antiquant_d / _p / _d_950
+ * (models/deepseek_v32_exp/sparse_attention_antiquant_impl.py:287-302,358-373,739-749).
+ * tensors[7], in order:
+ *   0 query_nope    [t*nq, 512] BF16
+ *   1 query_rope    [t*nq, 64]  BF16
+ *   2 nope_cache    [N, 656]    INT8: bytes 0..511 int8 nope | 512..639 64 x bf16 rope | 640..655 4 x fp32 scales
+ *   3 topk_indices  [t, n_kv*topk] INT32
+ *   4 block_table   [b, max_blocknum_perbatch] INT32
+ *   5 kv_act_seqs   [b] INT32
+ *   6 attention_out [t*nq, 512] BF16 (output)
+ */
+uint64_t pto_sfa_antiquant_workspace(const PtoTensorDesc* tensors, uint32_t n_tensors, const PtoSfaParams* params);
+int pto_sfa_antiquant_launch(const PtoTensorDesc* tensors, uint32_t n_tensors, const PtoSfaParams* params,
+                             void* workspace, uint64_t workspace_bytes, void* hip_stream);
+
+/*
+ * lightning_indexer_decode (models/deepseek_v32_exp/lightning_indexer_quant_impl.py:226-238).
+ * tensors[8], in order:
+ *   0 idx_query       [t, 64, 128]            INT8
+ *   1 idx_query_scale [t, 64]                 FP16
+ *   2 idx_key_cache   [blocks, block_size, 1, 128] INT8
+ *   3 idx_key_scale   [blocks, block_size, 1] FP16
+ *   4 idx_weight      [t, 64]                 FP16
+ *   5 act_seq_key     [b]                     INT32
+ *   6 block_table     [b, max_blocks]         INT32
+ *   7 topk_res        [t, 1, selected_count]  INT32 (output; -1 beyond a token's valid length)
+ */
+uint64_t pto_lightning_indexer_workspace(const PtoTensorDesc* tensors, uint32_t n_tensors,
+                                         const PtoIndexerParams* params);
+int pto_lightning_indexer_launch(const PtoTensorDesc* tensors, uint32_t n_tensors, const PtoIndexerParams* params,
+                                 void* workspace, uint64_t workspace_bytes, void* hip_stream);
+
+/* Message of the calling thread's most recent failed call ("" if none).  Replaces the message strings
+ * the reference's binding layer returns (python/src/bindings/runtime.cpp:270-335). */
+const char* pto_last_error(void);
+
+/* ABI version of this header. */
+int pto_abi_version(void);
+
+#ifdef __cplusplus
+}
+#endif
+
+#endif /* PYPTO_AMD_H */

@@ -1,0 +1,169 @@
+"""Host side of the operator boundary: torch tensors -> C ABI of libpypto_amd.so.
+
+Plays the role of the reference's call path ``JitCallableWrapper.__call__`` ->
+``LaunchKernelTorch`` (python/pypto/frontend/parser/entry.py:296-365,518-583,638-662 and
+python/src/bindings/runtime.cpp:625-723): split positional/keyword arguments into tensors and
+scalars, check that every tensor is a contiguous torch.Tensor on one device, allocate the workspace
+through the torch allocator and launch asynchronously on the caller's current stream.  PyTorch is
+used for device memory and streams only; all compute is in the HIP library.
+"""
+import ctypes
+import functools
+import os
+import threading
+
+import torch
+
+from .error import FeError, PyptoError, PyptoRtError
+
+_LIB_PATH = os.path.join(os.path.dirname(os.path.abspath(__file__)), "libpypto_amd.so")
+_lib = None
+_lib_lock = threading.Lock()
+
+
+class TensorDesc(ctypes.Structure):
+    _fields_ = [("addr", ctypes.c_void_p), ("dataType", ctypes.c_int32), ("rank", ctypes.c_int32),
+                ("shape", ctypes.c_int64 * 8)]
+
+
+class SfaParams(ctypes.Structure):
+    _fields_ = [("nq", ctypes.c_int32), ("n_kv", ctypes.c_int32), ("softmax_scale", ctypes.c_float),
+                ("topk", ctypes.c_int32), ("block_size", ctypes.c_int32),
+                ("max_blocknum_perbatch", ctypes.c_int32), ("kv_splits", ctypes.c_int32)]
+
+
+class IndexerParams(ctypes.Structure):
+    _fields_ = [("selected_count", ctypes.c_int32)]
+
+
+# framework/include/tilefwk/data_type.h:33-65
+_DTYPE_CODE = {torch.int8: 1, torch.int32: 3, torch.float16: 6, torch.float32: 7, torch.bfloat16: 8}
+
+_OPS = {
+    "sfa_quant": SfaParams,
+    "sfa_antiquant": SfaParams,
+    "lightning_indexer": IndexerParams,
+}
+
+# C status -> Python exception type wrapped by FeError
+_STATUS_EXC = {-1: RuntimeError, -2: ValueError, -3: ValueError, -4: ValueError, -5: RuntimeError, -6: RuntimeError,
+               -7: RuntimeError}
+
+
+def library_path():
+    return _LIB_PATH
+
+
+def load_library():
+    """Load libpypto_amd.so (built in-tree by ``python -m pypto_amd.build``).  There is no fallback:
+    without the library every operator call fails."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    with _lib_lock:
+        if _lib is not None:
+            return _lib
+        if not os.path.exists(_LIB_PATH):
+            raise PyptoRtError(RuntimeError(
+                f"{_LIB_PATH} is missing: build it with `python -m pypto_amd.build` (hipcc, gfx950)"))
+        lib = ctypes.CDLL(_LIB_PATH)
+        for op, ptype in _OPS.items():
+            ws = getattr(lib, f"pto_{op}_workspace")
+            ws.restype = ctypes.c_uint64
+            ws.argtypes = [ctypes.POINTER(TensorDesc), ctypes.c_uint32, ctypes.POINTER(ptype)]
+            ln = getattr(lib, f"pto_{op}_launch")
+            ln.restype = ctypes.c_int
+            ln.argtypes = [ctypes.POINTER(TensorDesc), ctypes.c_uint32, ctypes.POINTER(ptype), ctypes.c_void_p,
+                           ctypes.c_uint64, ctypes.c_void_p]
+        lib.pto_last_error.restype = ctypes.c_char_p
+        lib.pto_last_error.argtypes = []
+        lib.pto_abi_version.restype = ctypes.c_int
+        _lib = lib
+    return _lib
+
+
+def describe(tensors):
+    descs = (TensorDesc * len(tensors))()
+    for d, t in zip(descs, tensors):
+        code = _DTYPE_CODE.get(t.dtype)
+        if code is None:
+            raise ValueError(f"unsupported tensor dtype {t.dtype}")
+        if t.dim() > 8:
+            raise ValueError("tensors of more than 8 dimensions are not supported")
+        d.addr = t.data_ptr() if t.numel() else None
+        d.dataType = code
+        d.rank = t.dim()
+        for i, s in enumerate(t.shape):
+            d.shape[i] = s
+    return descs
+
+
+def _validate_tensors(tensors):
+    for idx, t in enumerate(tensors):
+        if not isinstance(t, torch.Tensor):
+            raise FeError(RuntimeError(f"Input {idx + 1} (index {idx}) must be a torch.Tensor, got {t.__class__}"))
+        if type(t).__name__ == "DTensor":
+            raise FeError(RuntimeError(f"Input {idx + 1} (index {idx}) must not be a DTensor, got {t.__class__}"))
+        if not t.is_contiguous():
+            raise FeError(RuntimeError("not all tensors are contiguous"))
+    dev = tensors[0].device
+    for t in tensors:
+        if t.device != dev:
+            raise FeError(RuntimeError(f"all tensors must be on the same device, got {dev} and {t.device}"))
+    if dev.type != "cuda":
+        raise FeError(RuntimeError(f"tensors must be on a HIP device (torch device type 'cuda'), got {dev}"))
+    return dev
+
+
+def launch(op, tensors, params):
+    """Validate, size the workspace, launch on the current stream of the tensors' device."""
+    lib = load_library()
+    dev = _validate_tensors(tensors)
+    descs = describe(tensors)
+    n = len(tensors)
+    with torch.cuda.device(dev):
+        ws_bytes = getattr(lib, f"pto_{op}_workspace")(descs, n, ctypes.byref(params))
+        ws = torch.empty(ws_bytes, dtype=torch.uint8, device=dev) if ws_bytes else None
+        stream = torch.cuda.current_stream(dev).cuda_stream
+        rc = getattr(lib, f"pto_{op}_launch")(descs, n, ctypes.byref(params), ws.data_ptr() if ws is not None else None,
+                                              ws_bytes, stream)
+    if rc != 0:
+        msg = lib.pto_last_error().decode()
+        raise _STATUS_EXC.get(rc, RuntimeError)(msg)
+
+
+def operator(n_tensors, scalar_names):
+    """Call convention of a jit-compiled reference operator: the first ``n_tensors`` positional
+    arguments are tensors (outputs included, caller-allocated), the rest are non-tensor arguments,
+    positional or by keyword; returns None; every failure surfaces as FeError
+    (python/pypto/frontend/parser/entry.py:296-322,518-583)."""
+
+    def deco(fn):
+        @functools.wraps(fn)
+        def wrapper(*args, **kwargs):
+            try:
+                if len(args) < n_tensors:
+                    raise RuntimeError(f"{fn.__name__} takes {n_tensors} tensors, got {len(args)} positional arguments")
+                tensors = list(args[:n_tensors])
+                rest = list(args[n_tensors:])
+                if len(rest) > len(scalar_names):
+                    raise RuntimeError(f"{fn.__name__} takes {len(scalar_names)} non-tensor arguments, got {len(rest)}")
+                scalars = dict(zip(scalar_names, rest))
+                for k, v in kwargs.items():
+                    if k not in scalar_names:
+                        raise TypeError(f"{fn.__name__} got an unexpected keyword argument '{k}'")
+                    scalars[k] = v
+                missing = [k for k in scalar_names if k not in scalars]
+                if missing:
+                    raise TypeError(f"{fn.__name__} missing non-tensor arguments: {', '.join(missing)}")
+                fn(*tensors, **scalars)
+            except PyptoError:
+                raise
+            except Exception as e:  # noqa: BLE001 - everything is re-raised under the boundary's error type
+                err = FeError(type(e)(f"Failed to call JIT function '{fn.__name__}'.\n{e}"))
+                raise err.with_traceback(e.__traceback__) from None
+            return None
+
+        return wrapper
+
+    return deco

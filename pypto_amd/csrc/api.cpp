@@ -1,0 +1,319 @@
+// C ABI of libpypto_amd (declared in include/pypto_amd.h): operand validation and kernel dispatch.
+//
+// Validation mirrors what the reference's binding layer checks before a launch
+// (python/pypto/frontend/parser/entry.py:351-365,664-747 and
+//  python/src/bindings/torch_tensor_converter.cpp:157-214): tensor count, dtypes, ranks, static dims.
+#include "pypto_amd.h"
+
+#include <cstdarg>
+#include <cstdio>
+#include <string>
+
+#include "kernels.h"
+
+namespace {
+
+thread_local std::string g_last_error;
+
+int fail(int code, const char* fmt, ...)
+{
+    char buf[512];
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(buf, sizeof(buf), fmt, ap);
+    va_end(ap);
+    g_last_error = buf;
+    return code;
+}
+
+const char* dtype_name(int dt)
+{
+    switch (dt) {
+        case PTO_DT_INT8: return "int8";
+        case PTO_DT_INT32: return "int32";
+        case PTO_DT_FP16: return "fp16";
+        case PTO_DT_FP32: return "fp32";
+        case PTO_DT_BF16: return "bf16";
+        default: return "unsupported";
+    }
+}
+
+int check_tensor(const char* op, const PtoTensorDesc& t, const char* name, int dtype, int rank, bool allow_empty = false)
+{
+    if (t.dataType != dtype)
+        return fail(PTO_ERR_DTYPE, "%s: %s must be %s, got %s", op, name, dtype_name(dtype), dtype_name(t.dataType));
+    if (t.rank != rank) return fail(PTO_ERR_SHAPE, "%s: %s must have rank %d, got %d", op, name, rank, t.rank);
+    int64_t numel = 1;
+    for (int i = 0; i < rank; ++i) {
+        if (t.shape[i] < 0) return fail(PTO_ERR_SHAPE, "%s: %s has a negative dimension", op, name);
+        numel *= t.shape[i];
+    }
+    if (numel > 0 && t.addr == nullptr) return fail(PTO_ERR_NULL, "%s: %s has a null address", op, name);
+    (void)allow_empty;
+    return PTO_OK;
+}
+
+struct SfaPlan {
+    pto::SfaArgs args;
+    uint64_t ws_bytes;
+};
+
+// Common checks of both attention entry points once the cache streams are resolved.
+int plan_sfa(const char* op, const PtoTensorDesc& qn, const PtoTensorDesc& qr, const PtoTensorDesc& tk,
+             const PtoTensorDesc& bt, const PtoTensorDesc& act, const PtoTensorDesc& out, int64_t out_rows,
+             const PtoSfaParams* p, SfaPlan* plan)
+{
+    if (p == nullptr) return fail(PTO_ERR_PARAM, "%s: params is null", op);
+    if (p->nq <= 0) return fail(PTO_ERR_PARAM, "%s: nq must be positive, got %d", op, p->nq);
+    if (p->n_kv != 1) return fail(PTO_ERR_PARAM, "%s: n_kv must be 1 (MLA shares one compressed KV head), got %d", op, p->n_kv);
+    if (p->topk <= 0 || p->topk > 2048) return fail(PTO_ERR_PARAM, "%s: topk must be in [1, 2048], got %d", op, p->topk);
+    if (p->block_size <= 0) return fail(PTO_ERR_PARAM, "%s: block_size must be positive, got %d", op, p->block_size);
+    if (p->kv_splits < 0 || p->kv_splits > 64) return fail(PTO_ERR_PARAM, "%s: kv_splits must be in [0, 64]", op);
+    if (!(p->softmax_scale == p->softmax_scale)) return fail(PTO_ERR_PARAM, "%s: softmax_scale is NaN", op);
+    if (qn.shape[1] != 512) return fail(PTO_ERR_SHAPE, "%s: query_nope last dim must be 512, got %lld", op, (long long)qn.shape[1]);
+    if (qr.shape[1] != 64) return fail(PTO_ERR_SHAPE, "%s: query_rope last dim must be 64, got %lld", op, (long long)qr.shape[1]);
+    if (qr.shape[0] != qn.shape[0]) return fail(PTO_ERR_SHAPE, "%s: query_nope and query_rope row counts differ", op);
+    if (qn.shape[0] % p->nq != 0) return fail(PTO_ERR_SHAPE, "%s: query rows (%lld) not a multiple of nq (%d)", op, (long long)qn.shape[0], p->nq);
+    const int64_t t = qn.shape[0] / p->nq;
+    const int64_t b = act.shape[0];
+    if (b == 0 ? t != 0 : t % b != 0)
+        return fail(PTO_ERR_SHAPE, "%s: query tokens (%lld) not a multiple of the batch (%lld)", op, (long long)t, (long long)b);
+    if (tk.shape[0] != t) return fail(PTO_ERR_SHAPE, "%s: topk_indices has %lld rows, expected %lld", op, (long long)tk.shape[0], (long long)t);
+    if (tk.shape[1] < (int64_t)p->n_kv * p->topk)
+        return fail(PTO_ERR_SHAPE, "%s: topk_indices has %lld columns, expected n_kv*topk = %d", op, (long long)tk.shape[1], p->n_kv * p->topk);
+    if (bt.shape[0] != b) return fail(PTO_ERR_SHAPE, "%s: block_table has %lld rows, expected %lld", op, (long long)bt.shape[0], (long long)b);
+    if (bt.shape[1] != p->max_blocknum_perbatch)
+        return fail(PTO_ERR_SHAPE, "%s: block_table has %lld columns, max_blocknum_perbatch is %d", op, (long long)bt.shape[1], p->max_blocknum_perbatch);
+    if (out_rows != qn.shape[0]) return fail(PTO_ERR_SHAPE, "%s: attention_out holds %lld head rows, expected %lld", op, (long long)out_rows, (long long)qn.shape[0]);
+    if (t > 0x7fffffff / 2048 || qn.shape[0] > 0x7fffffff) return fail(PTO_ERR_SHAPE, "%s: too many query tokens", op);
+
+    pto::SfaArgs& a = plan->args;
+    a.q_nope = qn.addr;
+    a.q_rope = qr.addr;
+    a.topk_idx = static_cast<const int32_t*>(tk.addr);
+    a.block_table = static_cast<const int32_t*>(bt.addr);
+    a.act_seq = static_cast<const int32_t*>(act.addr);
+    a.out = out.addr;
+    a.b = (int32_t)b;
+    a.s1 = b ? (int32_t)(t / b) : 0;
+    a.nq = p->nq;
+    a.topk = p->topk;
+    a.topk_stride = (int32_t)tk.shape[1];
+    a.block_size = p->block_size;
+    a.bt_stride = (int32_t)bt.shape[1];
+    a.softmax_scale = p->softmax_scale;
+    a.nsplit = p->kv_splits > 0 ? p->kv_splits : pto::sfa_pick_splits((int)t, p->nq, p->topk);
+    a.part_o = nullptr;
+    a.part_ml = nullptr;
+    plan->ws_bytes = pto::sfa_workspace_bytes((int)t, p->nq, a.nsplit);
+    return PTO_OK;
+}
+
+int bind_workspace(const char* op, SfaPlan* plan, void* ws, uint64_t ws_bytes)
+{
+    if (plan->ws_bytes == 0) return PTO_OK;
+    if (ws == nullptr || ws_bytes < plan->ws_bytes)
+        return fail(PTO_ERR_WORKSPACE, "%s: workspace of %llu bytes required, got %llu", op,
+                    (unsigned long long)plan->ws_bytes, (unsigned long long)(ws ? ws_bytes : 0));
+    pto::SfaArgs& a = plan->args;
+    const uint64_t rows = (uint64_t)a.b * a.s1 * a.nsplit * a.nq;
+    a.part_o = static_cast<float*>(ws);
+    a.part_ml = a.part_o + rows * 512;
+    return PTO_OK;
+}
+
+int plan_sfa_quant(const PtoTensorDesc* ts, uint32_t n, const PtoSfaParams* p, SfaPlan* plan)
+{
+    const char* op = "sparse_flash_attention_quant";
+    if (ts == nullptr || n != 9) return fail(PTO_ERR_ARG_COUNT, "%s: expected 9 tensors, got %u", op, n);
+    int rc;
+    if ((rc = check_tensor(op, ts[0], "query_nope", PTO_DT_BF16, 2))) return rc;
+    if ((rc = check_tensor(op, ts[1], "query_rope", PTO_DT_BF16, 2))) return rc;
+    const bool quant = ts[2].dataType == PTO_DT_INT8;
+    if (!quant && ts[2].dataType != PTO_DT_BF16)
+        return fail(PTO_ERR_DTYPE, "%s: key_nope_2d must be int8 or bf16, got %s", op, dtype_name(ts[2].dataType));
+    if ((rc = check_tensor(op, ts[2], "key_nope_2d", ts[2].dataType, 2))) return rc;
+    if ((rc = check_tensor(op, ts[3], "key_rope_2d", PTO_DT_BF16, 2))) return rc;
+    if ((rc = check_tensor(op, ts[4], "k_nope_scales", PTO_DT_FP32, 2))) return rc;
+    if ((rc = check_tensor(op, ts[5], "topk_indices", PTO_DT_INT32, 2))) return rc;
+    if ((rc = check_tensor(op, ts[6], "block_table", PTO_DT_INT32, 2))) return rc;
+    if ((rc = check_tensor(op, ts[7], "kv_act_seqs", PTO_DT_INT32, 1))) return rc;
+    if ((rc = check_tensor(op, ts[8], "attention_out", PTO_DT_BF16, 4))) return rc;
+    const int64_t n_rows = ts[2].shape[0];
+    if (ts[2].shape[1] != 512) return fail(PTO_ERR_SHAPE, "%s: key_nope_2d last dim must be 512", op);
+    if (ts[3].shape[0] != n_rows || ts[3].shape[1] != 64) return fail(PTO_ERR_SHAPE, "%s: key_rope_2d must be [%lld, 64]", op, (long long)n_rows);
+    if (quant && (ts[4].shape[0] != n_rows || ts[4].shape[1] != 4)) return fail(PTO_ERR_SHAPE, "%s: k_nope_scales must be [%lld, 4]", op, (long long)n_rows);
+    if (ts[8].shape[3] != 512) return fail(PTO_ERR_SHAPE, "%s: attention_out last dim must be 512", op);
+    if (n_rows > 0x7fffffff) return fail(PTO_ERR_SHAPE, "%s: cache has too many rows", op);
+    if (p && ts[8].shape[2] != p->nq) return fail(PTO_ERR_SHAPE, "%s: attention_out dim 2 must equal nq", op);
+    const int64_t out_rows = ts[8].shape[0] * ts[8].shape[1] * ts[8].shape[2];
+    if ((rc = plan_sfa(op, ts[0], ts[1], ts[5], ts[6], ts[7], ts[8], out_rows, p, plan))) return rc;
+    if (ts[8].shape[0] != plan->args.b) return fail(PTO_ERR_SHAPE, "%s: attention_out dim 0 must equal the batch", op);
+    pto::SfaArgs& a = plan->args;
+    a.quant = quant;
+    a.kn = static_cast<const uint8_t*>(ts[2].addr);
+    a.kr = static_cast<const uint8_t*>(ts[3].addr);
+    a.ks = static_cast<const uint8_t*>(ts[4].addr);
+    a.kn_stride = quant ? 512 : 1024;
+    a.kr_stride = 128;
+    a.ks_stride = 16;
+    a.n_rows = n_rows;
+    return PTO_OK;
+}
+
+int plan_sfa_antiquant(const PtoTensorDesc* ts, uint32_t n, const PtoSfaParams* p, SfaPlan* plan)
+{
+    const char* op = "sparse_attention_antiquant";
+    if (ts == nullptr || n != 7) return fail(PTO_ERR_ARG_COUNT, "%s: expected 7 tensors, got %u", op, n);
+    int rc;
+    if ((rc = check_tensor(op, ts[0], "query_nope", PTO_DT_BF16, 2))) return rc;
+    if ((rc = check_tensor(op, ts[1], "query_rope", PTO_DT_BF16, 2))) return rc;
+    if ((rc = check_tensor(op, ts[2], "nope_cache", PTO_DT_INT8, 2))) return rc;
+    if ((rc = check_tensor(op, ts[3], "topk_indices", PTO_DT_INT32, 2))) return rc;
+    if ((rc = check_tensor(op, ts[4], "block_table", PTO_DT_INT32, 2))) return rc;
+    if ((rc = check_tensor(op, ts[5], "kv_act_seqs", PTO_DT_INT32, 1))) return rc;
+    if ((rc = check_tensor(op, ts[6], "attention_out", PTO_DT_BF16, 2))) return rc;
+    if (ts[2].shape[1] != 656) return fail(PTO_ERR_SHAPE, "%s: nope_cache rows must be 656 bytes, got %lld", op, (long long)ts[2].shape[1]);
+    if (ts[6].shape[1] != 512) return fail(PTO_ERR_SHAPE, "%s: attention_out last dim must be 512", op);
+    if (ts[2].shape[0] > 0x7fffffff) return fail(PTO_ERR_SHAPE, "%s: cache has too many rows", op);
+    if ((rc = plan_sfa(op, ts[0], ts[1], ts[3], ts[4], ts[5], ts[6], ts[6].shape[0], p, plan))) return rc;
+    pto::SfaArgs& a = plan->args;
+    a.quant = true;
+    a.kn = static_cast<const uint8_t*>(ts[2].addr);
+    a.kr = a.kn + 512;
+    a.ks = a.kn + 640;
+    a.kn_stride = a.kr_stride = a.ks_stride = 656;
+    a.n_rows = ts[2].shape[0];
+    return PTO_OK;
+}
+
+int launch_sfa(const char* op, SfaPlan* plan, void* ws, uint64_t ws_bytes, void* stream)
+{
+    int rc = bind_workspace(op, plan, ws, ws_bytes);
+    if (rc) return rc;
+    hipError_t e = pto::sfa_launch(plan->args, static_cast<hipStream_t>(stream));
+    if (e != hipSuccess) return fail(PTO_ERR_HIP, "%s: HIP launch failed: %s", op, hipGetErrorString(e));
+    return PTO_OK;
+}
+
+struct IndexerPlan {
+    pto::IndexerArgs args;
+    uint64_t ws_bytes;
+};
+
+int plan_indexer(const PtoTensorDesc* ts, uint32_t n, const PtoIndexerParams* p, IndexerPlan* plan)
+{
+    const char* op = "lightning_indexer_decode";
+    if (ts == nullptr || n != 8) return fail(PTO_ERR_ARG_COUNT, "%s: expected 8 tensors, got %u", op, n);
+    if (p == nullptr) return fail(PTO_ERR_PARAM, "%s: params is null", op);
+    int rc;
+    if ((rc = check_tensor(op, ts[0], "idx_query", PTO_DT_INT8, 3))) return rc;
+    if ((rc = check_tensor(op, ts[1], "idx_query_scale", PTO_DT_FP16, 2))) return rc;
+    if ((rc = check_tensor(op, ts[2], "idx_key_cache", PTO_DT_INT8, 4))) return rc;
+    if ((rc = check_tensor(op, ts[3], "idx_key_scale", PTO_DT_FP16, 3))) return rc;
+    if ((rc = check_tensor(op, ts[4], "idx_weight", PTO_DT_FP16, 2))) return rc;
+    if ((rc = check_tensor(op, ts[5], "act_seq_key", PTO_DT_INT32, 1))) return rc;
+    if ((rc = check_tensor(op, ts[6], "block_table", PTO_DT_INT32, 2))) return rc;
+    if ((rc = check_tensor(op, ts[7], "topk_res", PTO_DT_INT32, 3))) return rc;
+    if (p->selected_count <= 0 || p->selected_count > 2048)
+        return fail(PTO_ERR_PARAM, "%s: selected_count must be in [1, 2048], got %d", op, p->selected_count);
+    const int64_t t = ts[0].shape[0], nh = ts[0].shape[1], d = ts[0].shape[2];
+    const int64_t blocks = ts[2].shape[0], bs = ts[2].shape[1];
+    const int64_t b = ts[5].shape[0];
+    if (nh != 64 || d != 128) return fail(PTO_ERR_SHAPE, "%s: idx_query must be [t, 64, 128], got [%lld, %lld, %lld]", op, (long long)t, (long long)nh, (long long)d);
+    if (ts[2].shape[2] != 1 || ts[2].shape[3] != d) return fail(PTO_ERR_SHAPE, "%s: idx_key_cache must be [blocks, block_size, 1, 128]", op);
+    if (bs <= 0) return fail(PTO_ERR_SHAPE, "%s: block_size must be positive", op);
+    if (ts[3].shape[0] != blocks || ts[3].shape[1] != bs || ts[3].shape[2] != 1) return fail(PTO_ERR_SHAPE, "%s: idx_key_scale must be [blocks, block_size, 1]", op);
+    if (ts[1].shape[0] != t || ts[1].shape[1] != nh) return fail(PTO_ERR_SHAPE, "%s: idx_query_scale must be [t, 64]", op);
+    if (ts[4].shape[0] != t || ts[4].shape[1] != nh) return fail(PTO_ERR_SHAPE, "%s: idx_weight must be [t, 64]", op);
+    if (b == 0 ? t != 0 : t % b != 0) return fail(PTO_ERR_SHAPE, "%s: query tokens (%lld) not a multiple of the batch (%lld)", op, (long long)t, (long long)b);
+    if (b && t / b > 4) return fail(PTO_ERR_SHAPE, "%s: at most 4 query tokens per sequence, got %lld", op, (long long)(t / b));
+    if (ts[6].shape[0] != b) return fail(PTO_ERR_SHAPE, "%s: block_table has %lld rows, expected %lld", op, (long long)ts[6].shape[0], (long long)b);
+    if (ts[7].shape[0] != t || ts[7].shape[1] != 1 || ts[7].shape[2] != p->selected_count)
+        return fail(PTO_ERR_SHAPE, "%s: topk_res must be [t, 1, selected_count]", op);
+    const int64_t max_ctx = ts[6].shape[1] * bs;
+    if (max_ctx > (1 << 20) || blocks * bs > 0x7fffffff || t > 65535) return fail(PTO_ERR_SHAPE, "%s: problem too large", op);
+    pto::IndexerArgs& a = plan->args;
+    a.q = static_cast<const int8_t*>(ts[0].addr);
+    a.q_scale = static_cast<const uint16_t*>(ts[1].addr);
+    a.k_cache = static_cast<const int8_t*>(ts[2].addr);
+    a.k_scale = static_cast<const uint16_t*>(ts[3].addr);
+    a.weights = static_cast<const uint16_t*>(ts[4].addr);
+    a.act_seq = static_cast<const int32_t*>(ts[5].addr);
+    a.block_table = static_cast<const int32_t*>(ts[6].addr);
+    a.topk_res = static_cast<int32_t*>(ts[7].addr);
+    a.scores = nullptr;
+    a.n_blocks = blocks;
+    a.b = (int32_t)b;
+    a.s1 = b ? (int32_t)(t / b) : 0;
+    a.nh = (int32_t)nh;
+    a.block_size = (int32_t)bs;
+    a.bt_stride = (int32_t)ts[6].shape[1];
+    a.k = p->selected_count;
+    a.score_stride = (int32_t)max_ctx;
+    plan->ws_bytes = pto::indexer_workspace_bytes((int)t, (int)max_ctx);
+    return PTO_OK;
+}
+
+} // namespace
+
+extern "C" {
+
+uint64_t pto_sfa_quant_workspace(const PtoTensorDesc* tensors, uint32_t n_tensors, const PtoSfaParams* params)
+{
+    SfaPlan plan;
+    return plan_sfa_quant(tensors, n_tensors, params, &plan) == PTO_OK ? plan.ws_bytes : 0;
+}
+
+int pto_sfa_quant_launch(const PtoTensorDesc* tensors, uint32_t n_tensors, const PtoSfaParams* params, void* workspace,
+                         uint64_t workspace_bytes, void* hip_stream)
+{
+    SfaPlan plan;
+    int rc = plan_sfa_quant(tensors, n_tensors, params, &plan);
+    if (rc) return rc;
+    return launch_sfa("sparse_flash_attention_quant", &plan, workspace, workspace_bytes, hip_stream);
+}
+
+uint64_t pto_sfa_antiquant_workspace(const PtoTensorDesc* tensors, uint32_t n_tensors, const PtoSfaParams* params)
+{
+    SfaPlan plan;
+    return plan_sfa_antiquant(tensors, n_tensors, params, &plan) == PTO_OK ? plan.ws_bytes : 0;
+}
+
+int pto_sfa_antiquant_launch(const PtoTensorDesc* tensors, uint32_t n_tensors, const PtoSfaParams* params,
+                             void* workspace, uint64_t workspace_bytes, void* hip_stream)
+{
+    SfaPlan plan;
+    int rc = plan_sfa_antiquant(tensors, n_tensors, params, &plan);
+    if (rc) return rc;
+    return launch_sfa("sparse_attention_antiquant", &plan, workspace, workspace_bytes, hip_stream);
+}
+
+uint64_t pto_lightning_indexer_workspace(const PtoTensorDesc* tensors, uint32_t n_tensors,
+                                         const PtoIndexerParams* params)
+{
+    IndexerPlan plan;
+    return plan_indexer(tensors, n_tensors, params, &plan) == PTO_OK ? plan.ws_bytes : 0;
+}
+
+int pto_lightning_indexer_launch(const PtoTensorDesc* tensors, uint32_t n_tensors, const PtoIndexerParams* params,
+                                 void* workspace, uint64_t workspace_bytes, void* hip_stream)
+{
+    const char* op = "lightning_indexer_decode";
+    IndexerPlan plan;
+    int rc = plan_indexer(tensors, n_tensors, params, &plan);
+    if (rc) return rc;
+    if (plan.ws_bytes > 0 && (workspace == nullptr || workspace_bytes < plan.ws_bytes))
+        return fail(PTO_ERR_WORKSPACE, "%s: workspace of %llu bytes required, got %llu", op,
+                    (unsigned long long)plan.ws_bytes, (unsigned long long)(workspace ? workspace_bytes : 0));
+    plan.args.scores = static_cast<float*>(workspace);
+    hipError_t e = pto::indexer_launch(plan.args, static_cast<hipStream_t>(hip_stream));
+    if (e != hipSuccess) return fail(PTO_ERR_HIP, "%s: HIP launch failed: %s", op, hipGetErrorString(e));
+    return PTO_OK;
+}
+
+const char* pto_last_error(void) { return g_last_error.c_str(); }
+
+int pto_abi_version(void) { return 1; }
+
+} // extern "C"

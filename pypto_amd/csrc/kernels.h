@@ -1,0 +1,52 @@
+// Host-side launch interface between the C ABI (api.cpp) and the gfx950 kernels.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace pto {
+
+// ---------------------------------------------------------------- sparse flash attention
+struct SfaArgs {
+    const void* q_nope; // [t*nq, 512] bf16
+    const void* q_rope; // [t*nq, 64]  bf16
+    // Cache streams, each addressed as base + row * stride (bytes): three tensors, or three
+    // offsets into one packed 656-byte row.
+    const uint8_t* kn; // 512 x int8 (or 512 x bf16 when !quant)
+    const uint8_t* kr; // 64 x bf16
+    const uint8_t* ks; // 4 x fp32
+    int64_t kn_stride, kr_stride, ks_stride;
+    int64_t n_rows;
+    const int32_t* topk_idx;    // [t, topk_stride]
+    const int32_t* block_table; // [b, bt_stride]
+    const int32_t* act_seq;     // [b]
+    void* out;                  // [t*nq, 512] bf16
+    float* part_o;              // [t, nsplit, nq, 512] fp32 (nsplit > 1)
+    float* part_ml;             // [t, nsplit, nq, 2]  fp32 (running max in log2 units, sum)
+    int32_t b, s1, nq, topk, topk_stride, block_size, bt_stride, nsplit;
+    float softmax_scale;
+    bool quant;
+};
+
+int sfa_pick_splits(int t, int nq, int topk);
+uint64_t sfa_workspace_bytes(int t, int nq, int nsplit);
+hipError_t sfa_launch(const SfaArgs& a, hipStream_t stream);
+
+// ---------------------------------------------------------------- lightning indexer
+struct IndexerArgs {
+    const int8_t* q;             // [t, nh, 128]
+    const uint16_t* q_scale;     // [t, nh] fp16
+    const int8_t* k_cache;       // [blocks*bs, 128]
+    const uint16_t* k_scale;     // [blocks*bs] fp16
+    const uint16_t* weights;     // [t, nh] fp16
+    const int32_t* act_seq;      // [b]
+    const int32_t* block_table;  // [b, bt_stride]
+    int32_t* topk_res;           // [t, k]
+    float* scores;               // workspace [t, score_stride]
+    int64_t n_blocks;
+    int32_t b, s1, nh, block_size, bt_stride, k, score_stride;
+};
+
+uint64_t indexer_workspace_bytes(int t, int max_ctx);
+hipError_t indexer_launch(const IndexerArgs& a, hipStream_t stream);
+
+} // namespace pto
