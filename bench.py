@@ -1,0 +1,216 @@
+#!/usr/bin/env python3
+"""Benchmark of the DeepSeek-V3.2 quantized decode-attention hot path on one MI355X.
+
+One step = one decode step of the path for a batch: lightning indexer (int8 index scores + top-2048) over
+the paged index-K cache, then sparse flash attention over the selected rows of the int8 paged MLA cache,
+chained (the indexer's output is the attention's top-k list).  Workload: batch 32, one query token per
+sequence, every context 65536 tokens, 64 index heads x 128, 128 absorbed heads, 512 nope + 64 rope, pages
+of 128 tokens.  Inputs are synthetic, resident in HBM before the timed region; three copies of the caches
+are rotated so that no step finds its cache lines in the 256 MB last-level cache from the step before.
+
+Prints ONE JSON line: whole-job decode tokens/s, the roofline object of the dominant kernel (duration from
+HIP events recorded on the launch stream inside the library, second pass over the same steps), and the
+CPU oracle timed on the host cores on a bounded sample of the same workload.
+"""
+import argparse
+import ctypes
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0
+MFMA_BF16_PEAK_TFLOPS = 2500.0
+
+
+def parse():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--batch", type=int, default=32)
+    ap.add_argument("--ctx", type=int, default=65536)
+    ap.add_argument("--s1", type=int, default=1)
+    ap.add_argument("--cpu-seqs", type=int, default=8, help="sequences of the workload timed on the CPU oracle")
+    ap.add_argument("--no-cpu", action="store_true")
+    ap.add_argument("--packed", action="store_true", help="use the packed 656-byte-row attention entry point")
+    return ap.parse_args()
+
+
+def make_workload(torch, dev, b, ctx, s1, nbuf, seed=0):
+    g = torch.Generator(device=dev).manual_seed(seed)
+    bs = 128
+    pages_per_seq = (ctx + bs - 1) // bs
+    n_pages = b * pages_per_seq
+    n_rows = n_pages * bs
+    table = torch.randperm(n_pages, generator=g, device=dev).to(torch.int32).reshape(b, pages_per_seq).contiguous()
+    t = b * s1
+    sets = []
+    for _ in range(nbuf):
+        sets.append({
+            "idx_k": torch.randint(-127, 128, (n_pages, bs, 1, 128), generator=g, device=dev, dtype=torch.int8),
+            "idx_ks": (0.005 + 0.015 * torch.rand((n_pages, bs, 1), generator=g, device=dev)).to(torch.float16),
+            "kn": torch.randint(-127, 128, (n_rows, 512), generator=g, device=dev, dtype=torch.int8),
+            "kr": torch.randn((n_rows, 64), generator=g, device=dev).to(torch.bfloat16),
+            "ks": (0.005 + 0.015 * torch.rand((n_rows, 4), generator=g, device=dev)).float(),
+        })
+    w = {
+        "b": b, "s1": s1, "ctx": ctx, "bs": bs, "pages_per_seq": pages_per_seq, "table": table, "sets": sets,
+        "idx_q": torch.randint(-127, 128, (t, 64, 128), generator=g, device=dev, dtype=torch.int8),
+        "idx_qs": (0.005 + 0.015 * torch.rand((t, 64), generator=g, device=dev)).to(torch.float16),
+        "idx_w": (torch.randn((t, 64), generator=g, device=dev) / 8).to(torch.float16),
+        "q_nope": torch.randn((t * 128, 512), generator=g, device=dev).to(torch.bfloat16),
+        "q_rope": torch.randn((t * 128, 64), generator=g, device=dev).to(torch.bfloat16),
+        "act": torch.full((b,), ctx, dtype=torch.int32, device=dev),
+        "topk_res": torch.zeros((t, 1, 2048), dtype=torch.int32, device=dev),
+        "out": torch.zeros((b, s1, 128, 512), dtype=torch.bfloat16, device=dev),
+    }
+    return w
+
+
+def main():
+    args = parse()
+    if args.gpus != 1:
+        print(f"bench.py measures one GPU only (this build has no multi-GPU path); got --gpus {args.gpus}",
+              file=sys.stderr)
+        sys.exit(2)
+    import torch
+    from pypto_amd import _runtime
+    from pypto_amd.deepseek_v32_exp.lightning_indexer_quant_impl import (LightningIndexerConfigs,
+                                                                         lightning_indexer_decode)
+    from pypto_amd.deepseek_v32_exp.sparse_attention_antiquant_impl import sparse_attention_antiquant_d
+    from pypto_amd.deepseek_v32_exp.sparse_flash_attention_quant_impl import (SaTileShapeConfig,
+                                                                              sparse_flash_attention_quant_d)
+    if not torch.cuda.is_available():
+        print("bench.py needs a GPU", file=sys.stderr)
+        sys.exit(2)
+    lib = _runtime.load_library()
+    dev = torch.device("cuda:0")
+    b, ctx, s1 = args.batch, args.ctx, args.s1
+    scale = 192 ** -0.5
+    nbuf = 3
+    w = make_workload(torch, dev, b, ctx, s1, nbuf)
+    if args.packed:
+        for s in w["sets"]:
+            rows = torch.empty((s["kn"].shape[0], 656), dtype=torch.int8, device=dev)
+            rows[:, :512] = s["kn"]
+            rows[:, 512:640] = s["kr"].view(torch.int8)
+            rows[:, 640:] = s["ks"].view(torch.int8)
+            s["rows"] = rows
+    cfg, tile = LightningIndexerConfigs(), SaTileShapeConfig()
+    unroll = [128, 64, 32, 16, 8, 4, 1]
+
+    def step(i):
+        s = w["sets"][i % nbuf]
+        lightning_indexer_decode(w["idx_q"], w["idx_qs"], s["idx_k"], s["idx_ks"], w["idx_w"], w["act"], w["table"],
+                                 w["topk_res"], unroll, cfg, 2048)
+        tk = w["topk_res"].view(b * s1, 2048)
+        if args.packed:
+            sparse_attention_antiquant_d(w["q_nope"], w["q_rope"], s["rows"], tk, w["table"], w["act"],
+                                         w["out"].view(b * s1 * 128, 512), 128, 1, scale, 2048, 128,
+                                         w["pages_per_seq"], tile)
+        else:
+            sparse_flash_attention_quant_d(w["q_nope"], w["q_rope"], s["kn"], s["kr"], s["ks"], tk, w["table"],
+                                           w["act"], w["out"], 128, 1, scale, 2048, 128, w["pages_per_seq"], tile)
+
+    for i in range(args.warmup):
+        step(i)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for i in range(args.steps):
+        step(i)
+    torch.cuda.synchronize()
+    t1 = time.perf_counter()
+    ms_per_step = (t1 - t0) * 1e3 / args.steps
+    tokens_per_s = b * s1 / (ms_per_step * 1e-3)
+
+    # second pass over the same steps with an event pair around every kernel launch
+    lib.pto_kernel_timing_enable(1)
+    for i in range(args.steps):
+        step(i)
+    torch.cuda.synchronize()
+    lib.pto_kernel_timing_enable(0)
+    lib.pto_kernel_name.restype = ctypes.c_char_p
+    kernels = {}
+    for kid in range(4):
+        ms, n = ctypes.c_double(0), ctypes.c_uint64(0)
+        lib.pto_kernel_timing_read(kid, ctypes.byref(ms), ctypes.byref(n))
+        if n.value:
+            kernels[lib.pto_kernel_name(kid).decode()] = ms.value * 1e3 / n.value  # us per launch
+
+    t = b * s1
+    L = ctx
+    # algorithmic traffic / work per launch
+    score_bytes = b * (L * 128 + L * 2 + (L + 127) // 128 * 4) + t * (64 * 128 + 64 * 2 + 64 * 2)
+    topk_bytes = t * 2048 * 4
+    cur = min(L, 2048)
+    sfa_bytes = t * (cur * 656 + 128 * 576 * 2 + 128 * 512 * 2 + 2048 * 4)
+    sfa_flops = t * 278528 * cur
+    info = {
+        "indexer_score_kernel": {"bound": "hbm", "work": score_bytes, "peak": HBM_PEAK_GBS, "unit": "GB/s"},
+        "indexer_topk_kernel": {"bound": "hbm", "work": topk_bytes, "peak": HBM_PEAK_GBS, "unit": "GB/s"},
+        "sfa_decode_kernel": {"bound": "mfma", "work": sfa_flops, "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s"},
+        "sfa_combine_kernel": {"bound": "hbm", "work": t * 128 * 512 * 2, "peak": HBM_PEAK_GBS, "unit": "GB/s"},
+    }
+    per_kernel = []
+    for name, us in kernels.items():
+        k = info[name]
+        div = 1e3 if k["unit"] == "GB/s" else 1e6  # bytes/us -> GB/s is /1e3 ; flop/us -> TFLOP/s is /1e6
+        achieved = k["work"] / us / div
+        per_kernel.append({"kernel": name, "us": round(us, 2), "bound": k["bound"], "achieved": round(achieved, 2),
+                           "peak": k["peak"], "unit": k["unit"], "frac": round(achieved / k["peak"], 4)})
+    per_kernel.sort(key=lambda r: -r["us"])
+    dom = per_kernel[0]
+    roofline = {"kernel": dom["kernel"], "bound": dom["bound"], "achieved": dom["achieved"], "peak": dom["peak"],
+                "unit": dom["unit"], "frac": dom["frac"], "traffic": None, "us_per_launch": dom["us"]}
+    sfa_row = next((r for r in per_kernel if r["kernel"] == "sfa_decode_kernel"), None)
+    if sfa_row:
+        sfa_row["hbm_gbs"] = round(sfa_bytes / sfa_row["us"] / 1e3, 1)
+
+    cpu_baseline = None
+    if not args.no_cpu:
+        cpu_baseline = time_cpu_oracle(torch, w, min(args.cpu_seqs, b), scale)
+
+    print(json.dumps({
+        "metric": "decode tokens/sec + achieved HBM GB/s (% of peak), V3.2 SFA b=32 ctx=64K",
+        "value": round(tokens_per_s, 1), "unit": "tokens/s", "n_gpus": 1, "steps": args.steps,
+        "warmup": args.warmup, "ms_per_step": round(ms_per_step, 4), "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": "int8 index scores (int32 acc) + bf16 attention (fp32 acc)",
+        "data": "synthetic",
+        "config": {"workload": f"lightning indexer top-2048 + sparse flash attention decode, batch {b}, "
+                               f"s1 {s1}, ctx {ctx}, 64x128 int8 index heads, 128 heads x (512 nope + 64 rope), "
+                               f"int8 paged MLA cache, block 128, {'packed 656 B rows' if args.packed else 'three cache tensors'}"},
+        "roofline": roofline, "kernels": per_kernel, "cpu_baseline": cpu_baseline,
+    }))
+
+
+def time_cpu_oracle(torch, w, n_seq, scale):
+    """Oracle (vectorised torch restatement of the reference's CPU golden) timed on the first n_seq sequences
+    of the same inputs (cache copy 0)."""
+    from oracle import indexer as oi
+    from oracle import sfa as osfa
+    s1, ctx = w["s1"], w["ctx"]
+    s = w["sets"][0]
+    host = {k: v.cpu() for k, v in s.items() if k != "rows"}
+    table = w["table"][:n_seq].cpu()
+    act = [ctx] * n_seq
+    t = n_seq * s1
+    idx_q, idx_qs, idx_w = w["idx_q"][:t].cpu(), w["idx_qs"][:t].cpu(), w["idx_w"][:t].cpu()
+    q = torch.cat([w["q_nope"][:t * 128].cpu().reshape(n_seq, s1, 128, 512),
+                   w["q_rope"][:t * 128].cpu().reshape(n_seq, s1, 128, 64)], dim=-1)
+    t0 = time.perf_counter()
+    tk = oi.lightning_indexer(idx_q, idx_qs, host["idx_k"], host["idx_ks"], idx_w, act, table, s1, 2048)
+    out = osfa.attention_no_flash(q, host["kn"], host["kr"], host["ks"], tk.reshape(t, 2048), table, act, 128, scale,
+                                  2048)
+    dt = time.perf_counter() - t0
+    return {"value": round(t / dt, 2), "unit": "tokens/s", "cores": torch.get_num_threads(), "kind": "port",
+            "sample": f"first {n_seq} of the {w['b']} sequences of the same workload, one pass "
+                      f"({dt:.2f} s): oracle.indexer.lightning_indexer + oracle.sfa.attention_no_flash",
+            "host_cpus": os.cpu_count()}
+
+
+if __name__ == "__main__":
+    main()

@@ -123,6 +123,18 @@ int pto_lightning_indexer_launch(const PtoTensorDesc* tensors, uint32_t n_tensor
  * the reference's binding layer returns (python/src/bindings/runtime.cpp:270-335). */
 const char* pto_last_error(void);
 
+/*
+ * Measurement hooks (no counterpart in the reference, whose profiling is Ascend-specific:
+ * framework/src/machine/device/dynamic/aicore_prof.cpp).  While enabled, every kernel launch of the library
+ * is bracketed by a HIP event pair recorded on the launch stream; pto_kernel_timing_read waits for the
+ * events recorded so far for one kernel, returns their summed duration and count, and forgets them.
+ * Kernel ids: 0 indexer_score_kernel, 1 indexer_topk_kernel, 2 sfa_decode_kernel, 3 sfa_combine_kernel.
+ * Off by default; not for use under graph capture.
+ */
+int pto_kernel_timing_enable(int on);
+int pto_kernel_timing_read(int kernel_id, double* total_ms, uint64_t* launches);
+const char* pto_kernel_name(int kernel_id);
+
 /* ABI version of this header. */
 int pto_abi_version(void);
 

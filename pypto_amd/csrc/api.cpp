@@ -10,6 +10,7 @@
 #include <string>
 
 #include "kernels.h"
+#include "timing.h"
 
 namespace {
 
@@ -310,6 +311,28 @@ int pto_lightning_indexer_launch(const PtoTensorDesc* tensors, uint32_t n_tensor
     hipError_t e = pto::indexer_launch(plan.args, static_cast<hipStream_t>(hip_stream));
     if (e != hipSuccess) return fail(PTO_ERR_HIP, "%s: HIP launch failed: %s", op, hipGetErrorString(e));
     return PTO_OK;
+}
+
+int pto_kernel_timing_enable(int on)
+{
+    pto::timing_set(on != 0);
+    return PTO_OK;
+}
+
+int pto_kernel_timing_read(int kernel_id, double* total_ms, uint64_t* launches)
+{
+    if (kernel_id < 0 || kernel_id >= pto::KID_COUNT || total_ms == nullptr || launches == nullptr)
+        return fail(PTO_ERR_PARAM, "pto_kernel_timing_read: bad kernel id or null output");
+    hipError_t e = pto::timing_collect(kernel_id, total_ms, launches);
+    if (e != hipSuccess) return fail(PTO_ERR_HIP, "pto_kernel_timing_read: %s", hipGetErrorString(e));
+    return PTO_OK;
+}
+
+const char* pto_kernel_name(int kernel_id)
+{
+    static const char* names[] = {"indexer_score_kernel", "indexer_topk_kernel", "sfa_decode_kernel",
+                                  "sfa_combine_kernel"};
+    return kernel_id >= 0 && kernel_id < pto::KID_COUNT ? names[kernel_id] : "";
 }
 
 const char* pto_last_error(void) { return g_last_error.c_str(); }

@@ -20,6 +20,7 @@
 // of (key, ~index) words orders them.
 #include "common.h"
 #include "kernels.h"
+#include "timing.h"
 
 namespace pto {
 namespace {
@@ -254,15 +255,21 @@ hipError_t indexer_launch(const IndexerArgs& a, hipStream_t stream)
     if (t == 0) return hipSuccess;
     const int max_ctx = a.score_stride;
     const int chunks = (max_ctx + CHUNK - 1) / CHUNK;
-    if (a.s1 % 2 == 0) {
-        hipLaunchKernelGGL((indexer_score_kernel<2, 4>), dim3(chunks, a.b, a.s1 / 2), dim3(256), 0, stream, a, 0);
-    } else {
-        hipLaunchKernelGGL((indexer_score_kernel<1, 4>), dim3(chunks, a.b, a.s1), dim3(256), 0, stream, a, 0);
+    {
+        ScopedKernelTimer tm(KID_INDEXER_SCORE, stream);
+        if (a.s1 % 2 == 0) {
+            hipLaunchKernelGGL((indexer_score_kernel<2, 4>), dim3(chunks, a.b, a.s1 / 2), dim3(256), 0, stream, a, 0);
+        } else {
+            hipLaunchKernelGGL((indexer_score_kernel<1, 4>), dim3(chunks, a.b, a.s1), dim3(256), 0, stream, a, 0);
+        }
     }
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) return e;
-    hipLaunchKernelGGL(indexer_topk_kernel, dim3(t), dim3(1024), 0, stream, a.scores, a.score_stride, a.act_seq, a.s1,
-                       a.k, a.topk_res);
+    {
+        ScopedKernelTimer tm(KID_INDEXER_TOPK, stream);
+        hipLaunchKernelGGL(indexer_topk_kernel, dim3(t), dim3(1024), 0, stream, a.scores, a.score_stride, a.act_seq,
+                           a.s1, a.k, a.topk_res);
+    }
     return hipGetLastError();
 }
 

@@ -23,6 +23,7 @@
 // KV splits write un-normalised fp32 partial outputs plus (m, l); sfa_combine_kernel merges them.
 #include "common.h"
 #include "kernels.h"
+#include "timing.h"
 
 namespace pto {
 namespace {
@@ -367,10 +368,14 @@ hipError_t sfa_launch(const SfaArgs& a, hipStream_t stream)
     }
     const int hgroups = (a.nq + HEADS_PER_WG - 1) / HEADS_PER_WG;
     dim3 grid(a.nsplit, t, hgroups);
-    hipLaunchKernelGGL(kern, grid, dim3(256), SMEM_BYTES, stream, a);
+    {
+        ScopedKernelTimer tm(KID_SFA_DECODE, stream);
+        hipLaunchKernelGGL(kern, grid, dim3(256), SMEM_BYTES, stream, a);
+    }
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) return e;
     if (a.nsplit > 1) {
+        ScopedKernelTimer tm(KID_SFA_COMBINE, stream);
         hipLaunchKernelGGL(sfa_combine_kernel, dim3(t * a.nq), dim3(128), 0, stream, a.part_o, a.part_ml, a.out, a.nq,
                            a.nsplit);
         e = hipGetLastError();

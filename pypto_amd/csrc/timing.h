@@ -1,0 +1,25 @@
+// Optional per-kernel timing with HIP events recorded on the launch stream (off by default).
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace pto {
+
+enum KernelId { KID_INDEXER_SCORE = 0, KID_INDEXER_TOPK = 1, KID_SFA_DECODE = 2, KID_SFA_COMBINE = 3, KID_COUNT = 4 };
+
+bool timing_enabled();
+void timing_set(bool on);
+// Record an event pair around one kernel launch; no-ops while timing is off.
+void timing_begin(int kid, hipStream_t s);
+void timing_end(int kid, hipStream_t s);
+// Wait for the recorded events, return their summed duration and count, and forget them.
+hipError_t timing_collect(int kid, double* total_ms, uint64_t* launches);
+
+struct ScopedKernelTimer {
+    int kid;
+    hipStream_t s;
+    ScopedKernelTimer(int k, hipStream_t st) : kid(k), s(st) { timing_begin(kid, s); }
+    ~ScopedKernelTimer() { timing_end(kid, s); }
+};
+
+} // namespace pto
