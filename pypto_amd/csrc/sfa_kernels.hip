@@ -9,16 +9,19 @@
 //   P~ = exp(S - m) rounded to bf16 un-normalised, l summed in fp32 from the unrounded values
 //   O = (sum P~ V) / l, one rounding to bf16
 //
-// Work decomposition.  One workgroup (4 wavefronts) owns one (query token, KV split): it walks its share of
-// the token's top-k list in tiles of 32 selected cache rows.  Per tile all 256 lanes gather the rows
-// (8-byte loads, a wavefront covers the 512 int8 of one row per instruction), dequantise in registers and
-// store the tile to LDS twice: row-major for the S = K Q^T product and token-minor ("V^T") for the O^T = V^T P
-// product, so both MFMA A-operands are single 16-byte LDS reads.  Wavefront w owns query heads
-// [32w, 32w+32): its slice of Q stays in registers (B operand of v_mfma_f32_32x32x16_bf16), S^T comes out
-// with one head per lane (row statistics are in-lane reductions plus one cross-half exchange), and the
-// rounded P~ registers are directly the B operand of the PV product.  O^T (512 x 32 per wavefront) lives in
-// 256 accumulator registers.  The LDS tile is double buffered: tile i+1 is dequantised while tile i is in
-// the matrix cores.
+// Work decomposition.  One workgroup (4 wavefronts) owns one (query token, KV split, group of 64 heads): it
+// walks its share of the token's top-k list in tiles of 32 selected cache rows.  Per tile all 256 lanes
+// gather the rows (8-byte loads, a wavefront covers the 512 int8 of one row per instruction), dequantise in
+// registers and store the tile row-major to LDS (16-byte chunks XOR-swizzled with the row, no padding).
+// Wavefronts pair up on 32 heads: wave (hg, kh) holds the Q columns of the k-steps with parity kh (B operand
+// of v_mfma_f32_32x32x16_bf16, 72 registers), computes its half of S^T = K Q^T, swaps the fp32 partial with
+// its partner through LDS, and both run the same softmax (one head per lane: row statistics are in-lane
+// reductions plus one cross-half exchange).  The rounded P~ registers are directly the B operand of
+// O^T = V^T P~, of which wave kh accumulates the 32-column blocks of parity kh (128 accumulator registers).
+// The V^T operand is read from the same row-major tile with ds_read_b64_tr_b16 (LDS transpose read: a 16-lane
+// group fetches 4 rows x 16 columns and each lane receives 4 rows of one column).  The LDS tile is double
+// buffered: tile i+1 is dequantised while tile i is in the matrix cores.  64 heads per workgroup (not 128)
+// keeps Q + O at 200 of the 512 registers per lane, which leaves room to overlap loads, dequant and MFMA.
 //
 // KV splits write un-normalised fp32 partial outputs plus (m, l); sfa_combine_kernel merges them.
 #include "common.h"
@@ -31,97 +34,94 @@ namespace {
 constexpr int T = 32;                  // selected rows per tile
 constexpr int DN = 512;                // nope / value width
 constexpr int DR = 64;                 // rope width
-constexpr int KSTEPS = (DN + DR) / 16; // 36 MFMA k-steps for S
-constexpr int KROW = (DN + DR) * 2 + 16; // bytes per row of the row-major tile (16 B pad: conflict-free b128 reads)
-constexpr int KBUF = T * KROW;           // 37376
-constexpr int VBUF = DN * T * 2;         // 32768
-constexpr int STAGE = KBUF + VBUF;       // 70144
-constexpr int MAX_SPLIT_TOKENS = 2048;   // rows[] capacity
-constexpr int SMEM_BYTES = 2 * STAGE + MAX_SPLIT_TOKENS * 4;
-constexpr int HEADS_PER_WG = 128;
+constexpr int KSTEPS = (DN + DR) / 16; // 36 MFMA k-steps for S, 18 per wave of a pair
+constexpr int KROW = (DN + DR) * 2;    // 1152 bytes per tile row = 72 chunks of 16 bytes
+constexpr int STAGE = T * KROW;        // 36864
+constexpr int MAX_SPLIT_TOKENS = 2048; // capacity of rows[] / scales[]
+constexpr int ROWS_OFF = 2 * STAGE;
+constexpr int SCALES_OFF = ROWS_OFF + MAX_SPLIT_TOKENS * 4;
+constexpr int XBUF_OFF = SCALES_OFF + MAX_SPLIT_TOKENS * 16;
+constexpr int SMEM_BYTES = XBUF_OFF + 4 * 4096; // 131072
+constexpr int HEADS_PER_WG = 64;
+
+typedef short s16x4 __attribute__((ext_vector_type(4)));
+typedef short s16x8 __attribute__((ext_vector_type(8)));
+typedef __attribute__((address_space(3))) s16x4 lds_s16x4;
+
+// ds_read_b64_tr_b16: within each group of 16 lanes, lane i receives element i%4 of the 8-byte chunks
+// addressed by lanes i/4, 4 + i/4, 8 + i/4 and 12 + i/4 of the group.
+__device__ __forceinline__ s16x4 lds_read_tr(uint8_t* p) { return __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)p); }
+
+// chunk swizzle of tile row t: a bijection of t % 8, so that 8 consecutive rows (b128 column reads) and the
+// 4 consecutive rows of a transpose read both land on distinct banks
+__device__ __forceinline__ int swz(int t) { return ((t & 3) << 1) | ((t >> 2) & 1); }
 
 template <bool QUANT>
 struct RawTile;
 template <>
 struct RawTile<true> {
-    u32x2 nope[8]; // 8 tokens x 8 int8 (this lane's 8 columns)
-    float scale[8];
+    u32x2 nope[8]; // 8 rows x 8 int8 (this lane's 8 columns)
     u32x4 rope;
 };
 template <>
 struct RawTile<false> {
-    u32x4 nope[8]; // 8 tokens x 8 bf16
+    u32x4 nope[8]; // 8 rows x 8 bf16
     u32x4 rope;
 };
 
-// token-in-tile of element e (0..7) of 8-token chunk c (0..3): the k-slot order of the PV B operand
-__device__ __forceinline__ int chunk_token(int c, int e) { return 16 * (c >> 1) + 8 * (e >> 2) + 4 * (c & 1) + (e & 3); }
-
+// Lane (wave w, lane l) fetches columns [8l, 8l+8) of tile rows 8w .. 8w+7 and one 16-byte piece of a rope row.
 template <bool QUANT>
 __device__ __forceinline__ void load_raw(RawTile<QUANT>& r, const SfaArgs& a, const int* rows, int tile, int wave,
                                          int lane, int tid)
 {
 #pragma unroll
     for (int e = 0; e < 8; ++e) {
-        const int row = rows[tile * T + chunk_token(wave, e)];
+        const int row = rows[tile * T + 8 * wave + e];
+        const int64_t rr = row < 0 ? 0 : row;
         if constexpr (QUANT) {
-            u32x2 v = {0u, 0u};
-            float s = 0.f;
-            if (row >= 0) {
-                v = *reinterpret_cast<const u32x2*>(a.kn + (int64_t)row * a.kn_stride + lane * 8);
-                s = *reinterpret_cast<const float*>(a.ks + (int64_t)row * a.ks_stride + (lane >> 4) * 4);
-            }
+            u32x2 v = *reinterpret_cast<const u32x2*>(a.kn + rr * a.kn_stride + lane * 8);
+            if (row < 0) v = u32x2{0u, 0u};
             r.nope[e] = v;
-            r.scale[e] = s;
         } else {
-            u32x4 v = {0u, 0u, 0u, 0u};
-            if (row >= 0) v = *reinterpret_cast<const u32x4*>(a.kn + (int64_t)row * a.kn_stride + lane * 16);
+            u32x4 v = *reinterpret_cast<const u32x4*>(a.kn + rr * a.kn_stride + lane * 16);
+            if (row < 0) v = u32x4{0u, 0u, 0u, 0u};
             r.nope[e] = v;
         }
     }
     {
         const int row = rows[tile * T + (tid >> 3)];
-        u32x4 v = {0u, 0u, 0u, 0u};
-        if (row >= 0) v = *reinterpret_cast<const u32x4*>(a.kr + (int64_t)row * a.kr_stride + (tid & 7) * 16);
+        const int64_t rr = row < 0 ? 0 : row;
+        u32x4 v = *reinterpret_cast<const u32x4*>(a.kr + rr * a.kr_stride + (tid & 7) * 16);
+        if (row < 0) v = u32x4{0u, 0u, 0u, 0u};
         r.rope = v;
     }
 }
 
 __device__ __forceinline__ float i8_at(uint32_t w, int k) { return (float)(int8_t)(w >> (8 * k)); }
 
-// Dequantise this lane's 8 tokens x 8 columns and store them to both LDS layouts of a stage.
+// Dequantise this lane's 8 rows x 8 columns and store them (and the rope piece) into an LDS stage.
 template <bool QUANT>
-__device__ __forceinline__ void dequant_store(const RawTile<QUANT>& r, uint8_t* stage, int wave, int lane, int tid)
+__device__ __forceinline__ void dequant_store(const RawTile<QUANT>& r, uint8_t* stage, const float* scales, int tile,
+                                              int wave, int lane, int tid)
 {
-    uint32_t kb[8][4]; // [token e][column pair]
 #pragma unroll
     for (int e = 0; e < 8; ++e) {
-        if constexpr (QUANT) {
-            const float s = r.scale[e];
-            const uint32_t w0 = r.nope[e][0], w1 = r.nope[e][1];
-            kb[e][0] = pack_bf16x2(i8_at(w0, 0) * s, i8_at(w0, 1) * s);
-            kb[e][1] = pack_bf16x2(i8_at(w0, 2) * s, i8_at(w0, 3) * s);
-            kb[e][2] = pack_bf16x2(i8_at(w1, 0) * s, i8_at(w1, 1) * s);
-            kb[e][3] = pack_bf16x2(i8_at(w1, 2) * s, i8_at(w1, 3) * s);
-        } else {
-#pragma unroll
-            for (int p = 0; p < 4; ++p) kb[e][p] = r.nope[e][p];
-        }
-        u32x4 v = {kb[e][0], kb[e][1], kb[e][2], kb[e][3]};
-        *reinterpret_cast<u32x4*>(stage + chunk_token(wave, e) * KROW + lane * 16) = v;
-    }
-    // token-minor layout: block (column group of 8 = lane, chunk = wave) is 128 contiguous bytes holding
-    // 8 columns x 8 tokens; the 16-byte slot of column d is swizzled with the column group.
-    uint8_t* vt = stage + KBUF + (lane * 4 + wave) * 128;
-#pragma unroll
-    for (int d = 0; d < 8; ++d) {
-        const uint32_t sel = (d & 1) ? 0x07060302u : 0x05040100u;
+        const int t = 8 * wave + e;
         u32x4 v;
-#pragma unroll
-        for (int p = 0; p < 4; ++p) v[p] = __builtin_amdgcn_perm(kb[2 * p + 1][d >> 1], kb[2 * p][d >> 1], sel);
-        *reinterpret_cast<u32x4*>(vt + ((d ^ (lane & 7)) * 16)) = v;
+        if constexpr (QUANT) {
+            const float s = scales[(tile * T + t) * 4 + (lane >> 4)];
+            const uint32_t w0 = r.nope[e][0], w1 = r.nope[e][1];
+            v[0] = pack_bf16x2(i8_at(w0, 0) * s, i8_at(w0, 1) * s);
+            v[1] = pack_bf16x2(i8_at(w0, 2) * s, i8_at(w0, 3) * s);
+            v[2] = pack_bf16x2(i8_at(w1, 0) * s, i8_at(w1, 1) * s);
+            v[3] = pack_bf16x2(i8_at(w1, 2) * s, i8_at(w1, 3) * s);
+        } else {
+            v = r.nope[e];
+        }
+        *reinterpret_cast<u32x4*>(stage + t * KROW + ((lane ^ swz(t)) << 4)) = v;
     }
-    *reinterpret_cast<u32x4*>(stage + (tid >> 3) * KROW + DN * 2 + (tid & 7) * 16) = r.rope;
+    const int t = tid >> 3;
+    *reinterpret_cast<u32x4*>(stage + t * KROW + DN * 2 + (((tid & 7) ^ swz(t)) << 4)) = r.rope;
 }
 
 template <bool QUANT>
@@ -129,11 +129,13 @@ __global__ __attribute__((amdgpu_flat_work_group_size(256, 256), amdgpu_waves_pe
     SfaArgs a)
 {
     extern __shared__ __align__(16) uint8_t smem[];
-    int* rows = reinterpret_cast<int*>(smem + 2 * STAGE);
+    int* rows = reinterpret_cast<int*>(smem + ROWS_OFF);
+    float* scales = reinterpret_cast<float*>(smem + SCALES_OFF);
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int l32 = lane & 31, hl = lane >> 5;
-    const int sp = blockIdx.x, tq = blockIdx.y, hg = blockIdx.z;
+    const int hg = wave >> 1, kh = wave & 1; // head group of 32 within the workgroup; k-step / dim-block parity
+    const int sp = blockIdx.x, tq = blockIdx.y, hz = blockIdx.z;
     const int bi = tq / a.s1, si = tq - bi * a.s1;
 
     int cur = a.act_seq[bi] - a.s1 + 1 + si;
@@ -144,7 +146,7 @@ __global__ __attribute__((amdgpu_flat_work_group_size(256, 256), amdgpu_waves_pe
     const int ntiles = max(min(ntiles_all, tile0 + per) - tile0, 0);
     const int tok0 = tile0 * T;
 
-    // logical top-k entries of this split -> physical cache rows (or -1: absent)
+    // logical top-k entries of this split -> physical cache rows (or -1: absent), and their 4 dequant scales
     const int64_t max_logical = (int64_t)a.bt_stride * a.block_size;
     for (int i = tid; i < ntiles * T; i += 256) {
         const int g = tok0 + i;
@@ -158,62 +160,99 @@ __global__ __attribute__((amdgpu_flat_work_group_size(256, 256), amdgpu_waves_pe
             }
         }
         rows[i] = row;
-    }
-
-    // this lane's query head and its Q slice (B operand: head = column, 8 consecutive k per half-wave)
-    const int head = hg * HEADS_PER_WG + wave * 32 + l32;
-    const bool head_ok = head < a.nq;
-    const bool wave_active = hg * HEADS_PER_WG + wave * 32 < a.nq;
-    bf16x8 q[KSTEPS];
-    {
-        const int64_t qrow = (int64_t)tq * a.nq + (head_ok ? head : 0);
-        const __bf16* qn = reinterpret_cast<const __bf16*>(a.q_nope) + qrow * DN + hl * 8;
-        const __bf16* qr = reinterpret_cast<const __bf16*>(a.q_rope) + qrow * DR + hl * 8;
-        const bf16x8 zero = {0, 0, 0, 0, 0, 0, 0, 0};
-#pragma unroll
-        for (int ks = 0; ks < KSTEPS; ++ks) {
-            const __bf16* p = ks < DN / 16 ? qn + ks * 16 : qr + (ks - DN / 16) * 16;
-            q[ks] = head_ok ? *reinterpret_cast<const bf16x8*>(p) : zero;
+        if constexpr (QUANT) {
+            f32x4 sc = {0.f, 0.f, 0.f, 0.f};
+            if (row >= 0) sc = *reinterpret_cast<const f32x4*>(a.ks + (int64_t)row * a.ks_stride);
+            *reinterpret_cast<f32x4*>(scales + i * 4) = sc;
         }
     }
 
-    f32x16 o[16];
+    // this lane's query head and its Q slice: k-steps 2*i + kh, i = 0..17 (0..15 nope, 16..17 rope); B operand
+    // layout: head = column, 8 consecutive k per half-wave.  Lanes past the last head reuse head 0's rows,
+    // their results are never written.
+    const int head = hz * HEADS_PER_WG + hg * 32 + l32;
+    const bool head_ok = head < a.nq;
+    const bool wave_active = hz * HEADS_PER_WG + hg * 32 < a.nq;
+    bf16x8 q[KSTEPS / 2];
+    {
+        const int64_t qrow = (int64_t)tq * a.nq + (head_ok ? head : 0);
+        const __bf16* qn = reinterpret_cast<const __bf16*>(a.q_nope) + qrow * DN + kh * 16 + hl * 8;
+        const __bf16* qr = reinterpret_cast<const __bf16*>(a.q_rope) + qrow * DR + kh * 16 + hl * 8;
 #pragma unroll
-    for (int i = 0; i < 16; ++i)
+        for (int i = 0; i < DN / 32; ++i) q[i] = *reinterpret_cast<const bf16x8*>(qn + i * 32);
+#pragma unroll
+        for (int i = 0; i < DR / 32; ++i) q[DN / 32 + i] = *reinterpret_cast<const bf16x8*>(qr + i * 32);
+    }
+
+    f32x16 o[8]; // O^T blocks db = 2*i + kh: dims [32*db, 32*db + 32) x 32 heads
+#pragma unroll
+    for (int i = 0; i < 8; ++i)
 #pragma unroll
         for (int r = 0; r < 16; ++r) o[i][r] = 0.f;
     float m_run = -INFINITY; // running max of S * scale * log2(e)
     float l_run = 0.f;       // this lane's share of sum exp
     const float c_log2 = a.softmax_scale * 1.4426950408889634f;
 
-    __syncthreads(); // rows[] ready
+    // S operand (b128): row l32, chunk 2*ks + hl with ks = 2*i + kh -> chunk 4*i + 2*kh + hl; swizzled offsets
+    // for even and odd i
+    uint32_t s_off[2];
+    {
+        const int sw = swz(l32), c = 2 * kh + hl;
+        s_off[0] = l32 * KROW + ((c ^ sw) << 4);
+        s_off[1] = l32 * KROW + (((4 + c) ^ sw) << 4);
+    }
+    // V^T operand (transpose read): lane jj of 16-lane group G points at row 4*hl + jj/4 (+ 16*j + 8*h2),
+    // columns 32*db + 16*(G&1) + 4*(jj&3) with db = 2*i + kh -> chunk 8*i + 4*kh + 2*(G&1) + (jj&3)/2
+    uint32_t v_off;
+    {
+        const int jj = lane & 15, mh = (lane >> 4) & 1;
+        const int cl = 4 * kh + 2 * mh + ((jj & 3) >> 1);
+        const int sw = ((jj >> 2) << 1) | hl;
+        v_off = (4 * hl + (jj >> 2)) * KROW + (jj & 1) * 8 + ((cl ^ sw) << 4);
+    }
+    uint8_t* xmine = smem + XBUF_OFF + wave * 4096 + lane * 16;
+    uint8_t* xpeer = smem + XBUF_OFF + (wave ^ 1) * 4096 + lane * 16;
+
+    __syncthreads(); // rows[] / scales[] ready
 
     RawTile<QUANT> raw;
     if (ntiles > 0) {
         load_raw<QUANT>(raw, a, rows, 0, wave, lane, tid);
-        dequant_store(raw, smem, wave, lane, tid);
+        dequant_store<QUANT>(raw, smem, scales, 0, wave, lane, tid);
         if (ntiles > 1) load_raw<QUANT>(raw, a, rows, 1, wave, lane, tid);
     }
     __syncthreads();
 
     for (int it = 0; it < ntiles; ++it) {
         uint8_t* stage = smem + (it & 1) * STAGE;
+        const uint32_t valid = (uint32_t)__ballot(rows[it * T + l32] >= 0);
+        // half of S^T[token, head] = K[token, :] . Q[head, :] (k-steps of parity kh)
+        f32x16 s;
+#pragma unroll
+        for (int r = 0; r < 16; ++r) s[r] = 0.f;
+#pragma unroll
+        for (int i = 0; i < KSTEPS / 2; ++i) {
+            const bf16x8 kf = *reinterpret_cast<const bf16x8*>(stage + s_off[i & 1] + (i >> 1) * 128);
+            s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf, q[i], s, 0, 0, 0);
+        }
+#pragma unroll
+        for (int g = 0; g < 4; ++g)
+            *reinterpret_cast<f32x4*>(xmine + g * 1024) = f32x4{s[4 * g], s[4 * g + 1], s[4 * g + 2], s[4 * g + 3]};
+        // next tile: dequantise into the other stage, start the loads of the one after
         if (it + 1 < ntiles) {
-            dequant_store(raw, smem + ((it + 1) & 1) * STAGE, wave, lane, tid);
+            dequant_store<QUANT>(raw, smem + ((it + 1) & 1) * STAGE, scales, it + 1, wave, lane, tid);
             if (it + 2 < ntiles) load_raw<QUANT>(raw, a, rows, it + 2, wave, lane, tid);
         }
-        const uint32_t valid = (uint32_t)__ballot(rows[it * T + l32] >= 0);
+        __syncthreads(); // partial S of both waves of each pair is in LDS
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+            const f32x4 p = *reinterpret_cast<const f32x4*>(xpeer + g * 1024);
+            s[4 * g] += p[0];
+            s[4 * g + 1] += p[1];
+            s[4 * g + 2] += p[2];
+            s[4 * g + 3] += p[3];
+        }
         if (wave_active && valid != 0u) {
-            // S^T[token, head] = K[token, :] . Q[head, :]
-            f32x16 s;
-#pragma unroll
-            for (int r = 0; r < 16; ++r) s[r] = 0.f;
-            const uint8_t* ka = stage + l32 * KROW + hl * 16;
-#pragma unroll
-            for (int ks = 0; ks < KSTEPS; ++ks) {
-                const bf16x8 kf = *reinterpret_cast<const bf16x8*>(ka + ks * 32);
-                s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf, q[ks], s, 0, 0, 0);
-            }
             // register r holds token 8*(r/4) + 4*hl + r%4 for head l32
             float mx = -INFINITY;
 #pragma unroll
@@ -229,10 +268,10 @@ __global__ __attribute__((amdgpu_flat_work_group_size(256, 256), amdgpu_waves_pe
             mx = fmaxf(mx, __shfl_xor(mx, 32));
             const float m_new = fmaxf(m_run, mx);
             if (__any(m_new > m_run)) {
-                const float alpha = exp2f(m_run - m_new); // 0 on the first tile (m_run = -inf)
+                const float alpha = __builtin_amdgcn_exp2f(m_run - m_new); // 0 on the first tile (m_run = -inf)
                 l_run *= alpha;
 #pragma unroll
-                for (int i = 0; i < 16; ++i)
+                for (int i = 0; i < 8; ++i)
 #pragma unroll
                     for (int r = 0; r < 16; ++r) o[i][r] *= alpha;
                 m_run = m_new;
@@ -240,58 +279,66 @@ __global__ __attribute__((amdgpu_flat_work_group_size(256, 256), amdgpu_waves_pe
             uint32_t pb[8];
 #pragma unroll
             for (int r = 0; r < 16; r += 2) {
-                const float p0 = exp2f(s[r] - m_run), p1 = exp2f(s[r + 1] - m_run);
+                const float p0 = __builtin_amdgcn_exp2f(s[r] - m_run), p1 = __builtin_amdgcn_exp2f(s[r + 1] - m_run);
                 l_run += p0 + p1;
                 pb[r >> 1] = pack_bf16x2(p0, p1);
             }
-            // O^T[dim, head] += V^T[dim, token] . P~[token, head]
-            const uint8_t* vt = stage + KBUF;
+            // O^T[dim, head] += V^T[dim, token] . P~[token, head]; k-slot s of half hl in block j is token
+            // 16*j + 8*(s/4) + 4*hl + s%4, the order in which the S^T registers hold the tokens
 #pragma unroll
             for (int j = 0; j < 2; ++j) {
                 u32x4 pw = {pb[4 * j], pb[4 * j + 1], pb[4 * j + 2], pb[4 * j + 3]};
                 const bf16x8 pf = __builtin_bit_cast(bf16x8, pw);
 #pragma unroll
-                for (int db = 0; db < 16; ++db) {
-                    const int dg = 4 * db + (l32 >> 3), d = l32 & 7;
-                    const bf16x8 vf =
-                        *reinterpret_cast<const bf16x8*>(vt + (dg * 4 + 2 * j + hl) * 128 + ((d ^ (dg & 7)) * 16));
-                    o[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf, pf, o[db], 0, 0, 0);
+                for (int i = 0; i < 8; ++i) {
+                    uint8_t* vp = stage + v_off + (16 * j) * KROW + i * 128;
+                    const s16x4 lo = lds_read_tr(vp);
+                    const s16x4 hi = lds_read_tr(vp + 8 * KROW);
+                    const s16x8 both = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+                    o[i] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, both), pf, o[i], 0, 0, 0);
                 }
             }
         }
-        __syncthreads();
+        __syncthreads(); // tile consumed: its stage and the exchange buffer may be overwritten
     }
 
     if (!wave_active) return;
     const float l_tot = l_run + __shfl_xor(l_run, 32);
     if (!head_ok) return;
-    // register r of block db holds dim 32*db + 8*(r/4) + 4*hl + r%4 of head l32
+    // register r of o[i] holds dim 32*(2*i + kh) + 8*(r/4) + 4*hl + r%4 of head l32
     if (a.nsplit == 1) {
         const float inv = l_tot > 0.f ? 1.f / l_tot : 0.f;
         uint8_t* dst = reinterpret_cast<uint8_t*>(a.out) + ((int64_t)tq * a.nq + head) * DN * 2;
 #pragma unroll
-        for (int db = 0; db < 16; ++db)
+        for (int i = 0; i < 8; ++i)
 #pragma unroll
             for (int g = 0; g < 4; ++g) {
-                u32x2 v = {pack_bf16x2(o[db][4 * g] * inv, o[db][4 * g + 1] * inv),
-                           pack_bf16x2(o[db][4 * g + 2] * inv, o[db][4 * g + 3] * inv)};
-                *reinterpret_cast<u32x2*>(dst + (32 * db + 8 * g + 4 * hl) * 2) = v;
+                u32x2 v = {pack_bf16x2(o[i][4 * g] * inv, o[i][4 * g + 1] * inv),
+                           pack_bf16x2(o[i][4 * g + 2] * inv, o[i][4 * g + 3] * inv)};
+                *reinterpret_cast<u32x2*>(dst + (32 * (2 * i + kh) + 8 * g + 4 * hl) * 2) = v;
             }
     } else {
         const int64_t prow = ((int64_t)tq * a.nsplit + sp) * a.nq + head;
         float* dst = a.part_o + prow * DN;
 #pragma unroll
-        for (int db = 0; db < 16; ++db)
+        for (int i = 0; i < 8; ++i)
 #pragma unroll
             for (int g = 0; g < 4; ++g) {
-                f32x4 v = {o[db][4 * g], o[db][4 * g + 1], o[db][4 * g + 2], o[db][4 * g + 3]};
-                *reinterpret_cast<f32x4*>(dst + 32 * db + 8 * g + 4 * hl) = v;
+                f32x4 v = {o[i][4 * g], o[i][4 * g + 1], o[i][4 * g + 2], o[i][4 * g + 3]};
+                *reinterpret_cast<f32x4*>(dst + 32 * (2 * i + kh) + 8 * g + 4 * hl) = v;
             }
-        if (hl == 0) {
+        if (hl == 0 && kh == 0) {
             a.part_ml[prow * 2] = m_run;
             a.part_ml[prow * 2 + 1] = l_tot;
         }
     }
+}
+
+// attention_out <- 0 (cache without rows: every selected entry is absent)
+__global__ void sfa_zero_kernel(uint32_t* out, int64_t n_words)
+{
+    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n_words) out[i] = 0u;
 }
 
 // out[row, :] = sum_s 2^(m_s - M) O_s[row, :] / sum_s 2^(m_s - M) l_s ; one block of 128 lanes per output row
@@ -358,6 +405,12 @@ hipError_t sfa_launch(const SfaArgs& a, hipStream_t stream)
 {
     const int t = a.b * a.s1;
     if (t == 0) return hipSuccess;
+    if (a.n_rows == 0) {
+        const int64_t words = (int64_t)t * a.nq * DN / 2;
+        hipLaunchKernelGGL(sfa_zero_kernel, dim3((unsigned)((words + 255) / 256)), dim3(256), 0, stream,
+                           static_cast<uint32_t*>(a.out), words);
+        return hipGetLastError();
+    }
     static bool attr_done[2] = {false, false};
     auto kern = a.quant ? sfa_decode_kernel<true> : sfa_decode_kernel<false>;
     if (!attr_done[a.quant]) {
