@@ -16,6 +16,9 @@ SOURCES = ["api.cpp", "timing.cpp", "sfa_kernels.hip", "indexer_kernels.hip"]
 HIPCC_FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-shared", "-x", "hip",
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+    # MFMA accumulators in architectural VGPRs: the attention kernel rescales its accumulators with VALU
+    # multiplies, and with AGPR accumulators the compiler keeps a VGPR copy of all of them alive
+    "-mllvm", "-amdgpu-mfma-vgpr-form=1",
     "-Wno-unused-command-line-argument", "-Wno-unknown-attributes",
 ]
 

@@ -62,39 +62,40 @@ template <>
 struct RawTile<true> {
     u32x2 nope[8]; // 8 rows x 8 int8 (this lane's 8 columns)
     u32x4 rope;
+    uint32_t absent;
 };
 template <>
 struct RawTile<false> {
     u32x4 nope[8]; // 8 rows x 8 bf16
     u32x4 rope;
+    uint32_t absent;
 };
 
 // Lane (wave w, lane l) fetches columns [8l, 8l+8) of tile rows 8w .. 8w+7 and one 16-byte piece of a rope row.
+// Absent rows (-1) read row 0 instead; `absent` keeps one bit per load and the data is zeroed when it is
+// consumed (dequant_store), so that no load has to be waited for here.
 template <bool QUANT>
 __device__ __forceinline__ void load_raw(RawTile<QUANT>& r, const SfaArgs& a, const int* rows, int tile, int wave,
                                          int lane, int tid)
 {
+    uint32_t absent = 0;
 #pragma unroll
     for (int e = 0; e < 8; ++e) {
         const int row = rows[tile * T + 8 * wave + e];
         const int64_t rr = row < 0 ? 0 : row;
-        if constexpr (QUANT) {
-            u32x2 v = *reinterpret_cast<const u32x2*>(a.kn + rr * a.kn_stride + lane * 8);
-            if (row < 0) v = u32x2{0u, 0u};
-            r.nope[e] = v;
-        } else {
-            u32x4 v = *reinterpret_cast<const u32x4*>(a.kn + rr * a.kn_stride + lane * 16);
-            if (row < 0) v = u32x4{0u, 0u, 0u, 0u};
-            r.nope[e] = v;
-        }
+        absent |= (row < 0 ? 1u : 0u) << e;
+        if constexpr (QUANT)
+            r.nope[e] = *reinterpret_cast<const u32x2*>(a.kn + rr * a.kn_stride + lane * 8);
+        else
+            r.nope[e] = *reinterpret_cast<const u32x4*>(a.kn + rr * a.kn_stride + lane * 16);
     }
     {
         const int row = rows[tile * T + (tid >> 3)];
         const int64_t rr = row < 0 ? 0 : row;
-        u32x4 v = *reinterpret_cast<const u32x4*>(a.kr + rr * a.kr_stride + (tid & 7) * 16);
-        if (row < 0) v = u32x4{0u, 0u, 0u, 0u};
-        r.rope = v;
+        absent |= (row < 0 ? 1u : 0u) << 8;
+        r.rope = *reinterpret_cast<const u32x4*>(a.kr + rr * a.kr_stride + (tid & 7) * 16);
     }
+    r.absent = absent;
 }
 
 __device__ __forceinline__ float i8_at(uint32_t w, int k) { return (float)(int8_t)(w >> (8 * k)); }
@@ -109,19 +110,20 @@ __device__ __forceinline__ void dequant_store(const RawTile<QUANT>& r, uint8_t* 
         const int t = 8 * wave + e;
         u32x4 v;
         if constexpr (QUANT) {
-            const float s = scales[(tile * T + t) * 4 + (lane >> 4)];
+            const float s = scales[(tile * T + t) * 4 + (lane >> 4)]; // 0 for an absent row
             const uint32_t w0 = r.nope[e][0], w1 = r.nope[e][1];
             v[0] = pack_bf16x2(i8_at(w0, 0) * s, i8_at(w0, 1) * s);
             v[1] = pack_bf16x2(i8_at(w0, 2) * s, i8_at(w0, 3) * s);
             v[2] = pack_bf16x2(i8_at(w1, 0) * s, i8_at(w1, 1) * s);
             v[3] = pack_bf16x2(i8_at(w1, 2) * s, i8_at(w1, 3) * s);
         } else {
-            v = r.nope[e];
+            v = ((r.absent >> e) & 1u) ? u32x4{0u, 0u, 0u, 0u} : r.nope[e];
         }
         *reinterpret_cast<u32x4*>(stage + t * KROW + ((lane ^ swz(t)) << 4)) = v;
     }
     const int t = tid >> 3;
-    *reinterpret_cast<u32x4*>(stage + t * KROW + DN * 2 + (((tid & 7) ^ swz(t)) << 4)) = r.rope;
+    const u32x4 rp = ((r.absent >> 8) & 1u) ? u32x4{0u, 0u, 0u, 0u} : r.rope;
+    *reinterpret_cast<u32x4*>(stage + t * KROW + DN * 2 + (((tid & 7) ^ swz(t)) << 4)) = rp;
 }
 
 template <bool QUANT>
@@ -215,15 +217,20 @@ __global__ __attribute__((amdgpu_flat_work_group_size(256, 256), amdgpu_waves_pe
 
     __syncthreads(); // rows[] / scales[] ready
 
-    RawTile<QUANT> raw;
+    // Gathered rows travel global -> registers -> LDS.  Two register tiles alternate so that the loads of a
+    // tile are issued two tiles before it is dequantised (one tile of flight time is not enough to cover the
+    // latency of scattered 656-byte rows with a single workgroup per CU).
+    RawTile<QUANT> raw0, raw1;
     if (ntiles > 0) {
-        load_raw<QUANT>(raw, a, rows, 0, wave, lane, tid);
-        dequant_store<QUANT>(raw, smem, scales, 0, wave, lane, tid);
-        if (ntiles > 1) load_raw<QUANT>(raw, a, rows, 1, wave, lane, tid);
+        load_raw<QUANT>(raw0, a, rows, 0, wave, lane, tid);
+        if (ntiles > 1) load_raw<QUANT>(raw1, a, rows, 1, wave, lane, tid);
+        dequant_store<QUANT>(raw0, smem, scales, 0, wave, lane, tid);
+        if (ntiles > 2) load_raw<QUANT>(raw0, a, rows, 2, wave, lane, tid);
     }
     __syncthreads();
 
-    for (int it = 0; it < ntiles; ++it) {
+    // one tile: `next` holds the raw rows of tile it + 1 and is refilled with tile it + 3
+    auto tile_step = [&](int it, RawTile<QUANT>& next) {
         uint8_t* stage = smem + (it & 1) * STAGE;
         const uint32_t valid = (uint32_t)__ballot(rows[it * T + l32] >= 0);
         // half of S^T[token, head] = K[token, :] . Q[head, :] (k-steps of parity kh)
@@ -240,8 +247,8 @@ __global__ __attribute__((amdgpu_flat_work_group_size(256, 256), amdgpu_waves_pe
             *reinterpret_cast<f32x4*>(xmine + g * 1024) = f32x4{s[4 * g], s[4 * g + 1], s[4 * g + 2], s[4 * g + 3]};
         // next tile: dequantise into the other stage, start the loads of the one after
         if (it + 1 < ntiles) {
-            dequant_store<QUANT>(raw, smem + ((it + 1) & 1) * STAGE, scales, it + 1, wave, lane, tid);
-            if (it + 2 < ntiles) load_raw<QUANT>(raw, a, rows, it + 2, wave, lane, tid);
+            dequant_store<QUANT>(next, smem + ((it + 1) & 1) * STAGE, scales, it + 1, wave, lane, tid);
+            if (it + 3 < ntiles) load_raw<QUANT>(next, a, rows, it + 3, wave, lane, tid);
         }
         __syncthreads(); // partial S of both waves of each pair is in LDS
 #pragma unroll
@@ -300,6 +307,10 @@ __global__ __attribute__((amdgpu_flat_work_group_size(256, 256), amdgpu_waves_pe
             }
         }
         __syncthreads(); // tile consumed: its stage and the exchange buffer may be overwritten
+    };
+    for (int it = 0; it < ntiles; it += 2) {
+        tile_step(it, raw1);
+        if (it + 1 < ntiles) tile_step(it + 1, raw0);
     }
 
     if (!wave_active) return;
