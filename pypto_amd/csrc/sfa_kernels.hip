@@ -111,23 +111,29 @@ __device__ __forceinline__ void dequant_store(const RawTile<QUANT>& r, uint8_t* 
         u32x4 v;
         if constexpr (QUANT) {
             const float s = scales[(tile * T + t) * 4 + (lane >> 4)]; // 0 for an absent row
-            const uint32_t w0 = r.nope[e][0], w1 = r.nope[e][1];
+            uint32_t w0 = r.nope[e][0], w1 = r.nope[e][1];
+            // keep the unpacking here: hoisted to the load, it would wait for the load right after issuing it
+            asm volatile("" : "+v"(w0), "+v"(w1));
             v[0] = pack_bf16x2(i8_at(w0, 0) * s, i8_at(w0, 1) * s);
             v[1] = pack_bf16x2(i8_at(w0, 2) * s, i8_at(w0, 3) * s);
             v[2] = pack_bf16x2(i8_at(w1, 0) * s, i8_at(w1, 1) * s);
             v[3] = pack_bf16x2(i8_at(w1, 2) * s, i8_at(w1, 3) * s);
         } else {
-            v = ((r.absent >> e) & 1u) ? u32x4{0u, 0u, 0u, 0u} : r.nope[e];
+            u32x4 w = r.nope[e];
+            asm volatile("" : "+v"(w)); // as above: consume the load here, not where it was issued
+            v = ((r.absent >> e) & 1u) ? u32x4{0u, 0u, 0u, 0u} : w;
         }
         *reinterpret_cast<u32x4*>(stage + t * KROW + ((lane ^ swz(t)) << 4)) = v;
     }
     const int t = tid >> 3;
-    const u32x4 rp = ((r.absent >> 8) & 1u) ? u32x4{0u, 0u, 0u, 0u} : r.rope;
+    u32x4 rp = r.rope;
+    asm volatile("" : "+v"(rp));
+    rp = ((r.absent >> 8) & 1u) ? u32x4{0u, 0u, 0u, 0u} : rp;
     *reinterpret_cast<u32x4*>(stage + t * KROW + DN * 2 + (((tid & 7) ^ swz(t)) << 4)) = rp;
 }
 
 template <bool QUANT>
-__global__ __attribute__((amdgpu_flat_work_group_size(256, 256), amdgpu_waves_per_eu(1, 1))) void sfa_decode_kernel(
+__global__ __attribute__((amdgpu_flat_work_group_size(512, 512), amdgpu_waves_per_eu(2, 2))) void sfa_decode_kernel(
     SfaArgs a)
 {
     extern __shared__ __align__(16) uint8_t smem[];
@@ -135,8 +141,6 @@ __global__ __attribute__((amdgpu_flat_work_group_size(256, 256), amdgpu_waves_pe
     float* scales = reinterpret_cast<float*>(smem + SCALES_OFF);
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const int l32 = lane & 31, hl = lane >> 5;
-    const int hg = wave >> 1, kh = wave & 1; // head group of 32 within the workgroup; k-step / dim-block parity
     const int sp = blockIdx.x, tq = blockIdx.y, hz = blockIdx.z;
     const int bi = tq / a.s1, si = tq - bi * a.s1;
 
@@ -145,15 +149,17 @@ __global__ __attribute__((amdgpu_flat_work_group_size(256, 256), amdgpu_waves_pe
     const int ntiles_all = (cur + T - 1) / T;
     const int per = (ntiles_all + a.nsplit - 1) / a.nsplit;
     const int tile0 = sp * per;
-    const int ntiles = max(min(ntiles_all, tile0 + per) - tile0, 0);
+    const int ntiles_real = max(min(ntiles_all, tile0 + per) - tile0, 0);
+    // an even number of tiles keeps the producer loop free of conditional loads (the odd one out is fully masked)
+    const int ntiles = (ntiles_real + 1) & ~1;
     const int tok0 = tile0 * T;
 
     // logical top-k entries of this split -> physical cache rows (or -1: absent), and their 4 dequant scales
     const int64_t max_logical = (int64_t)a.bt_stride * a.block_size;
-    for (int i = tid; i < ntiles * T; i += 256) {
+    for (int i = tid; i < ntiles * T; i += 512) {
         const int g = tok0 + i;
         int row = -1;
-        if (g < cur) {
+        if (g < cur && i < ntiles_real * T) { // the padding tile holds no token
             const int idx = a.topk_idx[(int64_t)tq * a.topk_stride + g];
             if (idx >= 0 && idx < max_logical) {
                 const int page = a.block_table[(int64_t)bi * a.bt_stride + idx / a.block_size];
@@ -168,6 +174,43 @@ __global__ __attribute__((amdgpu_flat_work_group_size(256, 256), amdgpu_waves_pe
             *reinterpret_cast<f32x4*>(scales + i * 4) = sc;
         }
     }
+    __syncthreads(); // rows[] / scales[] ready
+
+    // Both roles run the same barrier sequence: one before the first tile, then two per tile
+    // (partial S exchanged; tile consumed and next tile stored).
+    if (wave >= 4) {
+        // ---------------------------------------------------------------- producer wavefronts
+        // Gathered rows travel global -> registers -> LDS.  Two register tiles alternate so that the loads of
+        // a tile are issued two tiles before it is dequantised.
+        const int pw = wave - 4, ptid = tid - 256;
+        const int last = ntiles - 1;
+        RawTile<QUANT> raw0, raw1;
+        if (ntiles > 0) {
+            load_raw<QUANT>(raw0, a, rows, 0, pw, lane, ptid);
+            load_raw<QUANT>(raw1, a, rows, 1, pw, lane, ptid);
+            dequant_store<QUANT>(raw0, smem, scales, 0, pw, lane, ptid);
+            load_raw<QUANT>(raw0, a, rows, min(2, last), pw, lane, ptid);
+        }
+        __syncthreads();
+        // Every step stores one tile and issues the loads of another, unconditionally (past the end the last
+        // tile is loaded again and stored into a stage nobody reads): with a fixed number of loads in flight
+        // on every path the wait for a tile leaves the younger tile's loads outstanding.
+        auto produce = [&](int it, RawTile<QUANT>& next) {
+            dequant_store<QUANT>(next, smem + ((it + 1) & 1) * STAGE, scales, min(it + 1, last), pw, lane, ptid);
+            load_raw<QUANT>(next, a, rows, min(it + 3, last), pw, lane, ptid);
+            __syncthreads();
+            __syncthreads();
+        };
+        for (int it = 0; it < ntiles; it += 2) {
+            produce(it, raw1);
+            produce(it + 1, raw0);
+        }
+        return;
+    }
+
+    // -------------------------------------------------------------------- consumer wavefronts
+    const int l32 = lane & 31, hl = lane >> 5;
+    const int hg = wave >> 1, kh = wave & 1; // head group of 32 within the workgroup; k-step / dim-block parity
 
     // this lane's query head and its Q slice: k-steps 2*i + kh, i = 0..17 (0..15 nope, 16..17 rope); B operand
     // layout: head = column, 8 consecutive k per half-wave.  Lanes past the last head reuse head 0's rows,
@@ -215,22 +258,9 @@ __global__ __attribute__((amdgpu_flat_work_group_size(256, 256), amdgpu_waves_pe
     uint8_t* xmine = smem + XBUF_OFF + wave * 4096 + lane * 16;
     uint8_t* xpeer = smem + XBUF_OFF + (wave ^ 1) * 4096 + lane * 16;
 
-    __syncthreads(); // rows[] / scales[] ready
+    __syncthreads(); // tile 0 stored
 
-    // Gathered rows travel global -> registers -> LDS.  Two register tiles alternate so that the loads of a
-    // tile are issued two tiles before it is dequantised (one tile of flight time is not enough to cover the
-    // latency of scattered 656-byte rows with a single workgroup per CU).
-    RawTile<QUANT> raw0, raw1;
-    if (ntiles > 0) {
-        load_raw<QUANT>(raw0, a, rows, 0, wave, lane, tid);
-        if (ntiles > 1) load_raw<QUANT>(raw1, a, rows, 1, wave, lane, tid);
-        dequant_store<QUANT>(raw0, smem, scales, 0, wave, lane, tid);
-        if (ntiles > 2) load_raw<QUANT>(raw0, a, rows, 2, wave, lane, tid);
-    }
-    __syncthreads();
-
-    // one tile: `next` holds the raw rows of tile it + 1 and is refilled with tile it + 3
-    auto tile_step = [&](int it, RawTile<QUANT>& next) {
+    for (int it = 0; it < ntiles; ++it) {
         uint8_t* stage = smem + (it & 1) * STAGE;
         const uint32_t valid = (uint32_t)__ballot(rows[it * T + l32] >= 0);
         // half of S^T[token, head] = K[token, :] . Q[head, :] (k-steps of parity kh)
@@ -245,11 +275,6 @@ __global__ __attribute__((amdgpu_flat_work_group_size(256, 256), amdgpu_waves_pe
 #pragma unroll
         for (int g = 0; g < 4; ++g)
             *reinterpret_cast<f32x4*>(xmine + g * 1024) = f32x4{s[4 * g], s[4 * g + 1], s[4 * g + 2], s[4 * g + 3]};
-        // next tile: dequantise into the other stage, start the loads of the one after
-        if (it + 1 < ntiles) {
-            dequant_store<QUANT>(next, smem + ((it + 1) & 1) * STAGE, scales, it + 1, wave, lane, tid);
-            if (it + 3 < ntiles) load_raw<QUANT>(next, a, rows, it + 3, wave, lane, tid);
-        }
         __syncthreads(); // partial S of both waves of each pair is in LDS
 #pragma unroll
         for (int g = 0; g < 4; ++g) {
@@ -307,10 +332,6 @@ __global__ __attribute__((amdgpu_flat_work_group_size(256, 256), amdgpu_waves_pe
             }
         }
         __syncthreads(); // tile consumed: its stage and the exchange buffer may be overwritten
-    };
-    for (int it = 0; it < ntiles; it += 2) {
-        tile_step(it, raw1);
-        if (it + 1 < ntiles) tile_step(it + 1, raw0);
     }
 
     if (!wave_active) return;
@@ -434,7 +455,7 @@ hipError_t sfa_launch(const SfaArgs& a, hipStream_t stream)
     dim3 grid(a.nsplit, t, hgroups);
     {
         ScopedKernelTimer tm(KID_SFA_DECODE, stream);
-        hipLaunchKernelGGL(kern, grid, dim3(256), SMEM_BYTES, stream, a);
+        hipLaunchKernelGGL(kern, grid, dim3(512), SMEM_BYTES, stream, a);
     }
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) return e;
