@@ -128,7 +128,8 @@ const char* pto_last_error(void);
  * framework/src/machine/device/dynamic/aicore_prof.cpp).  While enabled, every kernel launch of the library
  * is bracketed by a HIP event pair recorded on the launch stream; pto_kernel_timing_read waits for the
  * events recorded so far for one kernel, returns their summed duration and count, and forgets them.
- * Kernel ids: 0 indexer_score_kernel, 1 indexer_topk_kernel, 2 sfa_decode_kernel, 3 sfa_combine_kernel.
+ * Kernel ids: 0 indexer_score_kernel, 1 indexer_topk_kernel, 2 sfa_decode_kernel, 3 sfa_combine_kernel,
+ * 4 indexer_select_kernel.
  * Off by default; not for use under graph capture.
  */
 int pto_kernel_timing_enable(int on);

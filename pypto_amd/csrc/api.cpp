@@ -251,8 +251,8 @@ int plan_indexer(const PtoTensorDesc* ts, uint32_t n, const PtoIndexerParams* p,
     a.block_size = (int32_t)bs;
     a.bt_stride = (int32_t)ts[6].shape[1];
     a.k = p->selected_count;
-    a.score_stride = (int32_t)max_ctx;
-    plan->ws_bytes = pto::indexer_workspace_bytes((int)t, (int)max_ctx);
+    a.score_stride = (int32_t)((max_ctx + 3) & ~(int64_t)3); // rows of the score matrix stay 16-byte aligned
+    plan->ws_bytes = pto::indexer_workspace_bytes((int)t, a.score_stride);
     return PTO_OK;
 }
 
@@ -307,7 +307,7 @@ int pto_lightning_indexer_launch(const PtoTensorDesc* tensors, uint32_t n_tensor
     if (plan.ws_bytes > 0 && (workspace == nullptr || workspace_bytes < plan.ws_bytes))
         return fail(PTO_ERR_WORKSPACE, "%s: workspace of %llu bytes required, got %llu", op,
                     (unsigned long long)plan.ws_bytes, (unsigned long long)(workspace ? workspace_bytes : 0));
-    plan.args.scores = static_cast<float*>(workspace);
+    pto::indexer_bind_workspace(plan.args, workspace);
     hipError_t e = pto::indexer_launch(plan.args, static_cast<hipStream_t>(hip_stream));
     if (e != hipSuccess) return fail(PTO_ERR_HIP, "%s: HIP launch failed: %s", op, hipGetErrorString(e));
     return PTO_OK;
@@ -331,7 +331,7 @@ int pto_kernel_timing_read(int kernel_id, double* total_ms, uint64_t* launches)
 const char* pto_kernel_name(int kernel_id)
 {
     static const char* names[] = {"indexer_score_kernel", "indexer_topk_kernel", "sfa_decode_kernel",
-                                  "sfa_combine_kernel"};
+                                  "sfa_combine_kernel", "indexer_select_kernel"};
     return kernel_id >= 0 && kernel_id < pto::KID_COUNT ? names[kernel_id] : "";
 }
 

@@ -11,13 +11,21 @@
 //
 // indexer_score_kernel: v_mfma_i32_16x16x64_i8 with the query heads as rows (A, resident in registers)
 // and 16 cached keys as columns (B, loaded from the paged cache straight in operand layout: lane l reads
-// 16 bytes of key l%16).  The result has one key per lane, so the relu / fp16 rounding / weighted head sum
-// is an in-lane chain over 16 accumulators and two cross-lane adds.  Scores go to a dense fp32 row per
-// query token.
+// 16 bytes of key l%16).  The result has one key per lane and 16 heads per lane; relu, the 2^-11 scaling and
+// the fp16 rounding are 4 VALU operations per (head, key), and the weighted head sum is a second MFMA
+// (v_mfma_f32_16x16x32_f16: row 0 of A holds w_scale, B is the fp16 tile just produced; every product of two
+// fp16 values is exact in fp32, so this is the golden's fp32 sum up to the order of additions).  Scores go to
+// a dense fp32 row per query token, and the top 11 bits of their order-preserving keys into a 2048-bin
+// histogram per query token (LDS per workgroup, flushed with global atomics).
 //
-// indexer_topk_kernel: one workgroup per query token.  Three radix-select passes (11+11+10 bits of an
-// order-preserving key) find the k-th largest key, a compaction pass collects the winners, a bitonic sort
-// of (key, ~index) words orders them.
+// indexer_select_kernel: every workgroup scans the histogram for the bin B that holds the k-th largest key,
+// then files its 4096 scores: bins above B are winners, bin B goes to a tie list (both lists in the
+// workspace, appended with one global atomic per workgroup).
+//
+// indexer_topk_kernel: one workgroup per query token takes the winners, picks the missing krem entries out of
+// the tie list by radix-selecting on the 64-bit words (key << 32 | ~index) (so equal keys resolve to the
+// smaller index), and bitonic-sorts the k words.  A tie list that overflowed its capacity (e.g. all scores
+// equal) falls back to radix-selecting over the whole score row.
 #include "common.h"
 #include "kernels.h"
 #include "timing.h"
@@ -28,13 +36,22 @@ namespace {
 constexpr int D = 128;          // index head dim
 constexpr int CHUNK = 512;      // keys per workgroup of the score kernel
 constexpr int MAX_K = 2048;     // top-k capacity
+constexpr int NBINS = 2048;     // histogram over the top 11 key bits
+constexpr int SEL_CHUNK = 4096; // scores per workgroup of the select kernel
+constexpr int TIE_CAP = 8192;   // capacity of the per-row tie list
 
 __device__ __forceinline__ float f16_bits_to_f32(uint16_t h) { return (float)__builtin_bit_cast(_Float16, h); }
+__device__ __forceinline__ uint32_t score_key(float f) { return f32_to_ordered(f + 0.0f); } // -0 -> +0
+__device__ __forceinline__ uint64_t make_cand(uint32_t key, int idx)
+{
+    return ((uint64_t)key << 32) | (uint32_t)(0xffffffffu - (uint32_t)idx);
+}
 
 // S1 query tokens of one sequence share every key fragment.
-template <int S1, int NHB>
-__global__ __launch_bounds__(256) void indexer_score_kernel(IndexerArgs a, int s1_base_stride)
+template <int S1>
+__global__ __launch_bounds__(256) void indexer_score_kernel(IndexerArgs a)
 {
+    __shared__ uint32_t hist[S1][NBINS];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int l16 = lane & 15, g = lane >> 4;
     const int bi = blockIdx.y;
@@ -45,37 +62,44 @@ __global__ __launch_bounds__(256) void indexer_score_kernel(IndexerArgs a, int s
     const int tok_end = min(L, tok_begin + CHUNK);
     const int row0 = bi * a.s1 + sgrp * S1;
 
-    // A fragments: head hb*16 + l16, bytes 64*ks + 16*g .. +15
-    i32x4 qf[S1][NHB][2];
-    float wsc[S1][NHB][4]; // fp32(w_scale) of heads hb*16 + 4*g + r
+    for (int i = tid; i < S1 * NBINS; i += 256) (&hist[0][0])[i] = 0;
+
+    // int8 A fragments: head hb*16 + l16, bytes 64*ks + 16*g .. +15
+    i32x4 qf[S1][4][2];
+    // fp16 A fragments of the head sum: row 0 (lanes with l16 == 0) holds w_scale, k-slot (g, e) of MFMA mm is
+    // head 32*mm + 16*(e/4) + 4*g + e%4 - the head whose int32 result this lane group holds in that slot
+    f16x8 wa[S1][2];
 #pragma unroll
-    for (int s = 0; s < S1; ++s)
+    for (int s = 0; s < S1; ++s) {
 #pragma unroll
-        for (int hb = 0; hb < NHB; ++hb) {
+        for (int hb = 0; hb < 4; ++hb) {
             const int8_t* qp = a.q + ((int64_t)(row0 + s) * a.nh + hb * 16 + l16) * D + 16 * g;
             qf[s][hb][0] = *reinterpret_cast<const i32x4*>(qp);
             qf[s][hb][1] = *reinterpret_cast<const i32x4*>(qp + 64);
+        }
 #pragma unroll
-            for (int r = 0; r < 4; ++r) {
-                const int64_t h = (int64_t)(row0 + s) * a.nh + hb * 16 + 4 * g + r;
+        for (int mm = 0; mm < 2; ++mm)
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+                const int64_t h = (int64_t)(row0 + s) * a.nh + 32 * mm + 16 * (e >> 2) + 4 * g + (e & 3);
                 const _Float16 qs = __builtin_bit_cast(_Float16, a.q_scale[h]);
                 const _Float16 w = __builtin_bit_cast(_Float16, a.weights[h]);
-                wsc[s][hb][r] = (float)(_Float16)(qs * w); // one fp16 rounding
+                wa[s][mm][e] = l16 == 0 ? (_Float16)(qs * w) : (_Float16)0.f; // one fp16 rounding
             }
-        }
+    }
+    __syncthreads(); // histogram zeroed
 
     for (int t0 = tok_begin + wave * 16; t0 < tok_end; t0 += 64) {
         const int tok = t0 + l16;
         const bool ok = tok < tok_end;
-        int64_t krow = 0;
+        int64_t krow = -1;
         if (ok) {
             const int page = a.block_table[(int64_t)bi * a.bt_stride + tok / a.block_size];
-            krow = (int64_t)page * a.block_size + tok % a.block_size;
-            if (page < 0 || page >= a.n_blocks) krow = -1;
+            if (page >= 0 && page < a.n_blocks) krow = (int64_t)page * a.block_size + tok % a.block_size;
         }
         i32x4 kf0 = {0, 0, 0, 0}, kf1 = {0, 0, 0, 0};
         float ksc = 0.f;
-        if (ok && krow >= 0) {
+        if (krow >= 0) {
             const int8_t* kp = a.k_cache + krow * D + 16 * g;
             kf0 = *reinterpret_cast<const i32x4*>(kp);
             kf1 = *reinterpret_cast<const i32x4*>(kp + 64);
@@ -83,34 +107,43 @@ __global__ __launch_bounds__(256) void indexer_score_kernel(IndexerArgs a, int s
         }
 #pragma unroll
         for (int s = 0; s < S1; ++s) {
-            float part = 0.f;
+            f16x8 y[2];
 #pragma unroll
-            for (int hb = 0; hb < NHB; ++hb) {
+            for (int hb = 0; hb < 4; ++hb) {
                 i32x4 acc = {0, 0, 0, 0};
                 acc = __builtin_amdgcn_mfma_i32_16x16x64_i8(qf[s][hb][0], kf0, acc, 0, 0, 0);
                 acc = __builtin_amdgcn_mfma_i32_16x16x64_i8(qf[s][hb][1], kf1, acc, 0, 0, 0);
 #pragma unroll
-                for (int r = 0; r < 4; ++r) {
-                    const float x = (float)max(acc[r], 0) * (1.0f / 2048.0f);
-                    const float y = (float)(_Float16)x;
-                    part = __builtin_fmaf(wsc[s][hb][r], y, part);
-                }
+                for (int r = 0; r < 4; ++r)
+                    y[hb >> 1][4 * (hb & 1) + r] = (_Float16)((float)max(acc[r], 0) * (1.0f / 2048.0f));
             }
-            part += __shfl_xor(part, 16);
-            part += __shfl_xor(part, 32);
-            if (ok && g == 0) a.scores[(int64_t)(row0 + s) * a.score_stride + tok] = part * ksc;
+            f32x4 sum = {0.f, 0.f, 0.f, 0.f};
+            sum = __builtin_amdgcn_mfma_f32_16x16x32_f16(wa[s][0], y[0], sum, 0, 0, 0);
+            sum = __builtin_amdgcn_mfma_f32_16x16x32_f16(wa[s][1], y[1], sum, 0, 0, 0);
+            // row 0 of the result: register 0 of lanes 0..15, one key each
+            const int eff = L - (a.s1 - 1 - (sgrp * S1 + s));
+            if (ok && g == 0) {
+                const float sc = sum[0] * ksc;
+                a.scores[(int64_t)(row0 + s) * a.score_stride + tok] = sc;
+                if (tok < eff) atomicAdd(&hist[s][score_key(sc) >> 21], 1u);
+            }
         }
+    }
+    __syncthreads();
+    for (int i = tid; i < S1 * NBINS; i += 256) {
+        const uint32_t c = (&hist[0][0])[i];
+        if (c) atomicAdd(a.hist + (int64_t)(row0 + i / NBINS) * NBINS + (i % NBINS), c);
     }
 }
 
-__device__ __forceinline__ uint32_t score_key(float f) { return f32_to_ordered(f + 0.0f); } // -0 -> +0
-
-__device__ __forceinline__ uint64_t make_cand(uint32_t key, int idx)
+__global__ void indexer_zero_kernel(uint32_t* p, int n)
 {
-    return ((uint64_t)key << 32) | (uint32_t)(0xffffffffu - (uint32_t)idx);
+    const int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) p[i] = 0u;
 }
 
-// block-wide inclusive suffix sum over 1024 lanes (lane t gets sum of v[t..1023]); tmp holds 16 words
+// block-wide inclusive suffix sum (lane t gets sum of v[t .. nthreads-1]); tmp holds one word per wavefront
+template <int NWAVES>
 __device__ __forceinline__ uint32_t block_suffix_sum(uint32_t v, uint32_t* tmp)
 {
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
@@ -123,114 +156,199 @@ __device__ __forceinline__ uint32_t block_suffix_sum(uint32_t v, uint32_t* tmp)
     if (lane == 0) tmp[wave] = v;
     __syncthreads();
     uint32_t add = 0;
-    for (int w = wave + 1; w < 16; ++w) add += tmp[w];
+    for (int w = wave + 1; w < NWAVES; ++w) add += tmp[w];
     return v + add;
 }
 
-__global__ __launch_bounds__(1024) void indexer_topk_kernel(const float* __restrict__ scores, int score_stride,
-                                                            const int32_t* __restrict__ act_seq, int s1, int k,
-                                                            int32_t* __restrict__ out)
+// Valid length of query token `row`'s score row.
+__device__ __forceinline__ int row_length(const int32_t* act_seq, int row, int s1, int cap)
 {
-    __shared__ uint32_t hist[2048];
-    __shared__ uint64_t cand[MAX_K];
-    __shared__ uint32_t tmp[16];
-    __shared__ uint32_t s_bin, s_krem, s_cnt_gt, s_cnt_eq, s_bin_count;
-
-    const int tid = threadIdx.x;
-    const int row = blockIdx.x;
     const int bi = row / s1, si = row - bi * s1;
-    int n = act_seq[bi] - (s1 - 1 - si);
-    n = min(max(n, 0), score_stride);
-    const float* x = scores + (int64_t)row * score_stride;
+    return min(max(act_seq[bi] - (s1 - 1 - si), 0), cap);
+}
 
-    for (int i = tid; i < MAX_K; i += 1024) cand[i] = 0ull;
+// grid (chunks of SEL_CHUNK scores, query tokens), 256 lanes
+__global__ __launch_bounds__(256) void indexer_select_kernel(IndexerArgs a)
+{
+    __shared__ uint32_t tmp[4];
+    __shared__ uint32_t s_bin, s_base_gt, s_base_tie;
+    const int tid = threadIdx.x, row = blockIdx.y;
+    const int n = row_length(a.act_seq, row, a.s1, a.score_stride);
+    const int i_begin = blockIdx.x * SEL_CHUNK;
+    if (i_begin >= n) return;
+    if (tid == 0) s_bin = 0xffffffffu; // n <= k: no threshold bin, everything is a winner
+
+    // bin of the k-th largest key: lane t owns bins 8t .. 8t+7
+    const uint32_t* hist = a.hist + (int64_t)row * NBINS;
+    const u32x4 ha = *reinterpret_cast<const u32x4*>(hist + 8 * tid);
+    const u32x4 hb = *reinterpret_cast<const u32x4*>(hist + 8 * tid + 4);
+    const uint32_t h[8] = {ha[0], ha[1], ha[2], ha[3], hb[0], hb[1], hb[2], hb[3]};
+    uint32_t own = 0;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) own += h[j];
+    uint32_t above = block_suffix_sum<4>(own, tmp) - own; // elements in bins > 8t+7
+    const uint32_t k = (uint32_t)a.k;
+#pragma unroll
+    for (int j = 7; j >= 0; --j) {
+        if (above < k && k <= above + h[j]) s_bin = 8 * tid + j;
+        above += h[j];
+    }
     __syncthreads();
+    const uint32_t bin = s_bin;
 
-    if (n <= k) {
-        for (int i = tid; i < n; i += 1024) cand[i] = make_cand(score_key(x[i]), i);
-    } else {
-        uint32_t prefix = 0; // key bits already fixed (aligned to the top)
-        uint32_t krem = (uint32_t)k;
-        uint32_t eq_total = 0;
-#pragma unroll 1
-        for (int pass = 0; pass < 3; ++pass) {
-            const int shift = pass == 0 ? 21 : (pass == 1 ? 10 : 0);
-            const int bits = pass == 2 ? 10 : 11;
-            const uint32_t mask = (1u << bits) - 1u;
-            hist[tid] = 0;
-            hist[tid + 1024] = 0;
-            __syncthreads();
-            for (int i = tid; i < n; i += 1024) {
-                const uint32_t u = score_key(x[i]);
-                const bool in = pass == 0 || (u >> (shift + bits)) == (prefix >> (shift + bits));
-                if (in) atomicAdd(&hist[(u >> shift) & mask], 1u);
-            }
-            __syncthreads();
-            // lane t owns bins 2t (low) and 2t+1 (high)
-            const uint32_t h_lo = hist[2 * tid], h_hi = hist[2 * tid + 1];
-            const uint32_t incl = block_suffix_sum(h_lo + h_hi, tmp);
-            const uint32_t above_hi = incl - h_lo - h_hi; // elements in bins > 2t+1
-            const uint32_t above_lo = above_hi + h_hi;     // elements in bins > 2t
-            if (above_hi < krem && krem <= above_hi + h_hi) {
-                s_bin = 2 * tid + 1;
-                s_krem = krem - above_hi;
-                s_bin_count = h_hi;
-            } else if (above_lo < krem && krem <= above_lo + h_lo) {
-                s_bin = 2 * tid;
-                s_krem = krem - above_lo;
-                s_bin_count = h_lo;
-            }
-            __syncthreads();
-            prefix |= s_bin << shift;
-            krem = s_krem;
-            eq_total = s_bin_count;
-            __syncthreads();
+    // file this workgroup's scores: 16 per lane
+    const float* x = a.scores + (int64_t)row * a.score_stride;
+    f32x4 v[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) v[j] = *reinterpret_cast<const f32x4*>(x + min(i_begin + 4 * (j * 256 + tid), a.score_stride - 4));
+    uint32_t key[16];
+    uint32_t c_gt = 0, c_tie = 0;
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+#pragma unroll
+        for (int c = 0; c < 4; ++c) {
+            const int i = i_begin + 4 * (j * 256 + tid) + c;
+            const uint32_t u = score_key(v[j][c]);
+            key[4 * j + c] = u;
+            const uint32_t b = u >> 21;
+            const bool in = i < n;
+            c_gt += in && (bin == 0xffffffffu || b > bin) ? 1u : 0u;
+            c_tie += in && b == bin ? 1u : 0u;
         }
-        // prefix = k-th largest key; take every key above it and the krem smallest indices equal to it
-        const uint32_t n_gt = (uint32_t)k - krem;
-        if (tid == 0) {
-            s_cnt_gt = 0;
-            s_cnt_eq = 0;
+    const uint32_t packed = block_suffix_sum<4>(c_gt | (c_tie << 16), tmp);
+    if (tid == 0) {
+        uint32_t* cnt = a.counters + (int64_t)row * 4;
+        s_base_gt = atomicAdd(cnt, packed & 0xffffu);
+        s_base_tie = atomicAdd(cnt + 1, packed >> 16);
+    }
+    __syncthreads();
+    uint32_t p_gt = s_base_gt + (packed & 0xffffu) - c_gt;
+    uint32_t p_tie = s_base_tie + (packed >> 16) - c_tie;
+    uint64_t* winners = a.winners + (int64_t)row * MAX_K;
+    uint64_t* ties = a.ties + (int64_t)row * TIE_CAP;
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+#pragma unroll
+        for (int c = 0; c < 4; ++c) {
+            const int i = i_begin + 4 * (j * 256 + tid) + c;
+            if (i >= n) continue;
+            const uint32_t u = key[4 * j + c], b = u >> 21;
+            if (bin == 0xffffffffu || b > bin) {
+                if (p_gt < MAX_K) winners[p_gt] = make_cand(u, i);
+                ++p_gt;
+            } else if (b == bin) {
+                if (p_tie < TIE_CAP) ties[p_tie] = make_cand(u, i);
+                ++p_tie;
+            }
+        }
+}
+
+// Radix-select the `need` largest of the 64-bit words f enumerates (all share the bits above `top`), top-down
+// in digits of 11 bits; every selected word is handed to emit().  Words are distinct, so the walk ends with a
+// bin that is taken whole.  Workgroup of 1024 lanes; hist has 2048 words, tmp 16.
+template <class Each, class Emit>
+__device__ __forceinline__ void radix_select64(Each&& for_each, Emit&& emit, uint32_t need, int top, uint32_t* hist,
+                                               uint32_t* tmp, uint32_t* s_bin, uint32_t* s_krem, uint32_t* s_cnt)
+{
+    const int tid = threadIdx.x;
+    uint64_t prefix = 0, known = 0; // bits fixed so far and their mask
+    while (need > 0 && top > 0) {
+        const int bits = top >= 11 ? 11 : top;
+        const int shift = top - bits;
+        const uint64_t dmask = (1ull << bits) - 1ull;
+        hist[tid] = 0;
+        hist[tid + 1024] = 0;
+        __syncthreads();
+        for_each([&](uint64_t w) {
+            if ((w & known) == prefix) atomicAdd(&hist[(uint32_t)((w >> shift) & dmask)], 1u);
+        });
+        __syncthreads();
+        const uint32_t h_lo = hist[2 * tid], h_hi = hist[2 * tid + 1]; // lane t owns bins 2t and 2t+1
+        const uint32_t incl = block_suffix_sum<16>(h_lo + h_hi, tmp);
+        const uint32_t above_hi = incl - h_lo - h_hi, above_lo = above_hi + h_hi;
+        if (above_hi < need && need <= above_hi + h_hi) {
+            *s_bin = 2 * tid + 1;
+            *s_krem = need - above_hi;
+            *s_cnt = h_hi;
+        } else if (above_lo < need && need <= above_lo + h_lo) {
+            *s_bin = 2 * tid;
+            *s_krem = need - above_lo;
+            *s_cnt = h_lo;
         }
         __syncthreads();
-        const bool take_all_eq = eq_total == krem;
-        for (int i = tid; i < n; i += 1024) {
-            const uint32_t u = score_key(x[i]);
-            if (u > prefix) {
-                cand[atomicAdd(&s_cnt_gt, 1u)] = make_cand(u, i);
-            } else if (take_all_eq && u == prefix) {
-                cand[n_gt + atomicAdd(&s_cnt_eq, 1u)] = make_cand(u, i);
+        const uint64_t b = *s_bin;
+        const uint32_t krem = *s_krem, cnt = *s_cnt;
+        // everything in the bins above b is selected; bin b whole if it is exactly what is missing
+        const bool whole = cnt == krem;
+        for_each([&](uint64_t w) {
+            if ((w & known) != prefix) return;
+            const uint64_t d = (w >> shift) & dmask;
+            if (d > b || (whole && d == b)) emit(w);
+        });
+        __syncthreads();
+        if (whole) return;
+        prefix |= b << shift;
+        known |= dmask << shift;
+        need = krem;
+        top = shift;
+    }
+}
+
+__global__ __launch_bounds__(1024) void indexer_topk_kernel(IndexerArgs a)
+{
+    __shared__ uint32_t hist[NBINS];
+    __shared__ uint64_t cand[MAX_K];
+    __shared__ uint64_t tie[TIE_CAP];
+    __shared__ uint32_t tmp[16];
+    __shared__ uint32_t s_bin, s_krem, s_cnt, s_out;
+
+    const int tid = threadIdx.x, row = blockIdx.x;
+    const int n = row_length(a.act_seq, row, a.s1, a.score_stride);
+    const int k = a.k;
+    const uint32_t n_gt = min(a.counters[(int64_t)row * 4], (uint32_t)MAX_K);
+    const uint32_t n_tie = a.counters[(int64_t)row * 4 + 1];
+    const uint32_t need = (uint32_t)min(n, k) - min(n_gt, (uint32_t)min(n, k));
+
+    for (int i = tid; i < MAX_K; i += 1024) cand[i] = i < (int)n_gt ? a.winners[(int64_t)row * MAX_K + i] : 0ull;
+    if (tid == 0) s_out = n_gt;
+    __syncthreads();
+    auto emit = [&](uint64_t w) {
+        const uint32_t p = atomicAdd(&s_out, 1u);
+        if (p < MAX_K) cand[p] = w;
+    };
+
+    if (need > 0 && n_tie <= TIE_CAP) {
+        // the usual case: the tie list (one histogram bin) fits in LDS; its words share the top 11 bits
+        for (int i = tid; i < (int)n_tie; i += 1024) tie[i] = a.ties[(int64_t)row * TIE_CAP + i];
+        __syncthreads();
+        auto each = [&](auto&& f) {
+            for (int i = tid; i < (int)n_tie; i += 1024) f(tie[i]);
+        };
+        radix_select64(each, emit, need, 53, hist, tmp, &s_bin, &s_krem, &s_cnt);
+    } else if (need > 0) {
+        // overflowed tie list: select over the whole row instead (winners are found again, so start empty)
+        if (tid == 0) s_out = 0;
+        __syncthreads();
+        const float* x = a.scores + (int64_t)row * a.score_stride;
+        auto each = [&](auto&& f) {
+            for (int i0 = 4 * tid; i0 < n; i0 += 4096) {
+                const f32x4 v = *reinterpret_cast<const f32x4*>(x + i0);
+#pragma unroll
+                for (int c = 0; c < 4; ++c)
+                    if (i0 + c < n) f(make_cand(score_key(v[c]), i0 + c));
             }
-        }
-        if (!take_all_eq) {
-            // more ties than slots: walk the row in index order and keep the first krem of them
-            uint32_t base = 0;
-            for (int i0 = 0; i0 < n && base < krem; i0 += 1024) {
-                const int i = i0 + tid;
-                const bool eq = i < n && score_key(x[i]) == prefix;
-                const uint64_t bal = __ballot(eq);
-                const int lane = tid & 63, wave = tid >> 6;
-                const uint32_t in_wave = __popcll(bal & ((1ull << lane) - 1ull));
-                __syncthreads();
-                if (lane == 0) tmp[wave] = __popcll(bal);
-                __syncthreads();
-                uint32_t before = 0, total = 0;
-                for (int w = 0; w < 16; ++w) {
-                    const uint32_t c = tmp[w];
-                    before += w < wave ? c : 0;
-                    total += c;
-                }
-                const uint32_t rank = base + before + in_wave;
-                if (eq && rank < krem) cand[n_gt + rank] = make_cand(prefix, i);
-                base += total;
-            }
-        }
+        };
+        radix_select64(each, emit, (uint32_t)min(n, k), 64, hist, tmp, &s_bin, &s_krem, &s_cnt);
     }
     __syncthreads();
 
-    // bitonic sort, descending, 2048 words, two per lane
+    // bitonic sort, descending, 2048 words, two per lane.  A compare-exchange step of stride <= 64 stays inside
+    // the 128 words owned by one wavefront (lane i of wave w handles the pair (128w + 2i - i%stride, + stride)),
+    // so only the steps of stride >= 128 need a workgroup barrier; the others rely on LDS operations of one
+    // wavefront completing in order.
     for (int size = 2; size <= MAX_K; size <<= 1) {
         for (int stride = size >> 1; stride > 0; stride >>= 1) {
+            if (stride >= 128) __syncthreads();
             const int pos = 2 * tid - (tid & (stride - 1)); // lower index of the pair
             const bool desc = (pos & size) == 0;
             const uint64_t lo = cand[pos], hi = cand[pos + stride];
@@ -238,37 +356,64 @@ __global__ __launch_bounds__(1024) void indexer_topk_kernel(const float* __restr
                 cand[pos] = hi;
                 cand[pos + stride] = lo;
             }
-            __syncthreads();
+            if (stride >= 128) __syncthreads();
+            else __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
         }
     }
+    __syncthreads();
     for (int j = tid; j < k; j += 1024)
-        out[(int64_t)row * k + j] = (int32_t)(0xffffffffu - (uint32_t)(cand[j] & 0xffffffffull));
+        a.topk_res[(int64_t)row * k + j] = (int32_t)(0xffffffffu - (uint32_t)(cand[j] & 0xffffffffull));
 }
 
 } // namespace
 
-uint64_t indexer_workspace_bytes(int t, int max_ctx) { return (uint64_t)t * (uint64_t)max_ctx * sizeof(float); }
+// workspace: scores [t, stride] f32 | hist [t, 2048] u32 | counters [t, 4] u32 | winners [t, 2048] u64 | ties [t, 8192] u64
+static uint64_t align256(uint64_t x) { return (x + 255) & ~(uint64_t)255; }
+
+uint64_t indexer_workspace_bytes(int t, int stride)
+{
+    return align256((uint64_t)t * stride * 4) + align256((uint64_t)t * (NBINS + 4) * 4) +
+           (uint64_t)t * (MAX_K + TIE_CAP) * 8;
+}
+
+void indexer_bind_workspace(IndexerArgs& a, void* ws)
+{
+    const int t = a.b * a.s1;
+    uint8_t* p = static_cast<uint8_t*>(ws);
+    a.scores = reinterpret_cast<float*>(p);
+    p += align256((uint64_t)t * a.score_stride * 4);
+    a.hist = reinterpret_cast<uint32_t*>(p);
+    a.counters = a.hist + (uint64_t)t * NBINS;
+    p += align256((uint64_t)t * (NBINS + 4) * 4);
+    a.winners = reinterpret_cast<uint64_t*>(p);
+    a.ties = a.winners + (uint64_t)t * MAX_K;
+}
 
 hipError_t indexer_launch(const IndexerArgs& a, hipStream_t stream)
 {
     const int t = a.b * a.s1;
     if (t == 0) return hipSuccess;
-    const int max_ctx = a.score_stride;
+    const int max_ctx = a.bt_stride * a.block_size;
     const int chunks = (max_ctx + CHUNK - 1) / CHUNK;
+    const int nzero = t * (NBINS + 4);
+    hipLaunchKernelGGL(indexer_zero_kernel, dim3((nzero + 255) / 256), dim3(256), 0, stream, a.hist, nzero);
     {
         ScopedKernelTimer tm(KID_INDEXER_SCORE, stream);
         if (a.s1 % 2 == 0) {
-            hipLaunchKernelGGL((indexer_score_kernel<2, 4>), dim3(chunks, a.b, a.s1 / 2), dim3(256), 0, stream, a, 0);
+            hipLaunchKernelGGL((indexer_score_kernel<2>), dim3(chunks, a.b, a.s1 / 2), dim3(256), 0, stream, a);
         } else {
-            hipLaunchKernelGGL((indexer_score_kernel<1, 4>), dim3(chunks, a.b, a.s1), dim3(256), 0, stream, a, 0);
+            hipLaunchKernelGGL((indexer_score_kernel<1>), dim3(chunks, a.b, a.s1), dim3(256), 0, stream, a);
         }
     }
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) return e;
     {
+        ScopedKernelTimer tm(KID_INDEXER_SELECT, stream);
+        hipLaunchKernelGGL(indexer_select_kernel, dim3((max_ctx + SEL_CHUNK - 1) / SEL_CHUNK, t), dim3(256), 0, stream, a);
+    }
+    {
         ScopedKernelTimer tm(KID_INDEXER_TOPK, stream);
-        hipLaunchKernelGGL(indexer_topk_kernel, dim3(t), dim3(1024), 0, stream, a.scores, a.score_stride, a.act_seq,
-                           a.s1, a.k, a.topk_res);
+        hipLaunchKernelGGL(indexer_topk_kernel, dim3(t), dim3(1024), 0, stream, a);
     }
     return hipGetLastError();
 }

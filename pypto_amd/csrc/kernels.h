@@ -42,11 +42,16 @@ struct IndexerArgs {
     const int32_t* block_table;  // [b, bt_stride]
     int32_t* topk_res;           // [t, k]
     float* scores;               // workspace [t, score_stride]
+    uint32_t* hist;              // workspace [t, 2048]: histogram of the top 11 bits of the score keys
+    uint32_t* counters;          // workspace [t, 4]: winners, ties
+    uint64_t* winners;           // workspace [t, 2048]
+    uint64_t* ties;              // workspace [t, 8192]
     int64_t n_blocks;
     int32_t b, s1, nh, block_size, bt_stride, k, score_stride;
 };
 
-uint64_t indexer_workspace_bytes(int t, int max_ctx);
+uint64_t indexer_workspace_bytes(int t, int score_stride);
+void indexer_bind_workspace(IndexerArgs& a, void* workspace);
 hipError_t indexer_launch(const IndexerArgs& a, hipStream_t stream);
 
 } // namespace pto
