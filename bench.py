@@ -135,7 +135,7 @@ def main():
     lib.pto_kernel_timing_enable(0)
     lib.pto_kernel_name.restype = ctypes.c_char_p
     kernels = {}
-    for kid in range(4):
+    for kid in range(5):
         ms, n = ctypes.c_double(0), ctypes.c_uint64(0)
         lib.pto_kernel_timing_read(kid, ctypes.byref(ms), ctypes.byref(n))
         if n.value:
@@ -154,6 +154,7 @@ def main():
         "indexer_topk_kernel": {"bound": "hbm", "work": topk_bytes, "peak": HBM_PEAK_GBS, "unit": "GB/s"},
         "sfa_decode_kernel": {"bound": "mfma", "work": sfa_flops, "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s"},
         "sfa_combine_kernel": {"bound": "hbm", "work": t * 128 * 512 * 2, "peak": HBM_PEAK_GBS, "unit": "GB/s"},
+        "indexer_select_kernel": {"bound": "hbm", "work": t * L * 4, "peak": HBM_PEAK_GBS, "unit": "GB/s"},
     }
     per_kernel = []
     for name, us in kernels.items():

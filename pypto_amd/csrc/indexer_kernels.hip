@@ -34,7 +34,8 @@ namespace pto {
 namespace {
 
 constexpr int D = 128;          // index head dim
-constexpr int CHUNK = 512;      // keys per workgroup of the score kernel
+constexpr int CHUNK = 512;      // keys per pass of a workgroup of the score kernel (8 groups of 16 per wavefront)
+constexpr int PASSES = 4;       // passes per workgroup (amortise the Q / w_scale set-up)
 constexpr int MAX_K = 2048;     // top-k capacity
 constexpr int NBINS = 2048;     // histogram over the top 11 key bits
 constexpr int SEL_CHUNK = 4096; // scores per workgroup of the select kernel
@@ -48,7 +49,8 @@ __device__ __forceinline__ uint64_t make_cand(uint32_t key, int idx)
 }
 
 // S1 query tokens of one sequence share every key fragment.
-template <int S1>
+// POW2: block_size is a power of two (page index by shift instead of an integer division per key).
+template <int S1, bool POW2>
 __global__ __launch_bounds__(256) void indexer_score_kernel(IndexerArgs a)
 {
     __shared__ uint32_t hist[S1][NBINS];
@@ -57,9 +59,7 @@ __global__ __launch_bounds__(256) void indexer_score_kernel(IndexerArgs a)
     const int bi = blockIdx.y;
     const int sgrp = blockIdx.z; // group of S1 consecutive query tokens of the sequence
     const int L = a.act_seq[bi];
-    const int tok_begin = blockIdx.x * CHUNK;
-    if (tok_begin >= L) return;
-    const int tok_end = min(L, tok_begin + CHUNK);
+    if (blockIdx.x * (CHUNK * PASSES) >= L) return;
     const int row0 = bi * a.s1 + sgrp * S1;
 
     for (int i = tid; i < S1 * NBINS; i += 256) (&hist[0][0])[i] = 0;
@@ -89,30 +89,50 @@ __global__ __launch_bounds__(256) void indexer_score_kernel(IndexerArgs a)
     }
     __syncthreads(); // histogram zeroed
 
-    for (int t0 = tok_begin + wave * 16; t0 < tok_end; t0 += 64) {
-        const int tok = t0 + l16;
+    for (int pass = 0; pass < PASSES; ++pass) {
+    const int tok_begin = (blockIdx.x * PASSES + pass) * CHUNK;
+    if (tok_begin >= L) break;
+    const int tok_end = min(L, tok_begin + CHUNK);
+    // Each wavefront owns 8 groups of 16 keys.  All page-table lookups are issued first, then all key loads
+    // (absent keys read row 0 and get scale 0), so that 4 KB per wavefront are in flight before the first MFMA.
+    constexpr int STEPS = CHUNK / 64;
+    const int bs = a.block_size, bs_shift = __builtin_ctz(bs);
+    int page[STEPS], tk[STEPS];
+#pragma unroll
+    for (int j = 0; j < STEPS; ++j) {
+        tk[j] = min(tok_begin + wave * 16 + 64 * j + l16, tok_end - 1);
+        const int pi = POW2 ? tk[j] >> bs_shift : tk[j] / bs;
+        page[j] = a.block_table[(int64_t)bi * a.bt_stride + pi];
+    }
+    int64_t krow[STEPS];
+    bool present[STEPS];
+#pragma unroll
+    for (int j = 0; j < STEPS; ++j) {
+        const int in_page = POW2 ? tk[j] & (bs - 1) : tk[j] % bs;
+        present[j] = tok_begin + wave * 16 + 64 * j + l16 < tok_end && page[j] >= 0 && page[j] < a.n_blocks;
+        krow[j] = present[j] ? (int64_t)page[j] * bs + in_page : 0;
+    }
+    i32x4 kf0[STEPS], kf1[STEPS];
+    uint16_t ksb[STEPS];
+#pragma unroll
+    for (int j = 0; j < STEPS; ++j) {
+        const int8_t* kp = a.k_cache + krow[j] * D + 16 * g;
+        kf0[j] = *reinterpret_cast<const i32x4*>(kp);
+        kf1[j] = *reinterpret_cast<const i32x4*>(kp + 64);
+        ksb[j] = a.k_scale[krow[j]];
+    }
+#pragma unroll
+    for (int j = 0; j < STEPS; ++j) {
+        const int tok = tok_begin + wave * 16 + 64 * j + l16;
         const bool ok = tok < tok_end;
-        int64_t krow = -1;
-        if (ok) {
-            const int page = a.block_table[(int64_t)bi * a.bt_stride + tok / a.block_size];
-            if (page >= 0 && page < a.n_blocks) krow = (int64_t)page * a.block_size + tok % a.block_size;
-        }
-        i32x4 kf0 = {0, 0, 0, 0}, kf1 = {0, 0, 0, 0};
-        float ksc = 0.f;
-        if (krow >= 0) {
-            const int8_t* kp = a.k_cache + krow * D + 16 * g;
-            kf0 = *reinterpret_cast<const i32x4*>(kp);
-            kf1 = *reinterpret_cast<const i32x4*>(kp + 64);
-            ksc = f16_bits_to_f32(a.k_scale[krow]);
-        }
 #pragma unroll
         for (int s = 0; s < S1; ++s) {
             f16x8 y[2];
 #pragma unroll
             for (int hb = 0; hb < 4; ++hb) {
                 i32x4 acc = {0, 0, 0, 0};
-                acc = __builtin_amdgcn_mfma_i32_16x16x64_i8(qf[s][hb][0], kf0, acc, 0, 0, 0);
-                acc = __builtin_amdgcn_mfma_i32_16x16x64_i8(qf[s][hb][1], kf1, acc, 0, 0, 0);
+                acc = __builtin_amdgcn_mfma_i32_16x16x64_i8(qf[s][hb][0], kf0[j], acc, 0, 0, 0);
+                acc = __builtin_amdgcn_mfma_i32_16x16x64_i8(qf[s][hb][1], kf1[j], acc, 0, 0, 0);
 #pragma unroll
                 for (int r = 0; r < 4; ++r)
                     y[hb >> 1][4 * (hb & 1) + r] = (_Float16)((float)max(acc[r], 0) * (1.0f / 2048.0f));
@@ -123,12 +143,13 @@ __global__ __launch_bounds__(256) void indexer_score_kernel(IndexerArgs a)
             // row 0 of the result: register 0 of lanes 0..15, one key each
             const int eff = L - (a.s1 - 1 - (sgrp * S1 + s));
             if (ok && g == 0) {
-                const float sc = sum[0] * ksc;
+                const float sc = sum[0] * (present[j] ? f16_bits_to_f32(ksb[j]) : 0.f);
                 a.scores[(int64_t)(row0 + s) * a.score_stride + tok] = sc;
                 if (tok < eff) atomicAdd(&hist[s][score_key(sc) >> 21], 1u);
             }
         }
     }
+    } // pass
     __syncthreads();
     for (int i = tid; i < S1 * NBINS; i += 256) {
         const uint32_t c = (&hist[0][0])[i];
@@ -394,15 +415,18 @@ hipError_t indexer_launch(const IndexerArgs& a, hipStream_t stream)
     const int t = a.b * a.s1;
     if (t == 0) return hipSuccess;
     const int max_ctx = a.bt_stride * a.block_size;
-    const int chunks = (max_ctx + CHUNK - 1) / CHUNK;
+    const int chunks = (max_ctx + CHUNK * PASSES - 1) / (CHUNK * PASSES);
     const int nzero = t * (NBINS + 4);
     hipLaunchKernelGGL(indexer_zero_kernel, dim3((nzero + 255) / 256), dim3(256), 0, stream, a.hist, nzero);
     {
         ScopedKernelTimer tm(KID_INDEXER_SCORE, stream);
+        const bool pow2 = (a.block_size & (a.block_size - 1)) == 0;
         if (a.s1 % 2 == 0) {
-            hipLaunchKernelGGL((indexer_score_kernel<2>), dim3(chunks, a.b, a.s1 / 2), dim3(256), 0, stream, a);
+            auto kern = pow2 ? indexer_score_kernel<2, true> : indexer_score_kernel<2, false>;
+            hipLaunchKernelGGL(kern, dim3(chunks, a.b, a.s1 / 2), dim3(256), 0, stream, a);
         } else {
-            hipLaunchKernelGGL((indexer_score_kernel<1>), dim3(chunks, a.b, a.s1), dim3(256), 0, stream, a);
+            auto kern = pow2 ? indexer_score_kernel<1, true> : indexer_score_kernel<1, false>;
+            hipLaunchKernelGGL(kern, dim3(chunks, a.b, a.s1), dim3(256), 0, stream, a);
         }
     }
     hipError_t e = hipGetLastError();
