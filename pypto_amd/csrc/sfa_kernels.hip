@@ -100,13 +100,14 @@ __device__ __forceinline__ void load_raw(RawTile<QUANT>& r, const SfaArgs& a, co
 
 __device__ __forceinline__ float i8_at(uint32_t w, int k) { return (float)(int8_t)(w >> (8 * k)); }
 
-// Dequantise this lane's 8 rows x 8 columns and store them (and the rope piece) into an LDS stage.
-template <bool QUANT>
+// Dequantise rows [E0, E1) of this lane's 8 rows x 8 columns and store them into an LDS stage; with ROPE also
+// the lane's rope piece.
+template <bool QUANT, int E0, int E1, bool ROPE>
 __device__ __forceinline__ void dequant_store(const RawTile<QUANT>& r, uint8_t* stage, const float* scales, int tile,
                                               int wave, int lane, int tid)
 {
 #pragma unroll
-    for (int e = 0; e < 8; ++e) {
+    for (int e = E0; e < E1; ++e) {
         const int t = 8 * wave + e;
         u32x4 v;
         if constexpr (QUANT) {
@@ -125,11 +126,13 @@ __device__ __forceinline__ void dequant_store(const RawTile<QUANT>& r, uint8_t* 
         }
         *reinterpret_cast<u32x4*>(stage + t * KROW + ((lane ^ swz(t)) << 4)) = v;
     }
-    const int t = tid >> 3;
-    u32x4 rp = r.rope;
-    asm volatile("" : "+v"(rp));
-    rp = ((r.absent >> 8) & 1u) ? u32x4{0u, 0u, 0u, 0u} : rp;
-    *reinterpret_cast<u32x4*>(stage + t * KROW + DN * 2 + (((tid & 7) ^ swz(t)) << 4)) = rp;
+    if constexpr (ROPE) {
+        const int t = tid >> 3;
+        u32x4 rp = r.rope;
+        asm volatile("" : "+v"(rp));
+        rp = ((r.absent >> 8) & 1u) ? u32x4{0u, 0u, 0u, 0u} : rp;
+        *reinterpret_cast<u32x4*>(stage + t * KROW + DN * 2 + (((tid & 7) ^ swz(t)) << 4)) = rp;
+    }
 }
 
 template <bool QUANT>
@@ -188,17 +191,21 @@ __global__ __attribute__((amdgpu_flat_work_group_size(512, 512), amdgpu_waves_pe
         if (ntiles > 0) {
             load_raw<QUANT>(raw0, a, rows, 0, pw, lane, ptid);
             load_raw<QUANT>(raw1, a, rows, 1, pw, lane, ptid);
-            dequant_store<QUANT>(raw0, smem, scales, 0, pw, lane, ptid);
+            dequant_store<QUANT, 0, 8, true>(raw0, smem, scales, 0, pw, lane, ptid);
             load_raw<QUANT>(raw0, a, rows, min(2, last), pw, lane, ptid);
         }
         __syncthreads();
         // Every step stores one tile and issues the loads of another, unconditionally (past the end the last
         // tile is loaded again and stored into a stage nobody reads): with a fixed number of loads in flight
         // on every path the wait for a tile leaves the younger tile's loads outstanding.
+        // The consumers spend about a third of a tile before their mid-tile barrier (half of S) and two thirds
+        // after it (softmax, PV); the store of the next tile is split the same way around that barrier.
         auto produce = [&](int it, RawTile<QUANT>& next) {
-            dequant_store<QUANT>(next, smem + ((it + 1) & 1) * STAGE, scales, min(it + 1, last), pw, lane, ptid);
-            load_raw<QUANT>(next, a, rows, min(it + 3, last), pw, lane, ptid);
+            uint8_t* dst = smem + ((it + 1) & 1) * STAGE;
+            dequant_store<QUANT, 0, 3, false>(next, dst, scales, min(it + 1, last), pw, lane, ptid);
             __syncthreads();
+            dequant_store<QUANT, 3, 8, true>(next, dst, scales, min(it + 1, last), pw, lane, ptid);
+            load_raw<QUANT>(next, a, rows, min(it + 3, last), pw, lane, ptid);
             __syncthreads();
         };
         for (int it = 0; it < ntiles; it += 2) {
@@ -267,10 +274,28 @@ __global__ __attribute__((amdgpu_flat_work_group_size(512, 512), amdgpu_waves_pe
         f32x16 s;
 #pragma unroll
         for (int r = 0; r < 16; ++r) s[r] = 0.f;
+        {
+            // operand reads run three k-steps ahead of the MFMAs that use them
+            constexpr int AHEAD = 3;
+            bf16x8 kf[KSTEPS / 2];
 #pragma unroll
-        for (int i = 0; i < KSTEPS / 2; ++i) {
-            const bf16x8 kf = *reinterpret_cast<const bf16x8*>(stage + s_off[i & 1] + (i >> 1) * 128);
-            s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf, q[i], s, 0, 0, 0);
+            for (int i = 0; i < AHEAD; ++i)
+                kf[i] = *reinterpret_cast<const bf16x8*>(stage + s_off[i & 1] + (i >> 1) * 128);
+#pragma unroll
+            for (int i = 0; i < KSTEPS / 2; ++i) {
+                if (i + AHEAD < KSTEPS / 2)
+                    kf[i + AHEAD] =
+                        *reinterpret_cast<const bf16x8*>(stage + s_off[(i + AHEAD) & 1] + ((i + AHEAD) >> 1) * 128);
+                s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf[i], q[i], s, 0, 0, 0);
+            }
+            // issue order: AHEAD reads, then (MFMA, read) pairs, then the last MFMAs
+            __builtin_amdgcn_sched_group_barrier(0x100, AHEAD, 0);
+#pragma unroll
+            for (int i = 0; i < KSTEPS / 2 - AHEAD; ++i) {
+                __builtin_amdgcn_sched_group_barrier(0x008, 1, 0); // one MFMA
+                __builtin_amdgcn_sched_group_barrier(0x100, 1, 0); // one LDS read
+            }
+            __builtin_amdgcn_sched_group_barrier(0x008, AHEAD, 0);
         }
 #pragma unroll
         for (int g = 0; g < 4; ++g)
@@ -317,18 +342,37 @@ __global__ __attribute__((amdgpu_flat_work_group_size(512, 512), amdgpu_waves_pe
             }
             // O^T[dim, head] += V^T[dim, token] . P~[token, head]; k-slot s of half hl in block j is token
             // 16*j + 8*(s/4) + 4*hl + s%4, the order in which the S^T registers hold the tokens
+            {
+                bf16x8 pf[2];
 #pragma unroll
-            for (int j = 0; j < 2; ++j) {
-                u32x4 pw = {pb[4 * j], pb[4 * j + 1], pb[4 * j + 2], pb[4 * j + 3]};
-                const bf16x8 pf = __builtin_bit_cast(bf16x8, pw);
-#pragma unroll
-                for (int i = 0; i < 8; ++i) {
-                    uint8_t* vp = stage + v_off + (16 * j) * KROW + i * 128;
-                    const s16x4 lo = lds_read_tr(vp);
-                    const s16x4 hi = lds_read_tr(vp + 8 * KROW);
-                    const s16x8 both = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
-                    o[i] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, both), pf, o[i], 0, 0, 0);
+                for (int j = 0; j < 2; ++j) {
+                    u32x4 pw = {pb[4 * j], pb[4 * j + 1], pb[4 * j + 2], pb[4 * j + 3]};
+                    pf[j] = __builtin_bit_cast(bf16x8, pw);
                 }
+                // 16 MFMAs (j, i); their two transpose reads each run two MFMAs ahead
+                constexpr int AHEAD = 2;
+                s16x4 lo[16], hi[16];
+                auto vread = [&](int n) {
+                    uint8_t* vp = stage + v_off + (16 * (n >> 3)) * KROW + (n & 7) * 128;
+                    lo[n] = lds_read_tr(vp);
+                    hi[n] = lds_read_tr(vp + 8 * KROW);
+                };
+#pragma unroll
+                for (int n = 0; n < AHEAD; ++n) vread(n);
+#pragma unroll
+                for (int n = 0; n < 16; ++n) {
+                    if (n + AHEAD < 16) vread(n + AHEAD);
+                    const s16x8 both = __builtin_shufflevector(lo[n], hi[n], 0, 1, 2, 3, 4, 5, 6, 7);
+                    o[n & 7] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, both), pf[n >> 3],
+                                                                       o[n & 7], 0, 0, 0);
+                }
+                __builtin_amdgcn_sched_group_barrier(0x100, 2 * AHEAD, 0);
+#pragma unroll
+                for (int n = 0; n < 16 - AHEAD; ++n) {
+                    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0); // one MFMA
+                    __builtin_amdgcn_sched_group_barrier(0x100, 2, 0); // two LDS reads
+                }
+                __builtin_amdgcn_sched_group_barrier(0x008, AHEAD, 0);
             }
         }
         __syncthreads(); // tile consumed: its stage and the exchange buffer may be overwritten
