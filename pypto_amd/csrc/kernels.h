@@ -14,7 +14,7 @@ struct SfaArgs {
     const uint8_t* kn; // 512 x int8 (or 512 x bf16 when !quant)
     const uint8_t* kr; // 64 x bf16
     const uint8_t* ks; // 4 x fp32
-    int64_t kn_stride, kr_stride, ks_stride;
+    uint32_t kn_stride, kr_stride, ks_stride;
     int64_t n_rows;
     const int32_t* topk_idx;    // [t, topk_stride]
     const int32_t* block_table; // [b, bt_stride]
@@ -23,6 +23,8 @@ struct SfaArgs {
     float* part_o;              // [t, nsplit, nq, 512] fp32 (nsplit > 1)
     float* part_ml;             // [t, nsplit, nq, 2]  fp32 (running max in log2 units, sum)
     int32_t b, s1, nq, topk, topk_stride, block_size, bt_stride, nsplit;
+    int32_t split_cap; // set by sfa_launch: capacity (tokens) of the per-split LDS arrays
+    int32_t bt_cached; // set by sfa_launch: the sequence's page table fits in LDS
     float softmax_scale;
     bool quant;
 };

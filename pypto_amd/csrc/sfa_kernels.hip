@@ -37,11 +37,19 @@ constexpr int DR = 64;                 // rope width
 constexpr int KSTEPS = (DN + DR) / 16; // 36 MFMA k-steps for S, 18 per wave of a pair
 constexpr int KROW = (DN + DR) * 2;    // 1152 bytes per tile row = 72 chunks of 16 bytes
 constexpr int STAGE = T * KROW;        // 36864
-constexpr int MAX_SPLIT_TOKENS = 2048; // capacity of rows[] / scales[]
-constexpr int ROWS_OFF = 2 * STAGE;
-constexpr int SCALES_OFF = ROWS_OFF + MAX_SPLIT_TOKENS * 4;
-constexpr int XBUF_OFF = SCALES_OFF + MAX_SPLIT_TOKENS * 16;
-constexpr int SMEM_BYTES = XBUF_OFF + 4 * 4096; // 131072
+constexpr int MAX_SPLIT_TOKENS = 2048; // largest share of a top-k list one workgroup may own
+constexpr int NREG_KSTEPS = 12;        // of a wave's 18 k-steps of Q, these stay in registers ...
+constexpr int NPARK = KSTEPS / 2 - NREG_KSTEPS; // ... and these are parked in LDS (16 bytes per lane each)
+// LDS layout: two tile stages | S exchange | parked Q | per-split arrays sized by SfaArgs::split_cap
+// (validity words, rows, scales) | this sequence's page table (when it fits)
+constexpr int XBUF_OFF = 2 * STAGE;
+constexpr int QPARK_OFF = XBUF_OFF + 4 * 4096;
+constexpr int SPLIT_OFF = QPARK_OFF + 4 * NPARK * 1024; // 114688
+constexpr int LDS_LIMIT = 160 * 1024;
+constexpr int OUT_ROW = DN * 4;  // epilogue staging: 64 heads x 512 fp32, reusing the front of LDS
+__host__ __device__ constexpr int tmask_bytes(int cap) { return (cap / T + 2) * 4; }
+__host__ __device__ constexpr int split_bytes(int cap) { return tmask_bytes(cap) + cap * 4 + cap * 16; }
+static_assert(64 * OUT_ROW <= LDS_LIMIT, "epilogue staging must fit");
 constexpr int HEADS_PER_WG = 64;
 
 typedef short s16x4 __attribute__((ext_vector_type(4)));
@@ -72,33 +80,34 @@ struct RawTile<false> {
 };
 
 // Lane (wave w, lane l) fetches columns [8l, 8l+8) of tile rows 8w .. 8w+7 and one 16-byte piece of a rope row.
-// Absent rows (-1) read row 0 instead; `absent` keeps one bit per load and the data is zeroed when it is
-// consumed (dequant_store), so that no load has to be waited for here.
+// rows[] holds valid cache rows only (absent entries point at row 0); the tile's validity word says which
+// rows are absent, and their data is zeroed when it is consumed (dequant_store), so that no load has to be
+// waited for here.
 template <bool QUANT>
-__device__ __forceinline__ void load_raw(RawTile<QUANT>& r, const SfaArgs& a, const int* rows, int tile, int wave,
-                                         int lane, int tid)
+__device__ __forceinline__ void load_raw(RawTile<QUANT>& r, const SfaArgs& a, const int* rows, const uint32_t* tmask,
+                                         int tile, int wave, int lane, int tid)
 {
-    uint32_t absent = 0;
 #pragma unroll
     for (int e = 0; e < 8; ++e) {
-        const int row = rows[tile * T + 8 * wave + e];
-        const int64_t rr = row < 0 ? 0 : row;
-        absent |= (row < 0 ? 1u : 0u) << e;
+        const uint32_t row = (uint32_t)rows[tile * T + 8 * wave + e];
         if constexpr (QUANT)
-            r.nope[e] = *reinterpret_cast<const u32x2*>(a.kn + rr * a.kn_stride + lane * 8);
+            r.nope[e] = *reinterpret_cast<const u32x2*>(a.kn + (uint64_t)row * a.kn_stride + lane * 8);
         else
-            r.nope[e] = *reinterpret_cast<const u32x4*>(a.kn + rr * a.kn_stride + lane * 16);
+            r.nope[e] = *reinterpret_cast<const u32x4*>(a.kn + (uint64_t)row * a.kn_stride + lane * 16);
     }
-    {
-        const int row = rows[tile * T + (tid >> 3)];
-        const int64_t rr = row < 0 ? 0 : row;
-        absent |= (row < 0 ? 1u : 0u) << 8;
-        r.rope = *reinterpret_cast<const u32x4*>(a.kr + rr * a.kr_stride + (tid & 7) * 16);
-    }
-    r.absent = absent;
+    const uint32_t row = (uint32_t)rows[tile * T + (tid >> 3)];
+    r.rope = *reinterpret_cast<const u32x4*>(a.kr + (uint64_t)row * a.kr_stride + (tid & 7) * 16);
+    const uint32_t present = tmask[tile];
+    r.absent = ((~present >> (8 * wave)) & 0xffu) | (((~present >> (tid >> 3)) & 1u) << 8);
 }
 
-__device__ __forceinline__ float i8_at(uint32_t w, int k) { return (float)(int8_t)(w >> (8 * k)); }
+// int8 -> fp32 -> * scale with one conversion and one fma per element: byte k of w holds x + 128 (the caller
+// flips the sign bits), so x * s = fma(float(byte), s, -128 s); -128 s is exact, hence one rounding, the same
+// as rounding the product x * s.
+__device__ __forceinline__ float dq(uint32_t w, int k, float s, float neg128s)
+{
+    return __builtin_fmaf((float)((w >> (8 * k)) & 0xffu), s, neg128s);
+}
 
 // Dequantise rows [E0, E1) of this lane's 8 rows x 8 columns and store them into an LDS stage; with ROPE also
 // the lane's rope piece.
@@ -115,10 +124,13 @@ __device__ __forceinline__ void dequant_store(const RawTile<QUANT>& r, uint8_t* 
             uint32_t w0 = r.nope[e][0], w1 = r.nope[e][1];
             // keep the unpacking here: hoisted to the load, it would wait for the load right after issuing it
             asm volatile("" : "+v"(w0), "+v"(w1));
-            v[0] = pack_bf16x2(i8_at(w0, 0) * s, i8_at(w0, 1) * s);
-            v[1] = pack_bf16x2(i8_at(w0, 2) * s, i8_at(w0, 3) * s);
-            v[2] = pack_bf16x2(i8_at(w1, 0) * s, i8_at(w1, 1) * s);
-            v[3] = pack_bf16x2(i8_at(w1, 2) * s, i8_at(w1, 3) * s);
+            w0 ^= 0x80808080u;
+            w1 ^= 0x80808080u;
+            const float c = -128.f * s;
+            v[0] = pack_bf16x2(dq(w0, 0, s, c), dq(w0, 1, s, c));
+            v[1] = pack_bf16x2(dq(w0, 2, s, c), dq(w0, 3, s, c));
+            v[2] = pack_bf16x2(dq(w1, 0, s, c), dq(w1, 1, s, c));
+            v[3] = pack_bf16x2(dq(w1, 2, s, c), dq(w1, 3, s, c));
         } else {
             u32x4 w = r.nope[e];
             asm volatile("" : "+v"(w)); // as above: consume the load here, not where it was issued
@@ -140,8 +152,10 @@ __global__ __attribute__((amdgpu_flat_work_group_size(512, 512), amdgpu_waves_pe
     SfaArgs a)
 {
     extern __shared__ __align__(16) uint8_t smem[];
-    int* rows = reinterpret_cast<int*>(smem + ROWS_OFF);
-    float* scales = reinterpret_cast<float*>(smem + SCALES_OFF);
+    uint32_t* tmask = reinterpret_cast<uint32_t*>(smem + SPLIT_OFF);
+    int* rows = reinterpret_cast<int*>(smem + SPLIT_OFF + tmask_bytes(a.split_cap));
+    float* scales = reinterpret_cast<float*>(smem + SPLIT_OFF + tmask_bytes(a.split_cap) + a.split_cap * 4);
+    int* bt_lds = reinterpret_cast<int*>(smem + SPLIT_OFF + split_bytes(a.split_cap));
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int sp = blockIdx.x, tq = blockIdx.y, hz = blockIdx.z;
@@ -157,27 +171,47 @@ __global__ __attribute__((amdgpu_flat_work_group_size(512, 512), amdgpu_waves_pe
     const int ntiles = (ntiles_real + 1) & ~1;
     const int tok0 = tile0 * T;
 
-    // logical top-k entries of this split -> physical cache rows (or -1: absent), and their 4 dequant scales
+    // this sequence's page table -> LDS (saves one dependent global load per selected token)
+    const bool bt_cached = a.bt_cached != 0;
+    if (bt_cached)
+        for (int i = tid; i < a.bt_stride; i += 512) bt_lds[i] = a.block_table[(int64_t)bi * a.bt_stride + i];
+    // logical top-k entries of this split
     const int64_t max_logical = (int64_t)a.bt_stride * a.block_size;
-    for (int i = tid; i < ntiles * T; i += 512) {
-        const int g = tok0 + i;
+    int my_idx[MAX_SPLIT_TOKENS / 512];
+#pragma unroll
+    for (int j = 0; j < MAX_SPLIT_TOKENS / 512; ++j) {
+        const int i = tid + 512 * j, g = tok0 + i;
+        my_idx[j] = -1;
+        if (i < ntiles_real * T && g < cur) my_idx[j] = a.topk_idx[(int64_t)tq * a.topk_stride + g];
+    }
+    __syncthreads();
+    // -> physical cache rows (absent entries: row 0 and a cleared bit in the tile's validity word) and their
+    // 4 dequant scales (0 when absent)
+#pragma unroll
+    for (int j = 0; j < MAX_SPLIT_TOKENS / 512; ++j) {
+        const int i = tid + 512 * j;
+        if (i >= ntiles * T) break; // wave-uniform: tiles are 32 wide, waves 64
+        const int idx = my_idx[j];
         int row = -1;
-        if (g < cur && i < ntiles_real * T) { // the padding tile holds no token
-            const int idx = a.topk_idx[(int64_t)tq * a.topk_stride + g];
-            if (idx >= 0 && idx < max_logical) {
-                const int page = a.block_table[(int64_t)bi * a.bt_stride + idx / a.block_size];
-                const int64_t r = (int64_t)page * a.block_size + idx % a.block_size;
-                if (page >= 0 && r < a.n_rows) row = (int)r;
-            }
+        if (idx >= 0 && idx < max_logical) {
+            const int page = bt_cached ? bt_lds[idx / a.block_size]
+                                       : a.block_table[(int64_t)bi * a.bt_stride + idx / a.block_size];
+            const int64_t r = (int64_t)page * a.block_size + idx % a.block_size;
+            if (page >= 0 && r < a.n_rows) row = (int)r;
         }
-        rows[i] = row;
+        rows[i] = max(row, 0);
+        const uint64_t present = __ballot(row >= 0);
+        if (lane == 0) {
+            tmask[i >> 5] = (uint32_t)present;
+            tmask[(i >> 5) + 1] = (uint32_t)(present >> 32);
+        }
         if constexpr (QUANT) {
             f32x4 sc = {0.f, 0.f, 0.f, 0.f};
-            if (row >= 0) sc = *reinterpret_cast<const f32x4*>(a.ks + (int64_t)row * a.ks_stride);
+            if (row >= 0) sc = *reinterpret_cast<const f32x4*>(a.ks + (uint64_t)row * a.ks_stride);
             *reinterpret_cast<f32x4*>(scales + i * 4) = sc;
         }
     }
-    __syncthreads(); // rows[] / scales[] ready
+    __syncthreads(); // rows[] / scales[] / tmask[] ready
 
     // Both roles run the same barrier sequence: one before the first tile, then two per tile
     // (partial S exchanged; tile consumed and next tile stored).
@@ -189,32 +223,30 @@ __global__ __attribute__((amdgpu_flat_work_group_size(512, 512), amdgpu_waves_pe
         const int last = ntiles - 1;
         RawTile<QUANT> raw0, raw1;
         if (ntiles > 0) {
-            load_raw<QUANT>(raw0, a, rows, 0, pw, lane, ptid);
-            load_raw<QUANT>(raw1, a, rows, 1, pw, lane, ptid);
+            load_raw<QUANT>(raw0, a, rows, tmask, 0, pw, lane, ptid);
+            load_raw<QUANT>(raw1, a, rows, tmask, 1, pw, lane, ptid);
             dequant_store<QUANT, 0, 8, true>(raw0, smem, scales, 0, pw, lane, ptid);
-            load_raw<QUANT>(raw0, a, rows, min(2, last), pw, lane, ptid);
+            load_raw<QUANT>(raw0, a, rows, tmask, min(2, last), pw, lane, ptid);
         }
         __syncthreads();
         // Every step stores one tile and issues the loads of another, unconditionally (past the end the last
         // tile is loaded again and stored into a stage nobody reads): with a fixed number of loads in flight
         // on every path the wait for a tile leaves the younger tile's loads outstanding.
-        // The consumers spend about a third of a tile before their mid-tile barrier (half of S) and two thirds
-        // after it (softmax, PV); the store of the next tile is split the same way around that barrier.
+        // The store of the next tile is split around the consumers' mid-tile barrier: most of it runs beside the
+        // S MFMAs, the rest (and the loads of a later tile) beside softmax and PV.
         auto produce = [&](int it, RawTile<QUANT>& next) {
             uint8_t* dst = smem + ((it + 1) & 1) * STAGE;
-            dequant_store<QUANT, 0, 3, false>(next, dst, scales, min(it + 1, last), pw, lane, ptid);
+            dequant_store<QUANT, 0, 5, false>(next, dst, scales, min(it + 1, last), pw, lane, ptid);
             __syncthreads();
-            dequant_store<QUANT, 3, 8, true>(next, dst, scales, min(it + 1, last), pw, lane, ptid);
-            load_raw<QUANT>(next, a, rows, min(it + 3, last), pw, lane, ptid);
+            dequant_store<QUANT, 5, 8, true>(next, dst, scales, min(it + 1, last), pw, lane, ptid);
+            load_raw<QUANT>(next, a, rows, tmask, min(it + 3, last), pw, lane, ptid);
             __syncthreads();
         };
         for (int it = 0; it < ntiles; it += 2) {
             produce(it, raw1);
             produce(it + 1, raw0);
         }
-        return;
-    }
-
+    } else {
     // -------------------------------------------------------------------- consumer wavefronts
     const int l32 = lane & 31, hl = lane >> 5;
     const int hg = wave >> 1, kh = wave & 1; // head group of 32 within the workgroup; k-step / dim-block parity
@@ -225,15 +257,22 @@ __global__ __attribute__((amdgpu_flat_work_group_size(512, 512), amdgpu_waves_pe
     const int head = hz * HEADS_PER_WG + hg * 32 + l32;
     const bool head_ok = head < a.nq;
     const bool wave_active = hz * HEADS_PER_WG + hg * 32 < a.nq;
-    bf16x8 q[KSTEPS / 2];
+    // 12 k-steps stay in registers; the other 6 (4 nope, 2 rope) are parked in LDS and read back by the same lane
+    // every tile, which keeps the consumer inside its 256 registers.
+    bf16x8 q[NREG_KSTEPS];
+    uint8_t* qpark = smem + QPARK_OFF + wave * (NPARK * 1024) + lane * 16;
     {
         const int64_t qrow = (int64_t)tq * a.nq + (head_ok ? head : 0);
         const __bf16* qn = reinterpret_cast<const __bf16*>(a.q_nope) + qrow * DN + kh * 16 + hl * 8;
         const __bf16* qr = reinterpret_cast<const __bf16*>(a.q_rope) + qrow * DR + kh * 16 + hl * 8;
 #pragma unroll
-        for (int i = 0; i < DN / 32; ++i) q[i] = *reinterpret_cast<const bf16x8*>(qn + i * 32);
-#pragma unroll
-        for (int i = 0; i < DR / 32; ++i) q[DN / 32 + i] = *reinterpret_cast<const bf16x8*>(qr + i * 32);
+        for (int i = 0; i < KSTEPS / 2; ++i) {
+            const bf16x8 v = *reinterpret_cast<const bf16x8*>(i < DN / 32 ? qn + i * 32 : qr + (i - DN / 32) * 32);
+            if (i < NREG_KSTEPS)
+                q[i < NREG_KSTEPS ? i : 0] = v;
+            else
+                *reinterpret_cast<bf16x8*>(qpark + (i - NREG_KSTEPS) * 1024) = v;
+        }
     }
 
     f32x16 o[8]; // O^T blocks db = 2*i + kh: dims [32*db, 32*db + 32) x 32 heads
@@ -263,39 +302,51 @@ __global__ __attribute__((amdgpu_flat_work_group_size(512, 512), amdgpu_waves_pe
         v_off = (4 * hl + (jj >> 2)) * KROW + (jj & 1) * 8 + ((cl ^ sw) << 4);
     }
     uint8_t* xmine = smem + XBUF_OFF + wave * 4096 + lane * 16;
-    uint8_t* xpeer = smem + XBUF_OFF + (wave ^ 1) * 4096 + lane * 16;
 
     __syncthreads(); // tile 0 stored
 
     for (int it = 0; it < ntiles; ++it) {
         uint8_t* stage = smem + (it & 1) * STAGE;
-        const uint32_t valid = (uint32_t)__ballot(rows[it * T + l32] >= 0);
+        const uint32_t valid = tmask[it];
         // half of S^T[token, head] = K[token, :] . Q[head, :] (k-steps of parity kh)
-        f32x16 s;
+        f32x16 s, s2; // even / odd k-steps: two independent accumulation chains keep the matrix core busy
 #pragma unroll
-        for (int r = 0; r < 16; ++r) s[r] = 0.f;
+        for (int r = 0; r < 16; ++r) s[r] = s2[r] = 0.f;
         {
-            // operand reads run three k-steps ahead of the MFMAs that use them
-            constexpr int AHEAD = 3;
-            bf16x8 kf[KSTEPS / 2];
-#pragma unroll
-            for (int i = 0; i < AHEAD; ++i)
+            // operand reads run AHEAD k-steps ahead of the MFMAs that use them
+            constexpr int AHEAD = 2, N = KSTEPS / 2;
+            bf16x8 kf[N], qp[N];
+            auto fetch = [&](int i) {
                 kf[i] = *reinterpret_cast<const bf16x8*>(stage + s_off[i & 1] + (i >> 1) * 128);
+                if (i >= NREG_KSTEPS) qp[i] = *reinterpret_cast<const bf16x8*>(qpark + (i - NREG_KSTEPS) * 1024);
+            };
 #pragma unroll
-            for (int i = 0; i < KSTEPS / 2; ++i) {
-                if (i + AHEAD < KSTEPS / 2)
-                    kf[i + AHEAD] =
-                        *reinterpret_cast<const bf16x8*>(stage + s_off[(i + AHEAD) & 1] + ((i + AHEAD) >> 1) * 128);
-                s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf[i], q[i], s, 0, 0, 0);
+            for (int i = 0; i < AHEAD; ++i) fetch(i);
+#pragma unroll
+            for (int i = 0; i < N; ++i) {
+                if (i + AHEAD < N) fetch(i + AHEAD);
+                const bf16x8 qi = i < NREG_KSTEPS ? q[i < NREG_KSTEPS ? i : 0] : qp[i];
+                if (i & 1)
+                    s2 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf[i], qi, s2, 0, 0, 0);
+                else
+                    s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf[i], qi, s, 0, 0, 0);
             }
-            // issue order: AHEAD reads, then (MFMA, read) pairs, then the last MFMAs
+            // issue order: AHEAD fetches, then (MFMA, fetch) pairs, then the last MFMAs; a fetch is one LDS read
+            // for a k-step whose Q fragment is in registers and two for a parked one
             __builtin_amdgcn_sched_group_barrier(0x100, AHEAD, 0);
 #pragma unroll
-            for (int i = 0; i < KSTEPS / 2 - AHEAD; ++i) {
-                __builtin_amdgcn_sched_group_barrier(0x008, 1, 0); // one MFMA
-                __builtin_amdgcn_sched_group_barrier(0x100, 1, 0); // one LDS read
+            for (int i = 0; i < NREG_KSTEPS - AHEAD; ++i) {
+                __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+                __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+            }
+#pragma unroll
+            for (int i = NREG_KSTEPS - AHEAD; i < N - AHEAD; ++i) {
+                __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+                __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
             }
             __builtin_amdgcn_sched_group_barrier(0x008, AHEAD, 0);
+#pragma unroll
+            for (int r = 0; r < 16; ++r) s[r] += s2[r];
         }
 #pragma unroll
         for (int g = 0; g < 4; ++g)
@@ -303,28 +354,31 @@ __global__ __attribute__((amdgpu_flat_work_group_size(512, 512), amdgpu_waves_pe
         __syncthreads(); // partial S of both waves of each pair is in LDS
 #pragma unroll
         for (int g = 0; g < 4; ++g) {
-            const f32x4 p = *reinterpret_cast<const f32x4*>(xpeer + g * 1024);
+            const f32x4 p = *reinterpret_cast<const f32x4*>(xmine + (kh ? -4096 : 4096) + g * 1024);
             s[4 * g] += p[0];
             s[4 * g + 1] += p[1];
             s[4 * g + 2] += p[2];
             s[4 * g + 3] += p[3];
         }
         if (wave_active && valid != 0u) {
-            // register r holds token 8*(r/4) + 4*hl + r%4 for head l32
+            // register r holds token 8*(r/4) + 4*hl + r%4 for head l32; statistics on the raw scores
+            // (softmax_scale > 0 commutes with max), exponent argument by one fma per score
             float mx = -INFINITY;
 #pragma unroll
             for (int r = 0; r < 16; ++r) {
-                float z = s[r] * c_log2;
                 if (valid != 0xffffffffu) {
                     const int tok = 8 * (r >> 2) + 4 * hl + (r & 3);
-                    z = ((valid >> tok) & 1u) ? z : -INFINITY;
+                    s[r] = ((valid >> tok) & 1u) ? s[r] : -INFINITY;
                 }
-                s[r] = z;
-                mx = fmaxf(mx, z);
+                mx = fmaxf(mx, s[r]);
             }
-            mx = fmaxf(mx, __shfl_xor(mx, 32));
+            mx = fmaxf(mx, __shfl_xor(mx, 32)) * c_log2;
+            // The reference exponent only follows the running maximum when it has grown by more than 2^8: until
+            // then P~ = 2^(z - m_run) may exceed 1 (by at most 2^8, no issue for bf16 or the fp32 sums), which
+            // makes the rescale of the 128 accumulator registers a rare event.  Every P~, l and O stay relative to
+            // the same m_run, so the result is unchanged.
             const float m_new = fmaxf(m_run, mx);
-            if (__any(m_new > m_run)) {
+            if (__any(m_new > m_run + 8.f)) {
                 const float alpha = __builtin_amdgcn_exp2f(m_run - m_new); // 0 on the first tile (m_run = -inf)
                 l_run *= alpha;
 #pragma unroll
@@ -336,7 +390,8 @@ __global__ __attribute__((amdgpu_flat_work_group_size(512, 512), amdgpu_waves_pe
             uint32_t pb[8];
 #pragma unroll
             for (int r = 0; r < 16; r += 2) {
-                const float p0 = __builtin_amdgcn_exp2f(s[r] - m_run), p1 = __builtin_amdgcn_exp2f(s[r + 1] - m_run);
+                const float p0 = __builtin_amdgcn_exp2f(__builtin_fmaf(s[r], c_log2, -m_run));
+                const float p1 = __builtin_amdgcn_exp2f(__builtin_fmaf(s[r + 1], c_log2, -m_run));
                 l_run += p0 + p1;
                 pb[r >> 1] = pack_bf16x2(p0, p1);
             }
@@ -349,8 +404,8 @@ __global__ __attribute__((amdgpu_flat_work_group_size(512, 512), amdgpu_waves_pe
                     u32x4 pw = {pb[4 * j], pb[4 * j + 1], pb[4 * j + 2], pb[4 * j + 3]};
                     pf[j] = __builtin_bit_cast(bf16x8, pw);
                 }
-                // 16 MFMAs (j, i); their two transpose reads each run two MFMAs ahead
-                constexpr int AHEAD = 2;
+                // 16 MFMAs (j, i); their two transpose reads each run AHEAD MFMAs ahead
+                constexpr int AHEAD = 3;
                 s16x4 lo[16], hi[16];
                 auto vread = [&](int n) {
                     uint8_t* vp = stage + v_off + (16 * (n >> 3)) * KROW + (n & 7) * 128;
@@ -378,34 +433,43 @@ __global__ __attribute__((amdgpu_flat_work_group_size(512, 512), amdgpu_waves_pe
         __syncthreads(); // tile consumed: its stage and the exchange buffer may be overwritten
     }
 
-    if (!wave_active) return;
+    // Epilogue, part 1: O^T blocks -> LDS as [head][512] fp32 rows (the tile stages are free now), 16-byte
+    // chunks XOR-swizzled with the head so that the 8 lanes of a b128 write hit distinct banks.  Register r of
+    // o[i] holds dim 32*(2*i + kh) + 8*(r/4) + 4*hl + r%4 of head l32.
     const float l_tot = l_run + __shfl_xor(l_run, 32);
-    if (!head_ok) return;
-    // register r of o[i] holds dim 32*(2*i + kh) + 8*(r/4) + 4*hl + r%4 of head l32
-    if (a.nsplit == 1) {
-        const float inv = l_tot > 0.f ? 1.f / l_tot : 0.f;
-        uint8_t* dst = reinterpret_cast<uint8_t*>(a.out) + ((int64_t)tq * a.nq + head) * DN * 2;
+    const float mul = a.nsplit == 1 ? (l_tot > 0.f ? 1.f / l_tot : 0.f) : 1.f;
+    const int hrow = hg * 32 + l32;
+    uint8_t* orow = smem + hrow * OUT_ROW;
 #pragma unroll
-        for (int i = 0; i < 8; ++i)
+    for (int i = 0; i < 8; ++i)
 #pragma unroll
-            for (int g = 0; g < 4; ++g) {
-                u32x2 v = {pack_bf16x2(o[i][4 * g] * inv, o[i][4 * g + 1] * inv),
-                           pack_bf16x2(o[i][4 * g + 2] * inv, o[i][4 * g + 3] * inv)};
-                *reinterpret_cast<u32x2*>(dst + (32 * (2 * i + kh) + 8 * g + 4 * hl) * 2) = v;
-            }
-    } else {
+        for (int g = 0; g < 4; ++g) {
+            const int c = 8 * (2 * i + kh) + 2 * g + hl;
+            const f32x4 v = {o[i][4 * g] * mul, o[i][4 * g + 1] * mul, o[i][4 * g + 2] * mul, o[i][4 * g + 3] * mul};
+            *reinterpret_cast<f32x4*>(orow + ((c ^ (hrow & 7)) << 4)) = v;
+        }
+    if (a.nsplit > 1 && head_ok && hl == 0 && kh == 0) {
         const int64_t prow = ((int64_t)tq * a.nsplit + sp) * a.nq + head;
-        float* dst = a.part_o + prow * DN;
-#pragma unroll
-        for (int i = 0; i < 8; ++i)
-#pragma unroll
-            for (int g = 0; g < 4; ++g) {
-                f32x4 v = {o[i][4 * g], o[i][4 * g + 1], o[i][4 * g + 2], o[i][4 * g + 3]};
-                *reinterpret_cast<f32x4*>(dst + 32 * (2 * i + kh) + 8 * g + 4 * hl) = v;
-            }
-        if (hl == 0 && kh == 0) {
-            a.part_ml[prow * 2] = m_run;
-            a.part_ml[prow * 2 + 1] = l_tot;
+        a.part_ml[prow * 2] = m_run;
+        a.part_ml[prow * 2 + 1] = l_tot;
+    }
+    } // consumer
+    __syncthreads();
+
+    // Epilogue, part 2: all 512 lanes copy the 64 rows out, a wavefront writing 1 KB (fp32 partial) or 512 B
+    // (bf16 output) of one row per instruction.
+#pragma unroll 4
+    for (int id = tid; id < HEADS_PER_WG * (DN / 4); id += 512) {
+        const int hrow = id / (DN / 4), c = id % (DN / 4);
+        const int head = hz * HEADS_PER_WG + hrow;
+        if (head >= a.nq) continue;
+        const f32x4 v = *reinterpret_cast<const f32x4*>(smem + hrow * OUT_ROW + ((c ^ (hrow & 7)) << 4));
+        if (a.nsplit == 1) {
+            const u32x2 w = {pack_bf16x2(v[0], v[1]), pack_bf16x2(v[2], v[3])};
+            *reinterpret_cast<u32x2*>(reinterpret_cast<uint8_t*>(a.out) + (((int64_t)tq * a.nq + head) * DN + c * 4) * 2) = w;
+        } else {
+            const int64_t prow = ((int64_t)tq * a.nsplit + sp) * a.nq + head;
+            *reinterpret_cast<f32x4*>(a.part_o + prow * DN + c * 4) = v;
         }
     }
 }
@@ -487,11 +551,18 @@ hipError_t sfa_launch(const SfaArgs& a, hipStream_t stream)
                            static_cast<uint32_t*>(a.out), words);
         return hipGetLastError();
     }
+    SfaArgs args = a;
+    const int tiles = (a.topk + T - 1) / T;
+    args.split_cap = (((tiles + a.nsplit - 1) / a.nsplit + 1) & ~1) * T;
+    int smem_bytes = SPLIT_OFF + split_bytes(args.split_cap);
+    args.bt_cached = smem_bytes + a.bt_stride * 4 <= LDS_LIMIT ? 1 : 0;
+    if (args.bt_cached) smem_bytes += a.bt_stride * 4;
+    if (smem_bytes < HEADS_PER_WG * OUT_ROW) smem_bytes = HEADS_PER_WG * OUT_ROW; // epilogue staging
     static bool attr_done[2] = {false, false};
     auto kern = a.quant ? sfa_decode_kernel<true> : sfa_decode_kernel<false>;
     if (!attr_done[a.quant]) {
         hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
-                                           hipFuncAttributeMaxDynamicSharedMemorySize, SMEM_BYTES);
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, LDS_LIMIT);
         if (e != hipSuccess) return e;
         attr_done[a.quant] = true;
     }
@@ -499,7 +570,7 @@ hipError_t sfa_launch(const SfaArgs& a, hipStream_t stream)
     dim3 grid(a.nsplit, t, hgroups);
     {
         ScopedKernelTimer tm(KID_SFA_DECODE, stream);
-        hipLaunchKernelGGL(kern, grid, dim3(512), SMEM_BYTES, stream, a);
+        hipLaunchKernelGGL(kern, grid, dim3(512), smem_bytes, stream, args);
     }
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) return e;
