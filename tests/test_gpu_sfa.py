@@ -1,30 +1,36 @@
-"""GPU parity: sparse flash attention (HIP, through the C ABI) against the CPU oracle."""
+"""GPU parity: sparse flash attention (HIP, through the C ABI) against the CPU oracle.
+
+Bars.  BASELINE: every element within 1e-2 absolute + 2e-2 relative of the reference's golden (checked against
+both of its goldens, no-flash and flash).  The reference's own comparator (at most 0.5 % of elements outside
+1e-4 + 5e-3 relative) presumes the golden's rounding points for P; the kernel rounds P~ = exp(s - m) to bf16
+relative to its running maximum, as the reference's online-softmax golden does per tile, and the two goldens
+themselves disagree under that comparator where the softmax is peaked (about 18 % of elements on the benchmark
+distribution).  So instead of that comparator the tests require the kernel to be as close to float64 attention
+as the goldens are.
+"""
+import ctypes
+
 import pytest
 import torch
 
 from oracle import sfa as osfa
-from oracle.compare import compare, count_violations
+from oracle.compare import count_violations
 
 from _cases import run_sfa, sfa_golden
+from _fixtures import load_sfa_small
 
 pytestmark = pytest.mark.gpu
 
-# BASELINE bar: within 2e-2 relative / 1e-2 absolute in bf16 (no element may exceed it);
-# the reference's own bar: at most 0.5 % of elements outside 1e-4 + 5e-3 * |ref|.
 ABS_TOL, REL_TOL = 1e-2, 2e-2
 
 
-def check(out, gold, name, strict=True):
+def check(out, gold, name):
     assert not torch.isnan(out).any() and not torch.isinf(out).any(), name
+    assert out.shape == gold.shape and out.dtype == gold.dtype, name
     assert count_violations(out, gold, ABS_TOL, REL_TOL) == 0, name
-    if strict:
-        compare(out, gold, name, atol=1e-4, rtol=5e-3)
 
 
 def check_vs_fp64(out, case, golds, name):
-    """Where the softmax is peaked the reference's goldens differ from each other by bf16 rounding of P
-    (no-flash vs flash disagree on ~18 % of elements under the strict comparator), so the strict comparator
-    cannot hold against either; instead the kernel must be as close to float64 attention as they are."""
     ref = osfa.attention_fp64(case["q"], case["kn"], case["kr"], case["kn_scales"], case["topk_indices"],
                               case["block_table"], case["act_seq"], case["block_size"], case["softmax_scale"],
                               case["topk"])
@@ -36,33 +42,183 @@ def check_vs_fp64(out, case, golds, name):
     assert bad <= 1.5 * gold_bad + 0.005, f"{name}: {bad} of elements off vs golden's own {gold_bad}"
 
 
+def full_check(out, case, name):
+    g0, g1 = sfa_golden(case), sfa_golden(case, flash=True, s2_tile=512)
+    check(out, g0, name + " vs no-flash golden")
+    check(out, g1, name + " vs flash golden")
+    check_vs_fp64(out, case, [g0, g1], name)
+
+
 def test_tiny_config1(cuda):
-    # b=1, 16 heads, 4096-token cache, top-256, scale 1/sqrt(192)
+    # BASELINE config 1: b=1, 16 heads, 4096-token cache, top-256, scale 1/sqrt(192)
     case = osfa.make_case(1, 16, 1, [4096], topk=256, seed=7, dist="bench", softmax_scale=192 ** -0.5)
-    out = run_sfa(case, cuda)
-    g0, g1 = sfa_golden(case), sfa_golden(case, flash=True, s2_tile=64)
-    check(out, g0, "config1 vs no-flash golden", strict=False)
-    check(out, g1, "config1 vs flash golden", strict=False)
-    check_vs_fp64(out, case, [g0, g1], "config1")
+    full_check(run_sfa(case, cuda), case, "config1")
 
 
 def test_tiny_reference_distribution(cuda):
     # same shape on the reference generator's distribution (U[-1,1), scale 576^-0.5)
     case = osfa.make_case(1, 16, 1, [4096], topk=256, seed=11)
+    full_check(run_sfa(case, cuda), case, "config1-uniform")
+
+
+def test_golden_fixture(cuda):
+    case, expect = load_sfa_small()
     out = run_sfa(case, cuda)
-    g0, g1 = sfa_golden(case), sfa_golden(case, flash=True, s2_tile=64)
-    check(out, g0, "config1-uniform vs no-flash golden", strict=False)
-    check(out, g1, "config1-uniform vs flash golden", strict=False)
-    check_vs_fp64(out, case, [g0, g1], "config1-uniform")
+    check(out, expect["no_flash"], "fixture vs no-flash")
+    check(out, expect["flash64"], "fixture vs flash")
+    out_p = run_sfa(case, cuda, packed=True, entry="d_950")
+    assert torch.equal(out_p, out), "packed-row entry must equal the three-tensor entry bit for bit"
 
 
-@pytest.mark.parametrize("packed", [False, True])
-def test_reference_case_mixed_lengths(cuda, packed):
-    # the reference's decode test case: (b, nq, nkv, s1) = (4, 128, 1, 2), lengths 65536 / 16381 / 666 / 15
+@pytest.mark.parametrize("packed,entry", [(False, "d"), (True, "d"), (False, "d_950"), (True, "p")])
+def test_reference_case_mixed_lengths(cuda, packed, entry):
+    # the reference's decode case: (b, nq, nkv, s1) = (4, 128, 1, 2), lengths 65536 / 16381 / 666 / 15
     case = osfa.make_case(4, 128, 2, [65536, 16381, 666, 15], seed=42)
-    out = run_sfa(case, cuda, packed=packed)
-    g0 = sfa_golden(case)
-    check(out, g0, "mixed lengths vs no-flash golden", strict=False)
-    check_vs_fp64(out, case, [g0], "mixed lengths")
-    # sequences 2 and 3 are shorter than s1 + topk: rows past cur_seq must not matter, row (3, 0) has cur_seq 14
+    out = run_sfa(case, cuda, packed=packed, entry=entry)
     assert out.shape == (4, 2, 128, 512)
+    full_check(out, case, "mixed lengths")
+
+
+def test_bf16_cache(cuda):
+    # the reference's non-quantised flavour: key_nope_2d in bf16, scales unused
+    case = osfa.make_case(2, 128, 2, [3000, 300], topk=2048, seed=5, quant=False)
+    full_check(run_sfa(case, cuda), case, "bf16 cache")
+
+
+@pytest.mark.parametrize("nq", [16, 48, 64, 96, 128])
+def test_head_counts(cuda, nq):
+    case = osfa.make_case(2, nq, 1, [2500, 40], topk=512, seed=nq, dist="bench", softmax_scale=192 ** -0.5)
+    full_check(run_sfa(case, cuda), case, f"nq={nq}")
+
+
+def test_no_token_to_attend_gives_zeros(cuda):
+    # s1 = 2 with act_seq 1: token 0 has cur_seq 0 (row of zeros), token 1 attends to one entry; act_seq 0: both empty
+    case = osfa.make_case(2, 32, 2, [1, 0], topk=64, seed=3)
+    out = run_sfa(case, cuda)
+    assert (out[0, 0] == 0).all() and (out[1] == 0).all() and (out[0, 1] != 0).any()
+    check(out, sfa_golden(case), "cur_seq 0")
+
+
+def test_entries_past_cur_seq_are_never_read(cuda):
+    case = osfa.make_case(3, 64, 2, [700, 33, 2048], topk=1024, seed=8)
+    base = run_sfa(case, cuda)
+    tk = case["topk_indices"].clone()
+    for bi, act in enumerate(case["act_seq"]):
+        for si in range(2):
+            n = osfa.cur_seq_of(act, 2, si, 1024)
+            tk[bi * 2 + si, n:] = torch.tensor([-1, 2 ** 31 - 1, -(2 ** 31), 10 ** 6])[torch.arange(1024 - n) % 4]
+    poisoned = dict(case, topk_indices=tk)
+    assert torch.equal(run_sfa(poisoned, cuda), base)
+    full_check(base, case, "poison baseline")
+
+
+def test_absent_entries_inside_the_list_are_skipped(cuda):
+    # entries that cannot be resolved (-1, beyond the page table, unused page) take no part in the softmax:
+    # the result equals attention over the remaining entries
+    case = osfa.make_case(1, 32, 1, [600], topk=256, seed=9)
+    tk = case["topk_indices"].clone()
+    dead = [0, 5, 31, 32, 100, 255]
+    tk[0, dead] = torch.tensor([-1, 10 ** 6, -7, 640, 5 * 128, -1], dtype=torch.int32)  # 640, 5*128: past the table
+    out = run_sfa(dict(case, topk_indices=tk), cuda)
+    keep = [j for j in range(256) if j not in dead]
+    ref_case = dict(case, topk_indices=case["topk_indices"][:, keep].contiguous(), topk=len(keep))
+    ref_case["act_seq"] = [600]
+    full_check(out, ref_case, "absent entries")
+
+
+def test_forced_kv_splits_agree(cuda):
+    """Drives the C ABI directly: 1, 2, 4 and 16 KV splits of the same problem."""
+    from pypto_amd import _runtime
+    lib = _runtime.load_library()
+    case = osfa.make_case(2, 128, 1, [5000, 900], topk=2048, seed=12, dist="bench", softmax_scale=192 ** -0.5)
+    dev = cuda
+    q = case["q"]
+    ts = [q[..., :512].reshape(-1, 512).contiguous().to(dev), q[..., 512:].reshape(-1, 64).contiguous().to(dev),
+          case["kn"].to(dev), case["kr"].to(dev), case["kn_scales"].to(dev), case["topk_indices"].to(dev),
+          case["block_table"].to(dev), torch.tensor(case["act_seq"], dtype=torch.int32, device=dev)]
+    outs = []
+    for splits in (1, 2, 4, 16):
+        out = torch.zeros((2, 1, 128, 512), dtype=torch.bfloat16, device=dev)
+        d = _runtime.describe(ts + [out])
+        p = _runtime.SfaParams(128, 1, case["softmax_scale"], 2048, 128, case["block_table"].shape[1], splits)
+        n = lib.pto_sfa_quant_workspace(d, 9, ctypes.byref(p))
+        assert (n == 0) == (splits == 1)
+        ws = torch.empty(max(n, 1), dtype=torch.uint8, device=dev)
+        rc = lib.pto_sfa_quant_launch(d, 9, ctypes.byref(p), ws.data_ptr(), n, torch.cuda.current_stream().cuda_stream)
+        assert rc == 0, lib.pto_last_error()
+        torch.cuda.synchronize()
+        outs.append(out.cpu())
+    for o, splits in zip(outs, (1, 2, 4, 16)):
+        full_check(o, case, f"{splits} split(s)")
+        # splits differ only in where P~ is rounded to bf16 (relative to each split's own maximum)
+        assert count_violations(o, outs[0], 2e-3, 2.0 ** -5) == 0
+
+
+def test_full_size_config5(cuda):
+    # BASELINE config 5: b=32, 128 heads, context lengths U[16384, 65536], top-2048, bench distribution
+    g = torch.Generator().manual_seed(55)
+    act = torch.randint(16384, 65537, (32,), generator=g).tolist()
+    case = osfa.make_case(32, 128, 1, act, topk=2048, seed=55, dist="bench", softmax_scale=192 ** -0.5)
+    out = run_sfa(case, cuda)
+    full_check(out, case, "config5")
+
+
+def test_full_size_config5_mtp(cuda):
+    # the MTP variant: two query tokens per sequence (batch 8 keeps the CPU oracle within seconds)
+    g = torch.Generator().manual_seed(56)
+    act = torch.randint(16384, 65537, (8,), generator=g).tolist()
+    case = osfa.make_case(8, 128, 2, act, topk=2048, seed=56, dist="bench", softmax_scale=192 ** -0.5)
+    full_check(run_sfa(case, cuda, packed=True, entry="d_950"), case, "config5 mtp")
+
+
+def test_bad_calls_raise_before_launch(cuda):
+    from pypto_amd.deepseek_v32_exp import sparse_flash_attention_quant_impl as impl
+    from pypto_amd.error import FeError
+    case = osfa.make_case(1, 16, 1, [300], topk=64, seed=1)
+    dev = cuda
+    q = case["q"]
+    ts = [q[..., :512].reshape(-1, 512).contiguous().to(dev), q[..., 512:].reshape(-1, 64).contiguous().to(dev),
+          case["kn"].to(dev), case["kr"].to(dev), case["kn_scales"].to(dev), case["topk_indices"].to(dev),
+          case["block_table"].to(dev), torch.tensor(case["act_seq"], dtype=torch.int32, device=dev),
+          torch.zeros((1, 1, 16, 512), dtype=torch.bfloat16, device=dev)]
+    ok = (16, 1, 0.1, 64, 128, case["block_table"].shape[1], impl.SaTileShapeConfig())
+    impl.sparse_flash_attention_quant_d(*ts, *ok)
+    with pytest.raises(FeError, match="ValueError"):
+        impl.sparse_flash_attention_quant_d(*(ts[:5] + [ts[5].long()] + ts[6:]), *ok)  # int64 indices
+    with pytest.raises(FeError, match="topk must be in"):
+        impl.sparse_flash_attention_quant_d(*ts, 16, 1, 0.1, 4096, 128, ok[5], ok[6])
+    with pytest.raises(FeError, match="same device"):
+        impl.sparse_flash_attention_quant_d(*(ts[:7] + [ts[7].cpu()] + ts[8:]), *ok)
+    with pytest.raises(FeError, match="contiguous"):
+        impl.sparse_flash_attention_quant_d(*(ts[:3] + [ts[3].t().contiguous().t()] + ts[4:]), *ok)
+
+
+def test_graph_capture_and_replay(cuda):
+    """The launch path allocates only through the torch allocator and never synchronises, so it can be captured;
+    every replay must reproduce the eager result."""
+    case = osfa.make_case(2, 128, 1, [4000, 700], topk=2048, seed=21)
+    from pypto_amd.deepseek_v32_exp import sparse_flash_attention_quant_impl as impl
+    dev = cuda
+    q = case["q"]
+    ts = [q[..., :512].reshape(-1, 512).contiguous().to(dev), q[..., 512:].reshape(-1, 64).contiguous().to(dev),
+          case["kn"].to(dev), case["kr"].to(dev), case["kn_scales"].to(dev), case["topk_indices"].to(dev),
+          case["block_table"].to(dev), torch.tensor(case["act_seq"], dtype=torch.int32, device=dev)]
+    args = (128, 1, case["softmax_scale"], 2048, 128, case["block_table"].shape[1], impl.SaTileShapeConfig())
+    eager = torch.zeros((2, 1, 128, 512), dtype=torch.bfloat16, device=dev)
+    impl.sparse_flash_attention_quant_d(*ts, eager, *args)
+    torch.cuda.synchronize()
+    out = torch.zeros_like(eager)
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        impl.sparse_flash_attention_quant_d(*ts, out, *args)  # warm-up on the capture stream
+    torch.cuda.current_stream().wait_stream(side)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        impl.sparse_flash_attention_quant_d(*ts, out, *args)
+    for _ in range(3):
+        out.zero_()
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(out, eager)
