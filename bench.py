@@ -25,6 +25,17 @@ sys.path.insert(0, ROOT)
 HBM_PEAK_GBS = 8000.0
 MFMA_BF16_PEAK_TFLOPS = 2500.0
 
+# HBM bytes per launch (read + written) from rocprofv3 FETCH_SIZE x 2.000 and WRITE_SIZE x 1.000, the factors being what
+# the same counters read for a 256 MiB-in / 256 MiB-out elementwise kernel (--calibrate-copy); measured on the default
+# workload only (batch 32, s1 1, ctx 65536, three cache tensors) and reported for that workload only.
+MEASURED_TRAFFIC_BYTES = {
+    "indexer_score_kernel": 275.4e6 + 9.0e6,
+    "sfa_decode_kernel": 70.6e6 + 34.5e6,
+    "sfa_combine_kernel": 35.7e6 + 4.2e6,
+    "indexer_select_kernel": 10.6e6 + 0.3e6,
+    "indexer_topk_kernel": 0.8e6 + 0.3e6,
+}
+
 
 def parse():
     ap = argparse.ArgumentParser()
@@ -176,8 +187,12 @@ def main():
                            "peak": k["peak"], "unit": k["unit"], "frac": round(achieved / k["peak"], 4)})
     per_kernel.sort(key=lambda r: -r["us"])
     dom = per_kernel[0]
+    default_workload = (b, ctx, s1, args.packed) == (32, 65536, 1, False)
     roofline = {"kernel": dom["kernel"], "bound": dom["bound"], "achieved": dom["achieved"], "peak": dom["peak"],
-                "unit": dom["unit"], "frac": dom["frac"], "traffic": None, "us_per_launch": dom["us"]}
+                "unit": dom["unit"], "frac": dom["frac"],
+                "traffic": MEASURED_TRAFFIC_BYTES.get(dom["kernel"]) if default_workload else None,
+                "traffic_unit": "bytes per launch (rocprofv3 FETCH_SIZE + WRITE_SIZE, calibrated)",
+                "work_per_launch": info[dom["kernel"]]["work"], "us_per_launch": dom["us"]}
     sfa_row = next((r for r in per_kernel if r["kernel"] == "sfa_decode_kernel"), None)
     if sfa_row:
         sfa_row["hbm_gbs"] = round(sfa_bytes / sfa_row["us"] / 1e3, 1)
