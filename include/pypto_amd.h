@@ -119,6 +119,34 @@ uint64_t pto_lightning_indexer_workspace(const PtoTensorDesc* tensors, uint32_t 
 int pto_lightning_indexer_launch(const PtoTensorDesc* tensors, uint32_t n_tensors, const PtoIndexerParams* params,
                                  void* workspace, uint64_t workspace_bytes, void* hip_stream);
 
+/* Scalar arguments of select_experts (models/glm_v4_5/glm_select_experts.py:317-330: top_k, renormalize, topk_group,
+ * num_expert_group).  routed_scaling_factor and fill_neg_inf come from the reference's generalised gating golden
+ * (python/tests/ut/interpreter/_ops/moe_gating_topk.py:272,285): the weights are multiplied by the factor, and the experts
+ * of unselected groups are filled with -inf instead of the GLM kernel's 0.0 (glm_select_experts.py:169). */
+typedef struct {
+    int32_t top_k;
+    int32_t renormalize;
+    int32_t topk_group;
+    int32_t num_expert_group;
+    float routed_scaling_factor;
+    int32_t fill_neg_inf;
+} PtoSelectExpertsParams;
+
+/*
+ * select_experts (models/glm_v4_5/glm_select_experts.py:316-364; kernel :193-228).
+ * tensors[4], in order:
+ *   0 router_logits            [T, ne]    FP32 (the reference's dtype) or BF16; ne <= 256
+ *   1 e_score_correction_bias  [ne]       BF16 (the reference's dtype) or FP32
+ *   2 topk_weights             [T, top_k] FP32  (output)
+ *   3 topk_ids                 [T, top_k] INT32 (output; descending biased score, equal scores by ascending id)
+ * Inputs must be finite.  Needs no workspace (the query returns 0 for valid and for invalid arguments alike; use the
+ * launch's status).
+ */
+uint64_t pto_select_experts_workspace(const PtoTensorDesc* tensors, uint32_t n_tensors,
+                                      const PtoSelectExpertsParams* params);
+int pto_select_experts_launch(const PtoTensorDesc* tensors, uint32_t n_tensors, const PtoSelectExpertsParams* params,
+                              void* workspace, uint64_t workspace_bytes, void* hip_stream);
+
 /* Message of the calling thread's most recent failed call ("" if none).  Replaces the message strings
  * the reference's binding layer returns (python/src/bindings/runtime.cpp:270-335). */
 const char* pto_last_error(void);
@@ -129,7 +157,7 @@ const char* pto_last_error(void);
  * is bracketed by a HIP event pair recorded on the launch stream; pto_kernel_timing_read waits for the
  * events recorded so far for one kernel, returns their summed duration and count, and forgets them.
  * Kernel ids: 0 indexer_score_kernel, 1 indexer_topk_kernel, 2 sfa_decode_kernel, 3 sfa_combine_kernel,
- * 4 indexer_select_kernel.
+ * 4 indexer_select_kernel, 5 select_experts_kernel.
  * Off by default; not for use under graph capture.
  */
 int pto_kernel_timing_enable(int on);

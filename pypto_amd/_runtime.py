@@ -36,6 +36,12 @@ class IndexerParams(ctypes.Structure):
     _fields_ = [("selected_count", ctypes.c_int32)]
 
 
+class SelectExpertsParams(ctypes.Structure):
+    _fields_ = [("top_k", ctypes.c_int32), ("renormalize", ctypes.c_int32), ("topk_group", ctypes.c_int32),
+                ("num_expert_group", ctypes.c_int32), ("routed_scaling_factor", ctypes.c_float),
+                ("fill_neg_inf", ctypes.c_int32)]
+
+
 # framework/include/tilefwk/data_type.h:33-65
 _DTYPE_CODE = {torch.int8: 1, torch.int32: 3, torch.float16: 6, torch.float32: 7, torch.bfloat16: 8}
 
@@ -43,6 +49,7 @@ _OPS = {
     "sfa_quant": SfaParams,
     "sfa_antiquant": SfaParams,
     "lightning_indexer": IndexerParams,
+    "select_experts": SelectExpertsParams,
 }
 
 # C status -> Python exception type wrapped by FeError

@@ -256,9 +256,63 @@ int plan_indexer(const PtoTensorDesc* ts, uint32_t n, const PtoIndexerParams* p,
     return PTO_OK;
 }
 
+int plan_select_experts(const PtoTensorDesc* ts, uint32_t n, const PtoSelectExpertsParams* p, pto::SelectExpertsArgs* a)
+{
+    const char* op = "select_experts";
+    if (ts == nullptr || n != 4) return fail(PTO_ERR_ARG_COUNT, "%s: expected 4 tensors, got %u", op, n);
+    if (p == nullptr) return fail(PTO_ERR_PARAM, "%s: params is null", op);
+    if (ts[0].dataType != PTO_DT_FP32 && ts[0].dataType != PTO_DT_BF16)
+        return fail(PTO_ERR_DTYPE, "%s: router_logits must be fp32 or bf16, got %s", op, dtype_name(ts[0].dataType));
+    if (ts[1].dataType != PTO_DT_BF16 && ts[1].dataType != PTO_DT_FP32)
+        return fail(PTO_ERR_DTYPE, "%s: e_score_correction_bias must be bf16 or fp32, got %s", op, dtype_name(ts[1].dataType));
+    int rc;
+    if ((rc = check_tensor(op, ts[0], "router_logits", ts[0].dataType, 2))) return rc;
+    if ((rc = check_tensor(op, ts[1], "e_score_correction_bias", ts[1].dataType, 1))) return rc;
+    if ((rc = check_tensor(op, ts[2], "topk_weights", PTO_DT_FP32, 2))) return rc;
+    if ((rc = check_tensor(op, ts[3], "topk_ids", PTO_DT_INT32, 2))) return rc;
+    const int64_t t = ts[0].shape[0], ne = ts[0].shape[1];
+    if (ts[1].shape[0] != ne) return fail(PTO_ERR_SHAPE, "%s: bias has %lld entries, router_logits has %lld experts", op, (long long)ts[1].shape[0], (long long)ne);
+    if (ts[2].shape[0] != t || ts[3].shape[0] != t || ts[2].shape[1] != p->top_k || ts[3].shape[1] != p->top_k)
+        return fail(PTO_ERR_SHAPE, "%s: topk_weights and topk_ids must be [%lld, %d]", op, (long long)t, p->top_k);
+    if (ne > 0x7fffffff || !pto::select_experts_supported((int)ne, p->num_expert_group, p->top_k))
+        return fail(PTO_ERR_PARAM, "%s: need 1 <= experts <= 256, 1 <= groups <= 64 dividing the experts, 1 <= top_k <= min(32, experts); got experts %lld, groups %d, top_k %d",
+                    op, (long long)ne, p->num_expert_group, p->top_k);
+    if (p->topk_group < 1 || p->topk_group > p->num_expert_group)
+        return fail(PTO_ERR_PARAM, "%s: topk_group must be in [1, num_expert_group], got %d", op, p->topk_group);
+    if (!(p->routed_scaling_factor == p->routed_scaling_factor)) return fail(PTO_ERR_PARAM, "%s: routed_scaling_factor is NaN", op);
+    a->logits = ts[0].addr;
+    a->bias = ts[1].addr;
+    a->topk_weights = static_cast<float*>(ts[2].addr);
+    a->topk_ids = static_cast<int32_t*>(ts[3].addr);
+    a->t = t;
+    a->ne = (int32_t)ne;
+    a->top_k = p->top_k;
+    a->topk_group = p->topk_group;
+    a->n_group = p->num_expert_group;
+    a->routed_scaling_factor = p->routed_scaling_factor;
+    a->renormalize = p->renormalize != 0;
+    a->fill_neg_inf = p->fill_neg_inf != 0;
+    a->logits_bf16 = ts[0].dataType == PTO_DT_BF16;
+    a->bias_bf16 = ts[1].dataType == PTO_DT_BF16;
+    return PTO_OK;
+}
+
 } // namespace
 
 extern "C" {
+
+uint64_t pto_select_experts_workspace(const PtoTensorDesc*, uint32_t, const PtoSelectExpertsParams*) { return 0; }
+
+int pto_select_experts_launch(const PtoTensorDesc* tensors, uint32_t n_tensors, const PtoSelectExpertsParams* params,
+                              void*, uint64_t, void* hip_stream)
+{
+    pto::SelectExpertsArgs a;
+    int rc = plan_select_experts(tensors, n_tensors, params, &a);
+    if (rc) return rc;
+    hipError_t e = pto::select_experts_launch(a, static_cast<hipStream_t>(hip_stream));
+    if (e != hipSuccess) return fail(PTO_ERR_HIP, "select_experts: HIP launch failed: %s", hipGetErrorString(e));
+    return PTO_OK;
+}
 
 uint64_t pto_sfa_quant_workspace(const PtoTensorDesc* tensors, uint32_t n_tensors, const PtoSfaParams* params)
 {
@@ -331,7 +385,7 @@ int pto_kernel_timing_read(int kernel_id, double* total_ms, uint64_t* launches)
 const char* pto_kernel_name(int kernel_id)
 {
     static const char* names[] = {"indexer_score_kernel", "indexer_topk_kernel", "sfa_decode_kernel",
-                                  "sfa_combine_kernel", "indexer_select_kernel"};
+                                  "sfa_combine_kernel", "indexer_select_kernel", "select_experts_kernel"};
     return kernel_id >= 0 && kernel_id < pto::KID_COUNT ? names[kernel_id] : "";
 }
 

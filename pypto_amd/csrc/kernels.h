@@ -56,4 +56,19 @@ uint64_t indexer_workspace_bytes(int t, int score_stride);
 void indexer_bind_workspace(IndexerArgs& a, void* workspace);
 hipError_t indexer_launch(const IndexerArgs& a, hipStream_t stream);
 
+// ---------------------------------------------------------------- grouped expert selection
+struct SelectExpertsArgs {
+    const void* logits; // [t, ne] fp32 or bf16
+    const void* bias;   // [ne] bf16 or fp32
+    float* topk_weights; // [t, top_k]
+    int32_t* topk_ids;   // [t, top_k]
+    int64_t t;
+    int32_t ne, top_k, topk_group, n_group;
+    float routed_scaling_factor;
+    bool renormalize, fill_neg_inf, logits_bf16, bias_bf16;
+};
+
+bool select_experts_supported(int ne, int n_group, int top_k);
+hipError_t select_experts_launch(const SelectExpertsArgs& a, hipStream_t stream);
+
 } // namespace pto

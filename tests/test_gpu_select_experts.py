@@ -1,0 +1,109 @@
+"""GPU parity: grouped expert selection (HIP, through the C ABI) against the CPU oracle.
+
+Bar: expert ids bit-exact; the one licence is that two experts whose biased scores differ by at most 2 fp32 ulps may
+swap (the golden's sigmoid is torch's CPU vector routine, the kernel's is the correctly rounded value; they can differ
+in the last bit).  Weights within 1e-6 relative.
+"""
+import pytest
+import torch
+
+from oracle import select_experts as ose
+
+pytestmark = pytest.mark.gpu
+
+
+def run(logits, bias, top_k, renorm, topk_group, n_group, dev, **kw):
+    from pypto_amd.glm_v4_5.glm_select_experts import select_experts
+    t = logits.shape[0]
+    w = torch.full((t, top_k), -1.0, dtype=torch.float32, device=dev)
+    ids = torch.full((t, top_k), -1, dtype=torch.int32, device=dev)
+    select_experts(logits.to(dev), top_k, renorm, topk_group, n_group, bias.to(dev), w, ids, **kw)
+    torch.cuda.synchronize()
+    return w.cpu(), ids.cpu()
+
+
+def check(logits, bias, top_k, renorm, topk_group, n_group, dev, scale=1.0, neg=False):
+    w, ids = run(logits, bias, top_k, renorm, topk_group, n_group, dev, routed_scaling_factor=scale, fill_neg_inf=neg)
+    gw, gids = ose.select_experts(logits, top_k, renorm, topk_group, n_group, bias, scale, neg)
+    x = ose.biased_scores(logits, bias)
+    bad_rows = (ids != gids).any(dim=-1).nonzero().flatten().tolist()
+    for r in bad_rows:
+        for j in (ids[r] != gids[r]).nonzero().flatten().tolist():
+            a, e = int(ids[r, j]), int(gids[r, j])
+            assert abs(float(x[r, a]) - float(x[r, e])) <= 3e-7 * max(abs(float(x[r, e])), 1e-3), (r, j, a, e)
+    assert len(bad_rows) <= max(1, logits.shape[0] // 1000)
+    same = (ids == gids).all(dim=-1)
+    assert torch.allclose(w[same], gw[same], rtol=1e-6, atol=1e-9)
+    return len(bad_rows)
+
+
+def test_reference_test_shapes(cuda):
+    # the reference's own test: 32 and 1026 tokens, 160 experts, one group, top-8, renormalised, U[0,1) inputs
+    for t in (32, 1026):
+        logits, bias = ose.make_case(t, 160, 0, dist="uniform")
+        check(logits, bias, 8, True, 1, 1, cuda)
+
+
+def test_config2_grouped(cuda):
+    # BASELINE's expert-selector configuration: 8192 tokens x 160 experts, bf16 logits, fp32 bias, 8 groups, top-4
+    # groups, top-8 experts, renormalised, x 2.5
+    logits, bias = ose.make_case(8192, 160, 2, logits_dtype=torch.bfloat16, bias_dtype=torch.float32)
+    check(logits, bias, 8, True, 4, 8, cuda, scale=2.5, neg=True)
+    check(logits, bias, 8, True, 4, 8, cuda, scale=2.5, neg=False)
+
+
+def test_dtypes_sizes_and_flags(cuda):
+    for seed, (t, ne, ng, tg, k, renorm) in enumerate([(5, 256, 64, 7, 32, False), (1, 1, 1, 1, 1, True),
+                                                        (300, 96, 3, 2, 6, True), (17, 64, 4, 4, 5, False)]):
+        for ld, bd in ((torch.float32, torch.bfloat16), (torch.bfloat16, torch.bfloat16), (torch.float32, torch.float32)):
+            logits, bias = ose.make_case(t, ne, 40 + seed, logits_dtype=ld, bias_dtype=bd)
+            check(logits, bias, k, renorm, tg, ng, cuda, scale=1.5, neg=bool(seed % 2))
+
+
+def test_exact_ties(cuda):
+    logits = torch.zeros((3, 160))
+    bias = torch.zeros(160, dtype=torch.bfloat16)
+    w, ids = run(logits, bias, 8, True, 4, 8, cuda)
+    assert ids.tolist() == [list(range(8))] * 3
+    assert torch.allclose(w, torch.full((3, 8), 0.125))
+    logits[:, 100:108] = 1.0   # a tie among eight better experts of one group
+    _, ids = run(logits, bias, 8, True, 1, 8, cuda)
+    assert ids.tolist() == [list(range(100, 108))] * 3
+
+
+def test_empty_and_errors(cuda):
+    from pypto_amd.error import FeError
+    logits, bias = ose.make_case(0, 160, 1)
+    w, ids = run(logits, bias, 8, True, 1, 1, cuda)
+    assert w.shape == (0, 8) and ids.shape == (0, 8)
+    logits, bias = ose.make_case(4, 160, 1)
+    with pytest.raises(FeError, match="topk_group"):
+        run(logits, bias, 8, True, 9, 8, cuda)
+    with pytest.raises(FeError, match="groups"):
+        run(logits, bias, 8, True, 1, 7, cuda)
+    with pytest.raises(AssertionError):
+        run(logits.double(), bias, 8, True, 1, 1, cuda)
+
+
+def test_graph_capture_and_replay(cuda):
+    from pypto_amd.glm_v4_5.glm_select_experts import select_experts
+    logits, bias = ose.make_case(512, 160, 9)
+    ew, eids = run(logits, bias, 8, True, 4, 8, cuda)
+    dl, db = logits.to(cuda), bias.to(cuda)
+    w = torch.zeros((512, 8), dtype=torch.float32, device=cuda)
+    ids = torch.zeros((512, 8), dtype=torch.int32, device=cuda)
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        select_experts(dl, 8, True, 4, 8, db, w, ids)
+    torch.cuda.current_stream().wait_stream(side)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        select_experts(dl, 8, True, 4, 8, db, w, ids)
+    for _ in range(3):
+        w.zero_()
+        ids.zero_()
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(ids.cpu(), eids) and torch.equal(w.cpu(), ew)
