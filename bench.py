@@ -157,7 +157,9 @@ def main():
     lib.pto_kernel_timing_enable(0)
     lib.pto_kernel_name.restype = ctypes.c_char_p
     kernels = {}
-    for kid in range(5):
+    for kid in range(64):
+        if not lib.pto_kernel_name(kid):
+            break
         ms, n = ctypes.c_double(0), ctypes.c_uint64(0)
         lib.pto_kernel_timing_read(kid, ctypes.byref(ms), ctypes.byref(n))
         if n.value:

@@ -147,6 +147,29 @@ uint64_t pto_select_experts_workspace(const PtoTensorDesc* tensors, uint32_t n_t
 int pto_select_experts_launch(const PtoTensorDesc* tensors, uint32_t n_tensors, const PtoSelectExpertsParams* params,
                               void* workspace, uint64_t workspace_bytes, void* hip_stream);
 
+/* Scalar arguments of the GLM-4.5 paged decode attention (models/glm_v4_5/glm_attention.py:1585-1594: softmax_scale; the
+ * trailing tile_config holds Ascend tiling knobs and has no counterpart here). */
+typedef struct {
+    float softmax_scale;
+    int32_t kv_chunk; /* 0 = choose; >0 forces the number of cached tokens one workgroup walks (rounded up to 128) */
+} PtoGqaParams;
+
+/*
+ * attention / attention_for_950 / attention_for_950_high_through / attention_for_910_high_performance /
+ * attention_for_910_s1_range_high_performance (models/glm_v4_5/glm_attention.py:1584-1700; kernel :427-568).
+ * tensors[6], in order:
+ *   0 query        [t, nq, 128]                    BF16 (t = b * s1; rotary embedding already applied)
+ *   1 key_cache    [blocks, block_size, nkv, 128]  BF16 (block_size a multiple of 32; nq a multiple of nkv)
+ *   2 value_cache  [blocks, block_size, nkv, 128]  BF16
+ *   3 block_tables [b, max_blocks]                 INT32 (-1 = unused)
+ *   4 actual_seqs  [b]                             INT32
+ *   5 attn_res     [t, nq, 128]                    BF16 (output; query token j of a sequence attends to the first
+ *                                                  actual_seq - (s1 - 1 - j) cached tokens, zeros if that is <= 0)
+ */
+uint64_t pto_gqa_decode_workspace(const PtoTensorDesc* tensors, uint32_t n_tensors, const PtoGqaParams* params);
+int pto_gqa_decode_launch(const PtoTensorDesc* tensors, uint32_t n_tensors, const PtoGqaParams* params, void* workspace,
+                          uint64_t workspace_bytes, void* hip_stream);
+
 /* Message of the calling thread's most recent failed call ("" if none).  Replaces the message strings
  * the reference's binding layer returns (python/src/bindings/runtime.cpp:270-335). */
 const char* pto_last_error(void);
@@ -157,7 +180,8 @@ const char* pto_last_error(void);
  * is bracketed by a HIP event pair recorded on the launch stream; pto_kernel_timing_read waits for the
  * events recorded so far for one kernel, returns their summed duration and count, and forgets them.
  * Kernel ids: 0 indexer_score_kernel, 1 indexer_topk_kernel, 2 sfa_decode_kernel, 3 sfa_combine_kernel,
- * 4 indexer_select_kernel, 5 select_experts_kernel.
+ * 4 indexer_select_kernel, 5 select_experts_kernel, 6 gqa_decode_kernel, 7 gqa_combine_kernel
+ * (pto_kernel_name returns "" past the last id).
  * Off by default; not for use under graph capture.
  */
 int pto_kernel_timing_enable(int on);

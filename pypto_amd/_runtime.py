@@ -45,11 +45,16 @@ class SelectExpertsParams(ctypes.Structure):
 # framework/include/tilefwk/data_type.h:33-65
 _DTYPE_CODE = {torch.int8: 1, torch.int32: 3, torch.float16: 6, torch.float32: 7, torch.bfloat16: 8}
 
+class GqaParams(ctypes.Structure):
+    _fields_ = [("softmax_scale", ctypes.c_float), ("kv_chunk", ctypes.c_int32)]
+
+
 _OPS = {
     "sfa_quant": SfaParams,
     "sfa_antiquant": SfaParams,
     "lightning_indexer": IndexerParams,
     "select_experts": SelectExpertsParams,
+    "gqa_decode": GqaParams,
 }
 
 # C status -> Python exception type wrapped by FeError

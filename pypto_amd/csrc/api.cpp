@@ -297,9 +297,94 @@ int plan_select_experts(const PtoTensorDesc* ts, uint32_t n, const PtoSelectExpe
     return PTO_OK;
 }
 
+struct GqaPlan {
+    pto::GqaArgs args;
+    uint64_t ws_bytes;
+};
+
+int plan_gqa(const PtoTensorDesc* ts, uint32_t n, const PtoGqaParams* p, GqaPlan* plan)
+{
+    const char* op = "attention";
+    if (ts == nullptr || n != 6) return fail(PTO_ERR_ARG_COUNT, "%s: expected 6 tensors, got %u", op, n);
+    if (p == nullptr) return fail(PTO_ERR_PARAM, "%s: params is null", op);
+    int rc;
+    if ((rc = check_tensor(op, ts[0], "query", PTO_DT_BF16, 3))) return rc;
+    if ((rc = check_tensor(op, ts[1], "key_cache", PTO_DT_BF16, 4))) return rc;
+    if ((rc = check_tensor(op, ts[2], "value_cache", PTO_DT_BF16, 4))) return rc;
+    if ((rc = check_tensor(op, ts[3], "block_tables", PTO_DT_INT32, 2))) return rc;
+    if ((rc = check_tensor(op, ts[4], "actual_seqs", PTO_DT_INT32, 1))) return rc;
+    if ((rc = check_tensor(op, ts[5], "attn_res", PTO_DT_BF16, 3))) return rc;
+    if (!(p->softmax_scale == p->softmax_scale)) return fail(PTO_ERR_PARAM, "%s: softmax_scale is NaN", op);
+    if (p->kv_chunk < 0 || p->kv_chunk > (1 << 20)) return fail(PTO_ERR_PARAM, "%s: kv_chunk must be in [0, 2^20]", op);
+    const int64_t t = ts[0].shape[0], nq = ts[0].shape[1], d = ts[0].shape[2];
+    const int64_t blocks = ts[1].shape[0], bs = ts[1].shape[1], nkv = ts[1].shape[2];
+    const int64_t b = ts[4].shape[0];
+    if (d != 128 || ts[1].shape[3] != 128) return fail(PTO_ERR_SHAPE, "%s: head dim must be 128", op);
+    for (int i = 0; i < 4; ++i)
+        if (ts[2].shape[i] != ts[1].shape[i]) return fail(PTO_ERR_SHAPE, "%s: key_cache and value_cache shapes differ", op);
+    for (int i = 0; i < 3; ++i)
+        if (ts[5].shape[i] != ts[0].shape[i]) return fail(PTO_ERR_SHAPE, "%s: attn_res and query shapes differ", op);
+    if (bs <= 0 || bs % 32 != 0) return fail(PTO_ERR_SHAPE, "%s: block_size must be a positive multiple of 32, got %lld", op, (long long)bs);
+    if (nkv <= 0 || nq <= 0 || nq % nkv != 0) return fail(PTO_ERR_SHAPE, "%s: nq (%lld) must be a positive multiple of nkv (%lld)", op, (long long)nq, (long long)nkv);
+    if (b == 0 ? t != 0 : t % b != 0) return fail(PTO_ERR_SHAPE, "%s: query tokens (%lld) not a multiple of the batch (%lld)", op, (long long)t, (long long)b);
+    if (ts[3].shape[0] != b) return fail(PTO_ERR_SHAPE, "%s: block_tables has %lld rows, expected %lld", op, (long long)ts[3].shape[0], (long long)b);
+    const int64_t max_ctx = ts[3].shape[1] * bs;
+    const int64_t hsub = (nq / nkv + 15) / 16;
+    if (max_ctx > 0x3fffffff || t > 65535 || nkv * hsub > 65535 || nq > 0x7fff || blocks > 0x7fffffff)
+        return fail(PTO_ERR_SHAPE, "%s: problem too large", op);
+    pto::GqaArgs& a = plan->args;
+    a.q = ts[0].addr;
+    a.k = ts[1].addr;
+    a.v = ts[2].addr;
+    a.block_table = static_cast<const int32_t*>(ts[3].addr);
+    a.act_seq = static_cast<const int32_t*>(ts[4].addr);
+    a.out = ts[5].addr;
+    a.part_o = nullptr;
+    a.part_ml = nullptr;
+    a.n_blocks = blocks;
+    a.b = (int32_t)b;
+    a.s1 = b ? (int32_t)(t / b) : 0;
+    a.nq = (int32_t)nq;
+    a.nkv = (int32_t)nkv;
+    a.hsub = (int32_t)hsub;
+    a.block_size = (int32_t)bs;
+    a.bt_stride = (int32_t)ts[3].shape[1];
+    a.softmax_scale = p->softmax_scale;
+    pto::gqa_pick_chunk((int)max_ctx, p->kv_chunk, &a.chunk, &a.nsplit);
+    plan->ws_bytes = pto::gqa_workspace_bytes(t, (int)nq, a.nsplit);
+    return PTO_OK;
+}
+
 } // namespace
 
 extern "C" {
+
+uint64_t pto_gqa_decode_workspace(const PtoTensorDesc* tensors, uint32_t n_tensors, const PtoGqaParams* params)
+{
+    GqaPlan plan;
+    return plan_gqa(tensors, n_tensors, params, &plan) == PTO_OK ? plan.ws_bytes : 0;
+}
+
+int pto_gqa_decode_launch(const PtoTensorDesc* tensors, uint32_t n_tensors, const PtoGqaParams* params, void* workspace,
+                          uint64_t workspace_bytes, void* hip_stream)
+{
+    const char* op = "attention";
+    GqaPlan plan;
+    int rc = plan_gqa(tensors, n_tensors, params, &plan);
+    if (rc) return rc;
+    if (plan.ws_bytes > 0) {
+        if (workspace == nullptr || workspace_bytes < plan.ws_bytes)
+            return fail(PTO_ERR_WORKSPACE, "%s: workspace of %llu bytes required, got %llu", op,
+                        (unsigned long long)plan.ws_bytes, (unsigned long long)(workspace ? workspace_bytes : 0));
+        pto::GqaArgs& a = plan.args;
+        const uint64_t rows = (uint64_t)a.b * a.s1 * a.nq;
+        a.part_o = static_cast<float*>(workspace);
+        a.part_ml = a.part_o + rows * a.nsplit * 128;
+    }
+    hipError_t e = pto::gqa_launch(plan.args, static_cast<hipStream_t>(hip_stream));
+    if (e != hipSuccess) return fail(PTO_ERR_HIP, "%s: HIP launch failed: %s", op, hipGetErrorString(e));
+    return PTO_OK;
+}
 
 uint64_t pto_select_experts_workspace(const PtoTensorDesc*, uint32_t, const PtoSelectExpertsParams*) { return 0; }
 
@@ -385,7 +470,8 @@ int pto_kernel_timing_read(int kernel_id, double* total_ms, uint64_t* launches)
 const char* pto_kernel_name(int kernel_id)
 {
     static const char* names[] = {"indexer_score_kernel", "indexer_topk_kernel", "sfa_decode_kernel",
-                                  "sfa_combine_kernel", "indexer_select_kernel", "select_experts_kernel"};
+                                  "sfa_combine_kernel", "indexer_select_kernel", "select_experts_kernel",
+                                  "gqa_decode_kernel", "gqa_combine_kernel"};
     return kernel_id >= 0 && kernel_id < pto::KID_COUNT ? names[kernel_id] : "";
 }
 

@@ -71,4 +71,23 @@ struct SelectExpertsArgs {
 bool select_experts_supported(int ne, int n_group, int top_k);
 hipError_t select_experts_launch(const SelectExpertsArgs& a, hipStream_t stream);
 
+// ---------------------------------------------------------------- paged GQA decode attention
+struct GqaArgs {
+    const void* q;  // [t, nq, 128] bf16
+    const void* k;  // [blocks, block_size, nkv, 128] bf16
+    const void* v;  // same shape
+    const int32_t* block_table; // [b, bt_stride]
+    const int32_t* act_seq;     // [b]
+    void* out;                  // [t, nq, 128] bf16
+    float* part_o;              // workspace [t*nq, nsplit, 128] fp32 (nsplit > 1)
+    float* part_ml;             // workspace [t*nq, nsplit, 2]: running max (log2 units), sum
+    int64_t n_blocks;
+    int32_t b, s1, nq, nkv, hsub, block_size, bt_stride, nsplit, chunk;
+    float softmax_scale;
+};
+
+void gqa_pick_chunk(int max_ctx, int forced_chunk, int* chunk, int* nsplit);
+uint64_t gqa_workspace_bytes(int64_t t, int nq, int nsplit);
+hipError_t gqa_launch(const GqaArgs& a, hipStream_t stream);
+
 } // namespace pto
