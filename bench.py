@@ -48,6 +48,10 @@ def parse():
     ap.add_argument("--cpu-seqs", type=int, default=8, help="sequences of the workload timed on the CPU oracle")
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--packed", action="store_true", help="use the packed 656-byte-row attention entry point")
+    ap.add_argument("--workload", choices=["v32", "gqa", "select_experts"], default="v32",
+                    help="v32 (default): the headline DeepSeek-V3.2 indexer + sparse attention decode step; gqa: GLM-4.5 "
+                         "paged GQA decode (batch 64, 96/8 heads, contexts U[4096, 32768]); select_experts: GLM-4.5 "
+                         "router (8192 tokens x 160 experts)")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also launch one plain elementwise kernel that reads 256 MiB and writes 256 MiB, so that a "
                          "counter run of this command holds a dispatch of known HBM traffic to scale FETCH_SIZE / "
@@ -86,6 +90,112 @@ def make_workload(torch, dev, b, ctx, s1, nbuf, seed=0):
     return w
 
 
+def read_kernel_times(lib):
+    """us per launch of every library kernel timed since timing was enabled."""
+    lib.pto_kernel_name.restype = ctypes.c_char_p
+    kernels = {}
+    for kid in range(64):
+        if not lib.pto_kernel_name(kid):
+            break
+        ms, n = ctypes.c_double(0), ctypes.c_uint64(0)
+        lib.pto_kernel_timing_read(kid, ctypes.byref(ms), ctypes.byref(n))
+        if n.value:
+            kernels[lib.pto_kernel_name(kid).decode()] = ms.value * 1e3 / n.value
+    return kernels
+
+
+def timed(torch, lib, step, args):
+    for i in range(args.warmup):
+        step(i)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for i in range(args.steps):
+        step(i)
+    torch.cuda.synchronize()
+    ms_per_step = (time.perf_counter() - t0) * 1e3 / args.steps
+    lib.pto_kernel_timing_enable(1)
+    for i in range(args.steps):
+        step(i)
+    torch.cuda.synchronize()
+    lib.pto_kernel_timing_enable(0)
+    return ms_per_step, read_kernel_times(lib)
+
+
+def bench_gqa(args, torch, lib, dev):
+    """GLM-4.5 GQA decode: batch 64, 96 query heads over 8 KV heads, head dim 128, bf16, pages of 128 tokens, context
+    lengths U[4096, 32768] (seed 0); q/k/v ~ N(0,1) (the rotary embedding is applied upstream of this operator and does
+    not change its cost)."""
+    from pypto_amd.glm_v4_5.glm_attention import IfaTileShapeConfig, attention
+    b, nq, nkv, d, bs = 64, 96, 8, 128, 128
+    g = torch.Generator(device=dev).manual_seed(0)
+    act = torch.randint(4096, 32769, (b,), generator=g, device=dev, dtype=torch.int32)
+    pages = ((act + bs - 1) // bs).tolist()
+    n_pages = sum(pages)
+    perm = torch.randperm(n_pages, generator=g, device=dev).to(torch.int32)
+    table = torch.full((b, max(pages)), -1, dtype=torch.int32, device=dev)
+    pos = 0
+    for i, n in enumerate(pages):
+        table[i, :n] = perm[pos:pos + n]
+        pos += n
+    k = torch.randn((n_pages, bs, nkv, d), generator=g, device=dev, dtype=torch.bfloat16)
+    v = torch.randn((n_pages, bs, nkv, d), generator=g, device=dev, dtype=torch.bfloat16)
+    q = torch.randn((b, nq, d), generator=g, device=dev, dtype=torch.bfloat16)
+    out = torch.zeros_like(q)
+    cfg = IfaTileShapeConfig()
+
+    def step(i):
+        attention(q, k, v, table, act, out, d ** -0.5, cfg)
+
+    ms, kernels = timed(torch, lib, step, args)
+    tokens = int(act.sum())
+    work = tokens * nkv * d * 2 * 2 + 2 * b * nq * d * 2
+    us = kernels["gqa_decode_kernel"]
+    achieved = work / us / 1e3
+    print(json.dumps({
+        "metric": "decode tokens/sec + achieved HBM GB/s (% of peak), GLM-4.5 GQA decode b=64 ctx U[4K,32K]",
+        "value": round(b / (ms * 1e-3), 1), "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(ms, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16",
+        "data": "synthetic",
+        "config": {"workload": f"paged GQA decode attention, batch {b}, {nq}/{nkv} heads x {d}, bf16 KV, block {bs}, "
+                               f"{tokens} cached tokens in total"},
+        "roofline": {"kernel": "gqa_decode_kernel", "bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS,
+                     "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None,
+                     "work_per_launch": work, "us_per_launch": round(us, 2)},
+        "kernels": [{"kernel": n, "us": round(u, 2)} for n, u in kernels.items()], "cpu_baseline": None,
+    }))
+
+
+def bench_select_experts(args, torch, lib, dev):
+    """GLM-4.5 router: 8192 tokens x 160 experts, bf16 logits ~ N(0,1), fp32 bias ~ N(0,0.1), 8 groups, top-4 groups,
+    top-8 experts, renormalised, x 2.5."""
+    from pypto_amd.glm_v4_5.glm_select_experts import select_experts
+    t, ne, k = 8192, 160, 8
+    g = torch.Generator(device=dev).manual_seed(0)
+    logits = torch.randn((t, ne), generator=g, device=dev).to(torch.bfloat16)
+    bias = 0.1 * torch.randn((ne,), generator=g, device=dev)
+    w = torch.zeros((t, k), dtype=torch.float32, device=dev)
+    ids = torch.zeros((t, k), dtype=torch.int32, device=dev)
+
+    def step(i):
+        select_experts(logits, k, True, 4, 8, bias, w, ids, routed_scaling_factor=2.5, fill_neg_inf=True)
+
+    ms, kernels = timed(torch, lib, step, args)
+    work = t * ne * 2 + ne * 4 + t * k * 8
+    us = kernels["select_experts_kernel"]
+    achieved = work / us / 1e3
+    print(json.dumps({
+        "metric": "routed tokens/sec, GLM-4.5 select_experts 8192 x 160", "value": round(t / (ms * 1e-3), 1),
+        "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms, 4),
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
+        "config": {"workload": f"grouped expert selection, {t} tokens x {ne} experts, 8 groups / top-4, top-{k}"},
+        "roofline": {"kernel": "select_experts_kernel", "bound": "hbm", "achieved": round(achieved, 1),
+                     "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None,
+                     "work_per_launch": work, "us_per_launch": round(us, 2),
+                     "note": "3 MB of traffic: bound by launch and memory latency, not by a roofline"},
+        "kernels": [{"kernel": n, "us": round(u, 2)} for n, u in kernels.items()], "cpu_baseline": None,
+    }))
+
+
 def main():
     args = parse()
     if args.gpus != 1:
@@ -104,6 +214,10 @@ def main():
         sys.exit(2)
     lib = _runtime.load_library()
     dev = torch.device("cuda:0")
+    if args.workload == "gqa":
+        return bench_gqa(args, torch, lib, dev)
+    if args.workload == "select_experts":
+        return bench_select_experts(args, torch, lib, dev)
     b, ctx, s1 = args.batch, args.ctx, args.s1
     scale = 192 ** -0.5
     nbuf = 3
@@ -155,15 +269,7 @@ def main():
         step(i)
     torch.cuda.synchronize()
     lib.pto_kernel_timing_enable(0)
-    lib.pto_kernel_name.restype = ctypes.c_char_p
-    kernels = {}
-    for kid in range(64):
-        if not lib.pto_kernel_name(kid):
-            break
-        ms, n = ctypes.c_double(0), ctypes.c_uint64(0)
-        lib.pto_kernel_timing_read(kid, ctypes.byref(ms), ctypes.byref(n))
-        if n.value:
-            kernels[lib.pto_kernel_name(kid).decode()] = ms.value * 1e3 / n.value  # us per launch
+    kernels = read_kernel_times(lib)
 
     t = b * s1
     L = ctx

@@ -3,8 +3,8 @@
 // python/tests/ut/interpreter/_ops/moe_gating_topk.py:223-287 (groups, -inf fill, scaling factor).
 //
 // The whole problem is a few MB (8192 x 160 logits), so the kernel is bound by launch and memory latency, not by a
-// roofline: one wavefront per token, the token's scores in LDS, ranks by counting (rank of e = number of experts that
-// come before e in the order "value descending, index ascending"), which needs no sort network and is exact on ties.
+// roofline: one wavefront per token; groups are ranked by counting (rank of g = number of groups that come before g in
+// the order "value descending, index ascending"), experts by top_k rounds of a wave-wide arg-max on 64-bit keys.
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
@@ -39,9 +39,6 @@ __global__ __launch_bounds__(64) void select_experts_kernel(SelectExpertsArgs a)
     const LT* logits = static_cast<const LT*>(a.logits);
     const BT* bias = static_cast<const BT*>(a.bias);
     const float fill = a.fill_neg_inf ? -__builtin_inff() : 0.0f;
-
-    // pad the tail of the score array so that the 4-wide ranking loop never counts it
-    for (int e = ne + lane; e < SE_MAX_NE; e += 64) s_x[e] = -__builtin_inff();
 
     for (int64_t tok = blockIdx.x; tok < a.t; tok += gridDim.x) {
         float own_x[4], own_s[4];
@@ -83,24 +80,30 @@ __global__ __launch_bounds__(64) void select_experts_kernel(SelectExpertsArgs a)
             }
         }
         __syncthreads();
-        int rank[4] = {0, 0, 0, 0};
-        const int ne4 = (ne + 3) & ~3;
-        for (int e2 = 0; e2 < ne4; e2 += 4) {
-            const float4 v = *reinterpret_cast<const float4*>(&s_x[e2]);
-#pragma unroll
-            for (int j = 0; j < 4; ++j) {
-                const int e = lane + 64 * j;
-                rank[j] += before(v.x, e2, own_x[j], e) + before(v.y, e2 + 1, own_x[j], e) +
-                           before(v.z, e2 + 2, own_x[j], e) + before(v.w, e2 + 3, own_x[j], e);
-            }
-        }
+        // top_k rounds of a wave-wide arg-max over 64-bit keys (ordered score << 32 | ~expert): the largest key is the
+        // largest score and, among equal scores, the smallest expert id
+        unsigned long long key[4];
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
             const int e = lane + 64 * j;
-            if (e < ne && rank[j] < a.top_k) {
-                a.topk_ids[tok * a.top_k + rank[j]] = e;
-                s_w[rank[j]] = own_s[j];
+            key[j] = e < ne ? ((unsigned long long)f32_to_ordered(own_x[j] + 0.0f) << 32) | (uint32_t)(~e) : 0ull;
+        }
+        for (int r = 0; r < a.top_k; ++r) {
+            unsigned long long best = key[0] > key[1] ? key[0] : key[1];
+            const unsigned long long b2 = key[2] > key[3] ? key[2] : key[3];
+            best = best > b2 ? best : b2;
+#pragma unroll
+            for (int sh = 1; sh < 64; sh <<= 1) {
+                const unsigned long long o = __shfl_xor(best, sh);
+                best = best > o ? best : o;
             }
+            const int e = (int)~(uint32_t)best;
+            if (lane == 0) {
+                a.topk_ids[tok * a.top_k + r] = e;
+                s_w[r] = s_sig[e];
+            }
+#pragma unroll
+            for (int j = 0; j < 4; ++j) key[j] = key[j] == best ? 0ull : key[j];
         }
         __syncthreads();
         if (lane < a.top_k) {
