@@ -251,7 +251,7 @@ int plan_indexer(const PtoTensorDesc* ts, uint32_t n, const PtoIndexerParams* p,
     a.block_size = (int32_t)bs;
     a.bt_stride = (int32_t)ts[6].shape[1];
     a.k = p->selected_count;
-    a.score_stride = (int32_t)((max_ctx + 3) & ~(int64_t)3); // rows of the score matrix stay 16-byte aligned
+    a.score_stride = (int32_t)((max_ctx + 4095) & ~(int64_t)4095); // whole workgroup spans of the score kernel
     plan->ws_bytes = pto::indexer_workspace_bytes((int)t, a.score_stride);
     return PTO_OK;
 }

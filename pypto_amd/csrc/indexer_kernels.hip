@@ -157,6 +157,161 @@ __global__ __launch_bounds__(256) void indexer_score_kernel(IndexerArgs a)
     }
 }
 
+// relu(a) * 2^-11 and relu(b) * 2^-11, each rounded once to fp16, packed (a in the low half).  The product is exact in
+// fp32 (|a| < 2^21) and relu commutes with the rounding, so it is taken on the packed pair.  (Written in plain C on
+// purpose: the compiler's hazard recognizer does not look inside inline assembly, and a hand-placed VALU write into a
+// register that an MFMA is still writing goes wrong.)
+typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ uint32_t relu_scale_pack(int a, int b)
+{
+    f16x2 v = {(_Float16)((float)a * 0x1p-11f), (_Float16)((float)b * 0x1p-11f)};
+    const f16x2 z = {(_Float16)0.f, (_Float16)0.f};
+    return __builtin_bit_cast(uint32_t, __builtin_elementwise_max(v, z));
+}
+
+// Score kernel for block sizes that are multiples of 128: a wavefront owns 128 consecutive keys of one page per pass
+// (one page-table entry; the entries of all its passes are fetched up front with one load, lane p holding pass p's),
+// keeps the loads of the next NBUF-1 half passes (64 keys, 8 KB each) in flight while it scores the current one, and
+// files its results 64 at a time: w_scale sits in every row of the head-sum operand, so every lane group holds the 16
+// scores of a key group and lane group g keeps those of key group g - after four key groups lane l holds the score of
+// key l of the 64, next to that key's scale (loaded with one 128-byte instruction per 64 keys).
+constexpr int PPASSES = 4; // passes (of 512 keys) per workgroup of the paged kernel
+template <int S1>
+__global__ __launch_bounds__(256, S1 == 1 ? 3 : 2) void indexer_score_paged_kernel(IndexerArgs a)
+{
+    constexpr int NBUF = 2; // half-pass buffers: NBUF-1 halves ahead (deeper prefetch measured no faster)
+    constexpr int NHALF = 2 * PPASSES;
+    __shared__ uint32_t hist[S1][NBINS];
+    __shared__ __align__(16) _Float16 s_ws[S1][64];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int l16 = lane & 15, g = lane >> 4;
+    const int bi = blockIdx.y;
+    const int sgrp = blockIdx.z;
+    const int L = a.act_seq[bi];
+    if (blockIdx.x * (CHUNK * PPASSES) >= L) return;
+    const int row0 = bi * a.s1 + sgrp * S1;
+    const int bs = a.block_size;
+    const int wtok = blockIdx.x * (CHUNK * PPASSES) + wave * 128; // first key of this wave's pass 0
+
+    // lane p: first cache row of pass p (-1: unmapped page); a pass past the end re-reads the sequence's first page
+    // and is discarded
+    int64_t myrow;
+    {
+        const int mytok = wtok + (lane < PPASSES ? lane : 0) * CHUNK;
+        const int tc = mytok < L ? mytok : 0;
+        const int pg = a.block_table[(int64_t)bi * a.bt_stride + tc / bs];
+        myrow = (pg >= 0 && pg < a.n_blocks) ? (int64_t)pg * bs + tc % bs : -1;
+    }
+    auto pass_row = [&](int pass) {
+        const uint32_t lo = __builtin_amdgcn_readlane((uint32_t)myrow, pass);
+        const uint32_t hi = __builtin_amdgcn_readlane((uint32_t)(myrow >> 32), pass);
+        return (int64_t)(((uint64_t)hi << 32) | lo);
+    };
+
+    i32x4 kf[NBUF][4][2];
+    uint16_t ksc[NBUF][2]; // [buffer][unused for odd halves]: the scales of a pass travel with its first half
+    auto load_half = [&](int hh, int buf) {
+        const int64_t r = pass_row(hh >> 1);
+        const int64_t rb = r < 0 ? 0 : r;
+        const int8_t* kp = a.k_cache + (rb + 64 * (hh & 1) + l16) * D + 16 * g;
+#pragma unroll
+        for (int jj = 0; jj < 4; ++jj) {
+            kf[buf][jj][0] = *reinterpret_cast<const i32x4*>(kp + jj * 16 * D);
+            kf[buf][jj][1] = *reinterpret_cast<const i32x4*>(kp + jj * 16 * D + 64);
+        }
+        ksc[buf][0] = a.k_scale[rb + 64 * (hh & 1) + lane];
+    };
+    for (int i = tid; i < S1 * NBINS; i += 256) (&hist[0][0])[i] = 0;
+    if (tid < 64 * S1) {
+        const int64_t h = (int64_t)row0 * a.nh + tid;
+        const _Float16 qs = __builtin_bit_cast(_Float16, a.q_scale[h]);
+        const _Float16 w = __builtin_bit_cast(_Float16, a.weights[h]);
+        (&s_ws[0][0])[tid] = (_Float16)(qs * w); // one fp16 rounding
+    }
+    // int8 A fragments: head hb*16 + l16, bytes 64*ks + 16*g .. +15
+    i32x4 qf[S1][4][2];
+#pragma unroll
+    for (int s = 0; s < S1; ++s)
+#pragma unroll
+        for (int hb = 0; hb < 4; ++hb) {
+            const int8_t* qp = a.q + ((int64_t)(row0 + s) * a.nh + hb * 16 + l16) * D + 16 * g;
+            qf[s][hb][0] = *reinterpret_cast<const i32x4*>(qp);
+            qf[s][hb][1] = *reinterpret_cast<const i32x4*>(qp + 64);
+        }
+    __syncthreads();
+    // fp16 A fragments of the head sum, the same in every row: k-slot (g, e) of MFMA mm is head
+    // 32*mm + 16*(e/4) + 4*g + e%4 - the head whose int32 result this lane group holds in that slot
+    f16x8 wa[S1][2];
+#pragma unroll
+    for (int s = 0; s < S1; ++s)
+#pragma unroll
+        for (int mm = 0; mm < 2; ++mm) {
+            typedef _Float16 f16x4 __attribute__((ext_vector_type(4)));
+            const f16x4 lo = *reinterpret_cast<const f16x4*>(&s_ws[s][32 * mm + 4 * g]);
+            const f16x4 hi = *reinterpret_cast<const f16x4*>(&s_ws[s][32 * mm + 16 + 4 * g]);
+            wa[s][mm] = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+        }
+    // The prefetch starts only here, and every memory operation of the loop below is unconditional, so that the
+    // number of memory operations in flight is the same on every path into the loop and the waits can count them
+#pragma unroll
+    for (int u = 0; u < NBUF - 1; ++u) load_half(u, u);
+
+    auto compute_half = [&](int hh, int buf) {
+        float res[S1];
+#pragma unroll
+        for (int s = 0; s < S1; ++s) res[s] = 0.f;
+#pragma unroll
+        for (int jj = 0; jj < 4; ++jj) {
+#pragma unroll
+            for (int s = 0; s < S1; ++s) {
+                u32x4 y[2];
+#pragma unroll
+                for (int hb = 0; hb < 4; ++hb) {
+                    i32x4 acc = {0, 0, 0, 0};
+                    acc = __builtin_amdgcn_mfma_i32_16x16x64_i8(qf[s][hb][0], kf[buf][jj][0], acc, 0, 0, 0);
+                    acc = __builtin_amdgcn_mfma_i32_16x16x64_i8(qf[s][hb][1], kf[buf][jj][1], acc, 0, 0, 0);
+                    y[hb >> 1][2 * (hb & 1)] = relu_scale_pack(acc[0], acc[1]);
+                    y[hb >> 1][2 * (hb & 1) + 1] = relu_scale_pack(acc[2], acc[3]);
+                }
+                f32x4 sum = {0.f, 0.f, 0.f, 0.f};
+                sum = __builtin_amdgcn_mfma_f32_16x16x32_f16(wa[s][0], __builtin_bit_cast(f16x8, y[0]), sum, 0, 0, 0);
+                sum = __builtin_amdgcn_mfma_f32_16x16x32_f16(wa[s][1], __builtin_bit_cast(f16x8, y[1]), sum, 0, 0, 0);
+                res[s] = jj == g ? sum[0] : res[s];
+            }
+        }
+        // score rows are padded to whole workgroup spans, so the store needs no bounds check
+        const int tok = wtok + (hh >> 1) * CHUNK + 64 * (hh & 1) + lane;
+        const float ks = pass_row(hh >> 1) >= 0 ? f16_bits_to_f32(ksc[buf][0]) : 0.f;
+#pragma unroll
+        for (int s = 0; s < S1; ++s) {
+            const float sc = res[s] * ks;
+            a.scores[(int64_t)(row0 + s) * a.score_stride + tok] = sc;
+            const int eff = L - (a.s1 - 1 - (sgrp * S1 + s));
+            if (tok < eff) atomicAdd(&hist[s][score_key(sc) >> 21], 1u);
+        }
+    };
+
+    // NBUF halves per trip, so that buffer indices are compile-time constants; past the end the last half is loaded
+    // again (a cache hit whose data is never used) so that the loads stay unconditional
+    static_assert(NHALF % NBUF == 0, "whole trips");
+    for (int base = 0; base < NHALF; base += NBUF) {
+#pragma unroll
+        for (int u = 0; u < NBUF; ++u) {
+            const int hh = base + u;
+            if (hh < NHALF) {
+                const int nx = hh + NBUF - 1;
+                load_half(nx < NHALF ? nx : NHALF - 1, (u + NBUF - 1) % NBUF);
+                compute_half(hh, u);
+            }
+        }
+    }
+    __syncthreads();
+    for (int i = tid; i < S1 * NBINS; i += 256) {
+        const uint32_t c = (&hist[0][0])[i];
+        if (c) atomicAdd(a.hist + (int64_t)(row0 + i / NBINS) * NBINS + (i % NBINS), c);
+    }
+}
+
 __global__ void indexer_zero_kernel(uint32_t* p, int n)
 {
     const int i = blockIdx.x * blockDim.x + threadIdx.x;
@@ -416,12 +571,18 @@ hipError_t indexer_launch(const IndexerArgs& a, hipStream_t stream)
     if (t == 0) return hipSuccess;
     const int max_ctx = a.bt_stride * a.block_size;
     const int chunks = (max_ctx + CHUNK * PASSES - 1) / (CHUNK * PASSES);
+    const int pchunks = (max_ctx + CHUNK * PPASSES - 1) / (CHUNK * PPASSES);
     const int nzero = t * (NBINS + 4);
     hipLaunchKernelGGL(indexer_zero_kernel, dim3((nzero + 255) / 256), dim3(256), 0, stream, a.hist, nzero);
     {
         ScopedKernelTimer tm(KID_INDEXER_SCORE, stream);
         const bool pow2 = (a.block_size & (a.block_size - 1)) == 0;
-        if (a.s1 % 2 == 0) {
+        if (a.block_size % 128 == 0) {
+            if (a.s1 % 2 == 0)
+                hipLaunchKernelGGL(indexer_score_paged_kernel<2>, dim3(pchunks, a.b, a.s1 / 2), dim3(256), 0, stream, a);
+            else
+                hipLaunchKernelGGL(indexer_score_paged_kernel<1>, dim3(pchunks, a.b, a.s1), dim3(256), 0, stream, a);
+        } else if (a.s1 % 2 == 0) {
             auto kern = pow2 ? indexer_score_kernel<2, true> : indexer_score_kernel<2, false>;
             hipLaunchKernelGGL(kern, dim3(chunks, a.b, a.s1 / 2), dim3(256), 0, stream, a);
         } else {
