@@ -470,6 +470,110 @@ __device__ __forceinline__ void radix_select64(Each&& for_each, Emit&& emit, uin
     }
 }
 
+// cand[0 .. m) holds the selected words in any order (the rest of its 2048 slots is zero): write their indices in
+// descending word order, then -1 up to k.  The words are first grouped by key into at most 2048 equal steps of the
+// selected keys' range, so a counting pass (histogram, suffix scan, scatter) puts every word within a few slots of
+// its place - and then ranked inside their group by direct comparison.  A bin with more than 64 words (heavily tied scores)
+// would make that ranking quadratic; then a bitonic sort of all 2048 words is used instead.
+// Workgroup of 1024 lanes; hist has 2048 words, scratch 8192 words (start | cursor | grouped words), tmp 16.
+__device__ __forceinline__ void order_and_write(uint64_t* cand, uint32_t m, uint32_t* hist, uint32_t* scratch,
+                                                uint32_t* tmp, uint32_t* s_flag, int32_t* out, int k)
+{
+    const int tid = threadIdx.x;
+    uint32_t* start = scratch;          // [2048] slots taken by the higher bins
+    uint32_t* cursor = scratch + NBINS; // [2048]
+    uint64_t* grouped = reinterpret_cast<uint64_t*>(scratch + 2 * NBINS); // [2048]
+    hist[tid] = 0;
+    hist[tid + 1024] = 0;
+    cursor[tid] = 0;
+    cursor[tid + 1024] = 0;
+    if (tid == 0) {
+        *s_flag = 0;
+        tmp[14] = 0xffffffffu; // smallest selected key
+        tmp[15] = 0u;          // largest selected key
+    }
+    __syncthreads();
+    uint64_t w[2];
+    uint32_t bin[2];
+    bool valid[2];
+    uint32_t kmin = 0xffffffffu, kmax = 0u;
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+        const int i = tid + 1024 * h;
+        valid[h] = (uint32_t)i < m;
+        w[h] = cand[i];
+        if (valid[h]) {
+            kmin = min(kmin, (uint32_t)(w[h] >> 32));
+            kmax = max(kmax, (uint32_t)(w[h] >> 32));
+        }
+    }
+#pragma unroll
+    for (int d = 1; d < 64; d <<= 1) {
+        kmin = min(kmin, (uint32_t)__shfl_xor((int)kmin, d));
+        kmax = max(kmax, (uint32_t)__shfl_xor((int)kmax, d));
+    }
+    if ((tid & 63) == 0) {
+        atomicMin(&tmp[14], kmin);
+        atomicMax(&tmp[15], kmax);
+    }
+    __syncthreads();
+    // bins: the selected keys' range cut into at most 2048 equal steps (the keys are order-preserving images of the
+    // scores, dense enough over the top-k range that a step holds a handful of words)
+    kmin = tmp[14];
+    const uint32_t range = tmp[15] - kmin;
+    const int shift = max(0, 21 - (int)__builtin_clz(range | 1u));
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+        bin[h] = ((uint32_t)(w[h] >> 32) - kmin) >> shift;
+        if (valid[h]) atomicAdd(&hist[bin[h]], 1u);
+    }
+    __syncthreads();
+    {
+        const uint32_t h_lo = hist[2 * tid], h_hi = hist[2 * tid + 1]; // lane t owns bins 2t and 2t+1
+        if (h_lo > 64u || h_hi > 64u) *s_flag = 1;
+        const uint32_t incl = block_suffix_sum<16>(h_lo + h_hi, tmp);
+        start[2 * tid + 1] = incl - h_lo - h_hi;
+        start[2 * tid] = incl - h_lo;
+    }
+    __syncthreads();
+    if (*s_flag == 0) {
+#pragma unroll
+        for (int h = 0; h < 2; ++h)
+            if (valid[h]) grouped[start[bin[h]] + atomicAdd(&cursor[bin[h]], 1u)] = w[h];
+        __syncthreads();
+#pragma unroll
+        for (int h = 0; h < 2; ++h)
+            if (valid[h]) {
+                const uint32_t s0 = start[bin[h]], c = hist[bin[h]];
+                uint32_t rank = 0;
+                for (uint32_t j = 0; j < c; ++j) rank += grouped[s0 + j] > w[h] ? 1u : 0u;
+                if ((int)(s0 + rank) < k) out[s0 + rank] = (int32_t)(0xffffffffu - (uint32_t)(w[h] & 0xffffffffull));
+            }
+        for (int j = (int)m + tid; j < k; j += 1024) out[j] = -1;
+        return;
+    }
+    // bitonic sort, descending, 2048 words, two per lane.  A compare-exchange step of stride <= 64 stays inside
+    // the 128 words owned by one wavefront (lane i of wave w handles the pair (128w + 2i - i%stride, + stride)),
+    // so only the steps of stride >= 128 need a workgroup barrier; the others rely on LDS operations of one
+    // wavefront completing in order.
+    for (int size = 2; size <= MAX_K; size <<= 1) {
+        for (int stride = size >> 1; stride > 0; stride >>= 1) {
+            if (stride >= 128) __syncthreads();
+            const int pos = 2 * tid - (tid & (stride - 1)); // lower index of the pair
+            const bool desc = (pos & size) == 0;
+            const uint64_t lo = cand[pos], hi = cand[pos + stride];
+            if ((lo < hi) == desc) {
+                cand[pos] = hi;
+                cand[pos + stride] = lo;
+            }
+            if (stride >= 128) __syncthreads();
+            else __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        }
+    }
+    __syncthreads();
+    for (int j = tid; j < k; j += 1024) out[j] = (int32_t)(0xffffffffu - (uint32_t)(cand[j] & 0xffffffffull));
+}
+
 __global__ __launch_bounds__(1024) void indexer_topk_kernel(IndexerArgs a)
 {
     __shared__ uint32_t hist[NBINS];
@@ -518,27 +622,8 @@ __global__ __launch_bounds__(1024) void indexer_topk_kernel(IndexerArgs a)
     }
     __syncthreads();
 
-    // bitonic sort, descending, 2048 words, two per lane.  A compare-exchange step of stride <= 64 stays inside
-    // the 128 words owned by one wavefront (lane i of wave w handles the pair (128w + 2i - i%stride, + stride)),
-    // so only the steps of stride >= 128 need a workgroup barrier; the others rely on LDS operations of one
-    // wavefront completing in order.
-    for (int size = 2; size <= MAX_K; size <<= 1) {
-        for (int stride = size >> 1; stride > 0; stride >>= 1) {
-            if (stride >= 128) __syncthreads();
-            const int pos = 2 * tid - (tid & (stride - 1)); // lower index of the pair
-            const bool desc = (pos & size) == 0;
-            const uint64_t lo = cand[pos], hi = cand[pos + stride];
-            if ((lo < hi) == desc) {
-                cand[pos] = hi;
-                cand[pos + stride] = lo;
-            }
-            if (stride >= 128) __syncthreads();
-            else __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-        }
-    }
-    __syncthreads();
-    for (int j = tid; j < k; j += 1024)
-        a.topk_res[(int64_t)row * k + j] = (int32_t)(0xffffffffu - (uint32_t)(cand[j] & 0xffffffffull));
+    order_and_write(cand, (uint32_t)min(n, k), hist, reinterpret_cast<uint32_t*>(tie), tmp, &s_bin,
+                    a.topk_res + (int64_t)row * k, k);
 }
 
 } // namespace

@@ -102,6 +102,13 @@ def test_reference_cases(cuda):
         check_topk(case, run_indexer(case, cuda))
 
 
+def test_contexts_beyond_131072_tokens(cuda):
+    case = oi.make_case(2, 1, [140000, 3000], seed=21)
+    check_topk(case, run_indexer(case, cuda))
+    case = oi.make_case(1, 2, [133000], seed=22, dist="driver")
+    check_topk(case, run_indexer(case, cuda))
+
+
 def test_full_size_config3(cuda):
     # BASELINE config 3: b=32, 64x128 index heads, context lengths U[8192, 65536], top-2048
     g = torch.Generator().manual_seed(33)
