@@ -29,10 +29,10 @@ MFMA_BF16_PEAK_TFLOPS = 2500.0
 # the same counters read for a 256 MiB-in / 256 MiB-out elementwise kernel (--calibrate-copy); measured on the default
 # workload only (batch 32, s1 1, ctx 65536, three cache tensors) and reported for that workload only.
 MEASURED_TRAFFIC_BYTES = {
-    "indexer_score_kernel": 275.4e6 + 9.0e6,
+    "indexer_score_kernel": 276.0e6 + 8.9e6,
     "sfa_decode_kernel": 70.6e6 + 34.5e6,
     "sfa_combine_kernel": 35.7e6 + 4.2e6,
-    "indexer_select_kernel": 10.6e6 + 0.3e6,
+    "indexer_select_kernel": 10.6e6 + 0.8e6,
     "indexer_topk_kernel": 0.8e6 + 0.3e6,
 }
 
@@ -52,6 +52,8 @@ def parse():
                     help="v32 (default): the headline DeepSeek-V3.2 indexer + sparse attention decode step; gqa: GLM-4.5 "
                          "paged GQA decode (batch 64, 96/8 heads, contexts U[4096, 32768]); select_experts: GLM-4.5 "
                          "router (8192 tokens x 160 experts)")
+    ap.add_argument("--graph", action="store_true",
+                    help="replay the step from HIP graphs (one per cache copy) instead of launching it eagerly")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also launch one plain elementwise kernel that reads 256 MiB and writes 256 MiB, so that a "
                          "counter run of this command holds a dispatch of known HBM traffic to scale FETCH_SIZE / "
@@ -91,8 +93,12 @@ def make_workload(torch, dev, b, ctx, s1, nbuf, seed=0):
 
 
 def read_kernel_times(lib):
-    """us per launch of every library kernel timed since timing was enabled."""
+    """us per launch of every library kernel timed since timing was enabled, less the offset of the event pairs (what
+    a pair around an empty kernel reads beyond that kernel's own duration)."""
+    import torch
     lib.pto_kernel_name.restype = ctypes.c_char_p
+    off = ctypes.c_double(0)
+    lib.pto_kernel_timing_overhead(ctypes.c_void_p(torch.cuda.current_stream().cuda_stream), ctypes.byref(off))
     kernels = {}
     for kid in range(64):
         if not lib.pto_kernel_name(kid):
@@ -100,7 +106,8 @@ def read_kernel_times(lib):
         ms, n = ctypes.c_double(0), ctypes.c_uint64(0)
         lib.pto_kernel_timing_read(kid, ctypes.byref(ms), ctypes.byref(n))
         if n.value:
-            kernels[lib.pto_kernel_name(kid).decode()] = ms.value * 1e3 / n.value
+            kernels[lib.pto_kernel_name(kid).decode()] = max(ms.value * 1e3 / n.value - off.value * 1e3, 0.05)
+    read_kernel_times.offset_us = off.value * 1e3
     return kernels
 
 
@@ -245,6 +252,24 @@ def main():
             sparse_flash_attention_quant_d(w["q_nope"], w["q_rope"], s["kn"], s["kr"], s["ks"], tk, w["table"],
                                            w["act"], w["out"], 128, 1, scale, 2048, 128, w["pages_per_seq"], tile)
 
+    eager_step = step
+    if args.graph:
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            for i in range(nbuf):
+                eager_step(i)
+        torch.cuda.current_stream().wait_stream(side)
+        graphs = []
+        for i in range(nbuf):
+            g = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(g):
+                eager_step(i)
+            graphs.append(g)
+
+        def step(i):  # noqa: F811 - the timed loop below replays the captured steps
+            graphs[i % nbuf].replay()
+
     if args.calibrate_copy:
         src = torch.ones(64 << 20, dtype=torch.int32, device=dev)
         dst = torch.empty_like(src)
@@ -266,7 +291,7 @@ def main():
     # second pass over the same steps with an event pair around every kernel launch
     lib.pto_kernel_timing_enable(1)
     for i in range(args.steps):
-        step(i)
+        eager_step(i)
     torch.cuda.synchronize()
     lib.pto_kernel_timing_enable(0)
     kernels = read_kernel_times(lib)
@@ -314,11 +339,12 @@ def main():
         "value": round(tokens_per_s, 1), "unit": "tokens/s", "n_gpus": 1, "steps": args.steps,
         "warmup": args.warmup, "ms_per_step": round(ms_per_step, 4), "higher_is_better": True, "scaling": "weak",
         "vs_baseline": None, "dtype": "int8+bf16",
-        "data": "synthetic",
+        "data": "synthetic", "launch": "hip graph replay" if args.graph else "eager",
         "config": {"workload": f"lightning indexer top-2048 + sparse flash attention decode, batch {b}, "
                                f"s1 {s1}, ctx {ctx}, 64x128 int8 index heads, 128 heads x (512 nope + 64 rope), "
                                f"int8 paged MLA cache, block 128, {'packed 656 B rows' if args.packed else 'three cache tensors'}"},
-        "roofline": roofline, "kernels": per_kernel, "cpu_baseline": cpu_baseline,
+        "roofline": roofline, "kernels": per_kernel, "event_pair_offset_us": round(read_kernel_times.offset_us, 2),
+        "cpu_baseline": cpu_baseline,
     }))
 
 

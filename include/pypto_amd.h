@@ -186,6 +186,10 @@ const char* pto_last_error(void);
  */
 int pto_kernel_timing_enable(int on);
 int pto_kernel_timing_read(int kernel_id, double* total_ms, uint64_t* launches);
+/* The offset of the instrument: what an event pair around an empty kernel reads on `hip_stream`, less that kernel's own
+ * duration (averaged over a few pairs; synchronises the stream).  Take it off every per-launch figure of
+ * pto_kernel_timing_read to get dispatch begin-to-end durations. */
+int pto_kernel_timing_overhead(void* hip_stream, double* ms);
 const char* pto_kernel_name(int kernel_id);
 
 /* ABI version of this header. */

@@ -1,4 +1,4 @@
-"""CPU oracle for the DeepSeek-V3.2 quantized decode-attention path.
+"""CPU oracle for the DeepSeek-V3.2 quantized decode-attention path and the two GLM-4.5 operators beside it.
 
 TEST INFRASTRUCTURE ONLY.  Nothing under ``pypto_amd/`` imports this package.
 It may be imported from ``tests/``, from ``__graft_entry__.smoke()`` and from
@@ -16,6 +16,10 @@ reference checkout):
   indexer.py  lightning indexer golden         models/deepseek_v32_exp/deepseekv32_lightning_indexer_quant.py:46-307
   topk.py     top-k ordering rule              framework/src/interface/interpreter/calculator/calc_torch.cpp:2481-2494,2734-2749
   compare.py  tolerance comparators            models/deepseek_v32_exp/utils/compare.py:16-125
+  select_experts.py  grouped expert selection  models/glm_v4_5/glm_select_experts.py:274-313
+                                               python/tests/ut/interpreter/_ops/moe_gating_topk.py:223-287
+  gqa.py      paged GQA decode goldens         models/glm_v4_5/glm_attention.py:1374-1483
+                                               models/glm_v4_5/utils/golden/attn_golden.py:97-130,300-321
 
 The arithmetic of those goldens is PyTorch's CPU arithmetic (an unpinned,
 un-vendored dependency of the reference), so every function here is pinned in

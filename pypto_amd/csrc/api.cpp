@@ -467,6 +467,14 @@ int pto_kernel_timing_read(int kernel_id, double* total_ms, uint64_t* launches)
     return PTO_OK;
 }
 
+int pto_kernel_timing_overhead(void* hip_stream, double* ms)
+{
+    if (ms == nullptr) return fail(PTO_ERR_PARAM, "pto_kernel_timing_overhead: null output");
+    hipError_t e = pto::timing_pair_overhead(static_cast<hipStream_t>(hip_stream), ms);
+    if (e != hipSuccess) return fail(PTO_ERR_HIP, "pto_kernel_timing_overhead: %s", hipGetErrorString(e));
+    return PTO_OK;
+}
+
 const char* pto_kernel_name(int kernel_id)
 {
     static const char* names[] = {"indexer_score_kernel", "indexer_topk_kernel", "sfa_decode_kernel",

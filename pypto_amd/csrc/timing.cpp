@@ -58,4 +58,44 @@ hipError_t timing_collect(int kid, double* total_ms, uint64_t* launches)
     return rc;
 }
 
+namespace {
+__global__ void timing_nop_kernel() {}
+// What the profiler reports for the begin-to-end duration of an empty dispatch on this part (rocprofv3 kernel trace).
+constexpr double kNopDispatchMs = 0.002;
+} // namespace
+
+hipError_t timing_pair_overhead(hipStream_t s, double* ms_out)
+{
+    // An event pair around a kernel reads the kernel's duration plus the time the command processor spends on the
+    // two events and the dispatch; that offset is what a pair around an empty kernel reads, less the empty kernel's
+    // own duration.  Averaged over a few pairs.
+    constexpr int N = 32;
+    hipEvent_t a[N], b[N];
+    hipError_t rc = hipStreamSynchronize(s);
+    for (int i = 0; i < N; ++i) {
+        if (rc == hipSuccess) rc = hipEventCreate(&a[i]);
+        if (rc == hipSuccess) rc = hipEventCreate(&b[i]);
+    }
+    if (rc != hipSuccess) return rc;
+    hipLaunchKernelGGL(timing_nop_kernel, dim3(1), dim3(64), 0, s); // first launch loads the code object
+    rc = hipStreamSynchronize(s);
+    for (int i = 0; i < N; ++i) {
+        (void)hipEventRecord(a[i], s);
+        hipLaunchKernelGGL(timing_nop_kernel, dim3(1), dim3(64), 0, s);
+        (void)hipEventRecord(b[i], s);
+    }
+    rc = hipStreamSynchronize(s);
+    double total = 0.0;
+    for (int i = 0; i < N; ++i) {
+        float ms = 0.f;
+        if (rc == hipSuccess) rc = hipEventElapsedTime(&ms, a[i], b[i]);
+        total += ms;
+        (void)hipEventDestroy(a[i]);
+        (void)hipEventDestroy(b[i]);
+    }
+    const double off = total / N - kNopDispatchMs;
+    *ms_out = off > 0.0 ? off : 0.0;
+    return rc;
+}
+
 } // namespace pto

@@ -15,6 +15,9 @@ void timing_end(int kid, hipStream_t s);
 // Wait for the recorded events, return their summed duration and count, and forget them.
 hipError_t timing_collect(int kid, double* total_ms, uint64_t* launches);
 
+// The instrument's own offset: an event pair around an empty kernel, less that kernel's duration.
+hipError_t timing_pair_overhead(hipStream_t s, double* ms_out);
+
 struct ScopedKernelTimer {
     int kid;
     hipStream_t s;
