@@ -48,7 +48,7 @@ def parse():
     ap.add_argument("--cpu-seqs", type=int, default=8, help="sequences of the workload timed on the CPU oracle")
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--packed", action="store_true", help="use the packed 656-byte-row attention entry point")
-    ap.add_argument("--workload", choices=["v32", "gqa", "select_experts"], default="v32",
+    ap.add_argument("--workload", choices=["v32", "gqa", "select_experts", "indexer_prolog"], default="v32",
                     help="v32 (default): the headline DeepSeek-V3.2 indexer + sparse attention decode step; gqa: GLM-4.5 "
                          "paged GQA decode (batch 64, 96/8 heads, contexts U[4096, 32768]); select_experts: GLM-4.5 "
                          "router (8192 tokens x 160 experts)")
@@ -203,6 +203,42 @@ def bench_select_experts(args, torch, lib, dev):
     }))
 
 
+def bench_indexer_prolog(args, torch, lib, dev):
+    """DeepSeek-V3.2 lightning-indexer prolog at decode size: 32 new tokens (batch 32, one each), h 7168, q_lora_rank
+    1536, 64 index heads x 128, a 64K-token paged index cache per sequence; the reference generator's distributions."""
+    from pypto_amd.deepseek_v32_exp import lightning_indexer_prolog_quant_impl as impl
+    sys.path.insert(0, os.path.join(ROOT, "tests"))
+    from oracle import indexer_prolog as op
+    b = args.batch
+    case = op.make_case(b, 1, 4096, seed=0)
+    d = {k: v.to(dev) for k, v in case.items()}
+    t, n = b, 64
+    tensors = [d["x"], d["q_norm"], d["q_norm_scale"], d["w_qb"], d["w_qb_scale"], d["w_k"], d["w_proj"], d["ln_gamma"],
+               d["ln_beta"], d["cos"], d["sin"], d["hadamard_q"], d["hadamard_k"], d["k_cache"], d["k_scale_cache"],
+               d["k_cache_index"], torch.zeros((t, n, 128), dtype=torch.int8, device=dev),
+               torch.zeros((t, n, 1), dtype=torch.float16, device=dev), d["k_cache"], d["k_scale_cache"],
+               torch.zeros((t, n), dtype=torch.float16, device=dev)]
+    cfg, attrs = impl.IndexerPrologQuantConfigs(), impl.IndexerPrologQuantAttr()
+
+    def step(i):
+        impl.lightning_indexer_prolog_quant(*tensors, cfg, attrs)
+
+    ms, kernels = timed(torch, lib, step, args)
+    work = 1536 * 8192 + 7168 * (128 + 64) * 2 + t * (7168 * 2 + 1536 + 64 * 130 + 64 * 2 + 130)
+    total_us = sum(kernels.values())
+    print(json.dumps({
+        "metric": "prolog tokens/sec, DeepSeek-V3.2 lightning_indexer_prolog_quant decode", "value": round(t / (ms * 1e-3), 1),
+        "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms, 4),
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "int8+bf16", "data": "synthetic",
+        "config": {"workload": f"lightning indexer prolog, {t} tokens, h 7168, q_lora_rank 1536, 64 x 128 index heads"},
+        "roofline": {"kernel": "prolog (4 kernels)", "bound": "hbm", "achieved": round(work / total_us / 1e3, 1),
+                     "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(work / total_us / 1e3 / HBM_PEAK_GBS, 4),
+                     "traffic": None, "work_per_launch": work, "us_per_launch": round(total_us, 2),
+                     "note": "15 MB of weights read once: bound by launch and memory latency at decode sizes"},
+        "kernels": [{"kernel": k, "us": round(u, 2)} for k, u in kernels.items()], "cpu_baseline": None,
+    }))
+
+
 def main():
     args = parse()
     if args.gpus != 1:
@@ -225,6 +261,8 @@ def main():
         return bench_gqa(args, torch, lib, dev)
     if args.workload == "select_experts":
         return bench_select_experts(args, torch, lib, dev)
+    if args.workload == "indexer_prolog":
+        return bench_indexer_prolog(args, torch, lib, dev)
     b, ctx, s1 = args.batch, args.ctx, args.s1
     scale = 192 ** -0.5
     nbuf = 3

@@ -32,7 +32,7 @@ typedef struct {
 } PtoTensorDesc;
 
 /* framework/include/tilefwk/data_type.h:33-65 (positions in the DataType enum) */
-enum PtoDataType { PTO_DT_INT8 = 1, PTO_DT_INT32 = 3, PTO_DT_FP16 = 6, PTO_DT_FP32 = 7, PTO_DT_BF16 = 8 };
+enum PtoDataType { PTO_DT_INT8 = 1, PTO_DT_INT32 = 3, PTO_DT_INT64 = 4, PTO_DT_FP16 = 6, PTO_DT_FP32 = 7, PTO_DT_BF16 = 8 };
 
 /* Error codes (negative).  pto_last_error() gives the message of the calling thread's last failure. */
 enum PtoStatus {
@@ -170,6 +170,43 @@ uint64_t pto_gqa_decode_workspace(const PtoTensorDesc* tensors, uint32_t n_tenso
 int pto_gqa_decode_launch(const PtoTensorDesc* tensors, uint32_t n_tensors, const PtoGqaParams* params, void* workspace,
                           uint64_t workspace_bytes, void* hip_stream);
 
+/* Scalar arguments of lightning_indexer_prolog_quant: attrs.eps of the LayerNorm
+ * (models/deepseek_v32_exp/lightning_indexer_prolog_quant_impl.py:84-88; the layout strings are fixed "TND" / "PA_BSND",
+ * the configs argument holds Ascend tiling knobs). */
+typedef struct {
+    float eps;
+} PtoIndexerPrologParams;
+
+/*
+ * lightning_indexer_prolog_quant (models/deepseek_v32_exp/lightning_indexer_prolog_quant_impl.py:203-243; tensors in the
+ * order of IndexerPrologQuantInput :63-80 followed by IndexerPrologQuantOutput :83-89).  tensors[21], in order:
+ *    0 x              [t, h]                 BF16   (h a multiple of 256)
+ *    1 q_norm         [t, r]                 INT8   (r a multiple of 64)
+ *    2 q_norm_scale   [t, 1]                 FP32
+ *    3 w_qb           [r, n*128]             INT8   (plain row-major; the reference's Ascend NZ tiling is a device format)
+ *    4 w_qb_scale     [n*128, 1]             FP32
+ *    5 wk             [h, 128]               BF16
+ *    6 w_proj         [h, n]                 BF16   (n a multiple of 32, at most 128)
+ *    7 ln_gamma_k     [128]                  BF16
+ *    8 ln_beta_k      [128]                  BF16
+ *    9 cos_idx_rope   [t, 64]                BF16
+ *   10 sin_idx_rope   [t, 64]                BF16
+ *   11 hadamard_q     [128, 128]             BF16
+ *   12 hadamard_k     [128, 128]             BF16
+ *   13 k_cache        [blocks, bs, 1, 128]   INT8   (updated in place at the rows k_cache_index names)
+ *   14 k_cache_scale  [blocks, bs, 1, 1]     FP16   (updated in place)
+ *   15 k_cache_index  [t]                    INT64  (cache row of each token; rows outside the cache are skipped)
+ *   16 q_int8         [t, n, 128]            INT8   (output)
+ *   17 q_scale        [t, n, 1]              FP16   (output)
+ *   18 k_int8         = tensor 13 (the reference passes the cache again as the output; it must be the same buffer)
+ *   19 k_scale        = tensor 14
+ *   20 weights        [t, n]                 FP16   (output)
+ */
+uint64_t pto_indexer_prolog_workspace(const PtoTensorDesc* tensors, uint32_t n_tensors,
+                                      const PtoIndexerPrologParams* params);
+int pto_indexer_prolog_launch(const PtoTensorDesc* tensors, uint32_t n_tensors, const PtoIndexerPrologParams* params,
+                              void* workspace, uint64_t workspace_bytes, void* hip_stream);
+
 /* Message of the calling thread's most recent failed call ("" if none).  Replaces the message strings
  * the reference's binding layer returns (python/src/bindings/runtime.cpp:270-335). */
 const char* pto_last_error(void);
@@ -180,7 +217,8 @@ const char* pto_last_error(void);
  * is bracketed by a HIP event pair recorded on the launch stream; pto_kernel_timing_read waits for the
  * events recorded so far for one kernel, returns their summed duration and count, and forgets them.
  * Kernel ids: 0 indexer_score_kernel, 1 indexer_topk_kernel, 2 sfa_decode_kernel, 3 sfa_combine_kernel,
- * 4 indexer_select_kernel, 5 select_experts_kernel, 6 gqa_decode_kernel, 7 gqa_combine_kernel
+ * 4 indexer_select_kernel, 5 select_experts_kernel, 6 gqa_decode_kernel, 7 gqa_combine_kernel, 8 prolog_transpose_kernel,
+ * 9 prolog_q_kernel, 10 prolog_xw_kernel, 11 prolog_k_kernel
  * (pto_kernel_name returns "" past the last id).
  * Off by default; not for use under graph capture.
  */

@@ -43,10 +43,14 @@ class SelectExpertsParams(ctypes.Structure):
 
 
 # framework/include/tilefwk/data_type.h:33-65
-_DTYPE_CODE = {torch.int8: 1, torch.int32: 3, torch.float16: 6, torch.float32: 7, torch.bfloat16: 8}
+_DTYPE_CODE = {torch.int8: 1, torch.int32: 3, torch.int64: 4, torch.float16: 6, torch.float32: 7, torch.bfloat16: 8}
 
 class GqaParams(ctypes.Structure):
     _fields_ = [("softmax_scale", ctypes.c_float), ("kv_chunk", ctypes.c_int32)]
+
+
+class IndexerPrologParams(ctypes.Structure):
+    _fields_ = [("eps", ctypes.c_float)]
 
 
 _OPS = {
@@ -55,6 +59,7 @@ _OPS = {
     "lightning_indexer": IndexerParams,
     "select_experts": SelectExpertsParams,
     "gqa_decode": GqaParams,
+    "indexer_prolog": IndexerPrologParams,
 }
 
 # C status -> Python exception type wrapped by FeError

@@ -32,6 +32,7 @@ const char* dtype_name(int dt)
     switch (dt) {
         case PTO_DT_INT8: return "int8";
         case PTO_DT_INT32: return "int32";
+        case PTO_DT_INT64: return "int64";
         case PTO_DT_FP16: return "fp16";
         case PTO_DT_FP32: return "fp32";
         case PTO_DT_BF16: return "bf16";
@@ -355,9 +356,106 @@ int plan_gqa(const PtoTensorDesc* ts, uint32_t n, const PtoGqaParams* p, GqaPlan
     return PTO_OK;
 }
 
+struct PrologPlan {
+    pto::PrologArgs args;
+    uint64_t ws_bytes;
+};
+
+int plan_prolog(const PtoTensorDesc* ts, uint32_t n, const PtoIndexerPrologParams* p, PrologPlan* plan)
+{
+    const char* op = "lightning_indexer_prolog_quant";
+    if (ts == nullptr || n != 21) return fail(PTO_ERR_ARG_COUNT, "%s: expected 21 tensors, got %u", op, n);
+    if (p == nullptr) return fail(PTO_ERR_PARAM, "%s: params is null", op);
+    static const struct { const char* name; int dtype; int rank; } spec[21] = {
+        {"x", PTO_DT_BF16, 2}, {"q_norm", PTO_DT_INT8, 2}, {"q_norm_scale", PTO_DT_FP32, 2}, {"w_qb", PTO_DT_INT8, 2},
+        {"w_qb_scale", PTO_DT_FP32, 2}, {"wk", PTO_DT_BF16, 2}, {"w_proj", PTO_DT_BF16, 2}, {"ln_gamma_k", PTO_DT_BF16, 1},
+        {"ln_beta_k", PTO_DT_BF16, 1}, {"cos_idx_rope", PTO_DT_BF16, 2}, {"sin_idx_rope", PTO_DT_BF16, 2},
+        {"hadamard_q", PTO_DT_BF16, 2}, {"hadamard_k", PTO_DT_BF16, 2}, {"k_cache", PTO_DT_INT8, 4},
+        {"k_cache_scale", PTO_DT_FP16, 4}, {"k_cache_index", PTO_DT_INT64, 1}, {"q_int8", PTO_DT_INT8, 3},
+        {"q_scale", PTO_DT_FP16, 3}, {"k_int8", PTO_DT_INT8, 4}, {"k_scale", PTO_DT_FP16, 4}, {"weights", PTO_DT_FP16, 2}};
+    int rc;
+    for (int i = 0; i < 21; ++i)
+        if ((rc = check_tensor(op, ts[i], spec[i].name, spec[i].dtype, spec[i].rank))) return rc;
+    if (!(p->eps >= 0.f)) return fail(PTO_ERR_PARAM, "%s: eps must be non-negative", op);
+    const int64_t t = ts[0].shape[0], h = ts[0].shape[1], r = ts[1].shape[1], nd = ts[3].shape[1];
+    const int64_t d = ts[11].shape[0], rope = ts[9].shape[1], nh = ts[6].shape[1];
+    if (d != 128 || nd != nh * d || !pto::prolog_supported(h, r, nh, d, rope))
+        return fail(PTO_ERR_SHAPE, "%s: need head dim 128, rotary dim 64, heads a multiple of 32 (at most 128), w_qb [r, heads*128] with r a multiple of 64 and h a multiple of 256; got h %lld r %lld heads %lld dim %lld rotary %lld w_qb cols %lld",
+                    op, (long long)h, (long long)r, (long long)nh, (long long)d, (long long)rope, (long long)nd);
+    const bool ok = ts[1].shape[0] == t && ts[2].shape[0] == t && ts[2].shape[1] == 1 && ts[3].shape[0] == r &&
+                    ts[4].shape[0] == nd && ts[4].shape[1] == 1 && ts[5].shape[0] == h && ts[5].shape[1] == d &&
+                    ts[6].shape[0] == h && ts[7].shape[0] == d && ts[8].shape[0] == d && ts[9].shape[0] == t &&
+                    ts[10].shape[0] == t && ts[10].shape[1] == rope && ts[11].shape[1] == d && ts[12].shape[0] == d &&
+                    ts[12].shape[1] == d && ts[13].shape[2] == 1 && ts[13].shape[3] == d &&
+                    ts[14].shape[0] == ts[13].shape[0] && ts[14].shape[1] == ts[13].shape[1] && ts[14].shape[2] == 1 &&
+                    ts[14].shape[3] == 1 && ts[15].shape[0] == t && ts[16].shape[0] == t && ts[16].shape[1] == nh &&
+                    ts[16].shape[2] == d && ts[17].shape[0] == t && ts[17].shape[1] == nh && ts[17].shape[2] == 1 &&
+                    ts[20].shape[0] == t && ts[20].shape[1] == nh;
+    if (!ok) return fail(PTO_ERR_SHAPE, "%s: operand shapes do not fit together (t %lld, h %lld, r %lld, heads %lld)", op, (long long)t, (long long)h, (long long)r, (long long)nh);
+    if (ts[18].addr != ts[13].addr || ts[19].addr != ts[14].addr)
+        return fail(PTO_ERR_PARAM, "%s: k_int8 / k_scale must be the k_cache / k_cache_scale buffers (the cache is updated in place)", op);
+    if (t > 0x7fffffff / 256) return fail(PTO_ERR_SHAPE, "%s: too many tokens", op);
+    pto::PrologArgs& a = plan->args;
+    a.x = static_cast<const uint16_t*>(ts[0].addr);
+    a.q_norm = static_cast<const int8_t*>(ts[1].addr);
+    a.q_norm_scale = static_cast<const float*>(ts[2].addr);
+    a.w_qb = static_cast<const int8_t*>(ts[3].addr);
+    a.w_qb_scale = static_cast<const float*>(ts[4].addr);
+    a.w_k = static_cast<const uint16_t*>(ts[5].addr);
+    a.w_proj = static_cast<const uint16_t*>(ts[6].addr);
+    a.ln_gamma = static_cast<const uint16_t*>(ts[7].addr);
+    a.ln_beta = static_cast<const uint16_t*>(ts[8].addr);
+    a.cos = static_cast<const uint16_t*>(ts[9].addr);
+    a.sin = static_cast<const uint16_t*>(ts[10].addr);
+    a.had_q = static_cast<const uint16_t*>(ts[11].addr);
+    a.had_k = static_cast<const uint16_t*>(ts[12].addr);
+    a.k_cache = static_cast<int8_t*>(ts[13].addr);
+    a.k_scale_cache = static_cast<uint16_t*>(ts[14].addr);
+    a.k_cache_index = static_cast<const int64_t*>(ts[15].addr);
+    a.q_int8 = static_cast<int8_t*>(ts[16].addr);
+    a.q_scale = static_cast<uint16_t*>(ts[17].addr);
+    a.weights = static_cast<uint16_t*>(ts[20].addr);
+    a.w_qb_t = nullptr;
+    a.xw_part = nullptr;
+    a.cache_rows = ts[13].shape[0] * ts[13].shape[1];
+    a.t = (int32_t)t;
+    a.h = (int32_t)h;
+    a.r = (int32_t)r;
+    a.n = (int32_t)nh;
+    a.ksplits = (int32_t)(h / 256);
+    a.eps = p->eps;
+    a.wscale_n = (float)(1.0 / __builtin_sqrt((double)nh));
+    a.wscale_d = (float)(1.0 / __builtin_sqrt((double)d));
+    plan->ws_bytes = pto::prolog_workspace_bytes(t, h, r, nh);
+    return PTO_OK;
+}
+
 } // namespace
 
 extern "C" {
+
+uint64_t pto_indexer_prolog_workspace(const PtoTensorDesc* tensors, uint32_t n_tensors,
+                                      const PtoIndexerPrologParams* params)
+{
+    PrologPlan plan;
+    return plan_prolog(tensors, n_tensors, params, &plan) == PTO_OK ? plan.ws_bytes : 0;
+}
+
+int pto_indexer_prolog_launch(const PtoTensorDesc* tensors, uint32_t n_tensors, const PtoIndexerPrologParams* params,
+                              void* workspace, uint64_t workspace_bytes, void* hip_stream)
+{
+    const char* op = "lightning_indexer_prolog_quant";
+    PrologPlan plan;
+    int rc = plan_prolog(tensors, n_tensors, params, &plan);
+    if (rc) return rc;
+    if (workspace == nullptr || workspace_bytes < plan.ws_bytes)
+        return fail(PTO_ERR_WORKSPACE, "%s: workspace of %llu bytes required, got %llu", op,
+                    (unsigned long long)plan.ws_bytes, (unsigned long long)(workspace ? workspace_bytes : 0));
+    pto::prolog_bind_workspace(plan.args, workspace);
+    hipError_t e = pto::prolog_launch(plan.args, static_cast<hipStream_t>(hip_stream));
+    if (e != hipSuccess) return fail(PTO_ERR_HIP, "%s: HIP launch failed: %s", op, hipGetErrorString(e));
+    return PTO_OK;
+}
 
 uint64_t pto_gqa_decode_workspace(const PtoTensorDesc* tensors, uint32_t n_tensors, const PtoGqaParams* params)
 {
@@ -479,7 +577,8 @@ const char* pto_kernel_name(int kernel_id)
 {
     static const char* names[] = {"indexer_score_kernel", "indexer_topk_kernel", "sfa_decode_kernel",
                                   "sfa_combine_kernel", "indexer_select_kernel", "select_experts_kernel",
-                                  "gqa_decode_kernel", "gqa_combine_kernel"};
+                                  "gqa_decode_kernel", "gqa_combine_kernel", "prolog_transpose_kernel", "prolog_q_kernel",
+                                  "prolog_xw_kernel", "prolog_k_kernel"};
     return kernel_id >= 0 && kernel_id < pto::KID_COUNT ? names[kernel_id] : "";
 }
 

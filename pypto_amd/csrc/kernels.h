@@ -90,4 +90,37 @@ void gqa_pick_chunk(int max_ctx, int forced_chunk, int* chunk, int* nsplit);
 uint64_t gqa_workspace_bytes(int64_t t, int nq, int nsplit);
 hipError_t gqa_launch(const GqaArgs& a, hipStream_t stream);
 
+// ---------------------------------------------------------------- lightning indexer prolog
+struct PrologArgs {
+    const uint16_t* x;         // [t, h] bf16
+    const int8_t* q_norm;      // [t, r]
+    const float* q_norm_scale; // [t]
+    const int8_t* w_qb;        // [r, n*128]
+    const float* w_qb_scale;   // [n*128]
+    const uint16_t* w_k;       // [h, 128] bf16
+    const uint16_t* w_proj;    // [h, n] bf16
+    const uint16_t* ln_gamma;  // [128] bf16
+    const uint16_t* ln_beta;   // [128] bf16
+    const uint16_t* cos;       // [t, 64] bf16
+    const uint16_t* sin;       // [t, 64] bf16
+    const uint16_t* had_q;     // [128, 128] bf16
+    const uint16_t* had_k;     // [128, 128] bf16
+    int8_t* k_cache;           // [cache_rows, 128], updated in place
+    uint16_t* k_scale_cache;   // [cache_rows] fp16, updated in place
+    const int64_t* k_cache_index; // [t]
+    int8_t* q_int8;            // [t, n, 128]
+    uint16_t* q_scale;         // [t, n] fp16
+    uint16_t* weights;         // [t, n] fp16
+    int8_t* w_qb_t;            // workspace [n*128, r]
+    float* xw_part;            // workspace [ksplits, t, 128 + n]
+    int64_t cache_rows;
+    int32_t t, h, r, n, ksplits;
+    float eps, wscale_n, wscale_d;
+};
+
+bool prolog_supported(int64_t h, int64_t r, int64_t n, int64_t d, int64_t rope);
+uint64_t prolog_workspace_bytes(int64_t t, int64_t h, int64_t r, int64_t n);
+void prolog_bind_workspace(PrologArgs& a, void* workspace);
+hipError_t prolog_launch(const PrologArgs& a, hipStream_t stream);
+
 } // namespace pto

@@ -1,0 +1,399 @@
+// Lightning-indexer prolog (the producer of everything the lightning indexer reads) - gfx950 kernels.
+//
+// Replaces the device side of lightning_indexer_prolog_quant
+// (models/deepseek_v32_exp/lightning_indexer_prolog_quant_impl.py:203-543); arithmetic follows the golden
+// indexer_prolog (models/deepseek_v32_exp/deepseekv32_lightning_indexer_prolog_quant.py:209-288):
+//   query   q = bf16(int32(q_norm @ w_qb) * q_norm_scale * w_qb_scale); rotary embedding on the first 64 of each head's
+//           128 dims; q = bf16(q @ hadamard_q) (fp32 accumulate); per (token, head): s = 127 / max|q|, int8 rint(q s),
+//           dequant scale fp16(1 / s)
+//   key     k = bf16(LayerNorm(x @ w_k)); rotary; bf16(k @ hadamard_k); same quantisation; written into the paged int8
+//           index cache and its fp16 scale cache at row k_cache_index[token]
+//   weights fp16(bf16(x @ w_proj) * n^-0.5 * d^-0.5)
+//
+// At decode sizes (tens of tokens) the operator streams 15 MB of weights once and is bound by that read and by launch
+// latency, not by the matrix cores; the kernels are laid out for coalesced weight reads:
+//   prolog_transpose_kernel  w_qb [r, n d] -> [n d, r] in the workspace, so that both operands of the int8 GEMM are
+//                            contiguous along the contraction (16 bytes per lane straight into the MFMA operand layout)
+//   prolog_q_kernel          one workgroup per (head, 32 tokens): int8 MFMA GEMM over r, scale and round to bf16 into
+//                            LDS, rotary in LDS, hadamard as a bf16 MFMA (matrix read with transposing LDS reads),
+//                            quantisation
+//   prolog_xw_kernel         x @ [w_k | w_proj] split over the contraction (256 rows of the weights per workgroup, staged
+//                            in LDS and read with transposing reads); fp32 partials to the workspace
+//   prolog_k_kernel          one workgroup per token: sums the partials in a fixed order, LayerNorm, rotary, hadamard,
+//                            quantisation, cache write, weights
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "common.h"
+#include "kernels.h"
+#include "timing.h"
+
+namespace pto {
+namespace {
+
+constexpr int PD = 128;      // index head dim
+constexpr int PROPE = 64;    // rotary dims
+constexpr int PTOK = 32;     // tokens per workgroup tile
+constexpr int XW_K = 256;    // contraction rows per workgroup of prolog_xw_kernel
+constexpr int XROW = PD * 2 + 16; // bytes per LDS row of the 32 x 128 bf16 tile (padded)
+
+typedef short s16x4 __attribute__((ext_vector_type(4)));
+typedef short s16x8 __attribute__((ext_vector_type(8)));
+typedef __attribute__((address_space(3))) s16x4 lds_s16x4;
+__device__ __forceinline__ s16x4 lds_read_tr(const uint8_t* p)
+{
+    return __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)const_cast<uint8_t*>(p));
+}
+__device__ __forceinline__ float bf16_to_f32(uint16_t v) { return __builtin_bit_cast(float, (uint32_t)v << 16); }
+__device__ __forceinline__ uint16_t f32_to_bf16(float f)
+{
+    return __builtin_bit_cast(uint16_t, (__bf16)f);
+}
+
+// ------------------------------------------------------------------------------------------------ transpose
+__global__ __launch_bounds__(256) void prolog_transpose_kernel(const int8_t* __restrict__ w, int8_t* __restrict__ wt,
+                                                               int r, int nd)
+{
+    __shared__ uint8_t tile[64][68];
+    const int n0 = blockIdx.x * 64, r0 = blockIdx.y * 64;
+    const int tx = threadIdx.x & 15, ty = threadIdx.x >> 4;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const int row = ty + 16 * i;
+        const uint32_t v = *reinterpret_cast<const uint32_t*>(w + (int64_t)(r0 + row) * nd + n0 + 4 * tx);
+        *reinterpret_cast<uint32_t*>(&tile[row][4 * tx]) = v;
+    }
+    __syncthreads();
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const int nn = ty + 16 * i;
+        const uint32_t v = (uint32_t)tile[4 * tx][nn] | ((uint32_t)tile[4 * tx + 1][nn] << 8) |
+                           ((uint32_t)tile[4 * tx + 2][nn] << 16) | ((uint32_t)tile[4 * tx + 3][nn] << 24);
+        *reinterpret_cast<uint32_t*>(wt + (int64_t)(n0 + nn) * r + r0 + 4 * tx) = v;
+    }
+}
+
+// Rotary embedding of the first 64 dims of the 32 x 128 bf16 tile in LDS, fp32 arithmetic with every product and sum
+// rounded (the golden's x * cos + rotate_half(x) * sin), back to bf16.  256 lanes: 4 (token, pair) items each.
+__device__ __forceinline__ void rope_tile(uint8_t* xt, const uint16_t* cosp, const uint16_t* sinp, int tok0, int t, int tid)
+{
+#pragma clang fp contract(off)
+#pragma unroll
+    for (int it = 0; it < 4; ++it) {
+        const int item = tid + 256 * it;
+        const int tok = item >> 5, i = item & 31;
+        const int gt = min(tok0 + tok, t - 1);
+        uint16_t* row = reinterpret_cast<uint16_t*>(xt + tok * XROW);
+        const float x1 = bf16_to_f32(row[i]), x2 = bf16_to_f32(row[i + 32]);
+        const float c1 = bf16_to_f32(cosp[(int64_t)gt * PROPE + i]), c2 = bf16_to_f32(cosp[(int64_t)gt * PROPE + i + 32]);
+        const float s1 = bf16_to_f32(sinp[(int64_t)gt * PROPE + i]), s2 = bf16_to_f32(sinp[(int64_t)gt * PROPE + i + 32]);
+        const float o1 = x1 * c1 + (-x2) * s1;
+        const float o2 = x2 * c2 + x1 * s2;
+        row[i] = f32_to_bf16(o1);
+        row[i + 32] = f32_to_bf16(o2);
+    }
+}
+
+// ------------------------------------------------------------------------------------------------ query path
+// grid (heads, token tiles of 32), 256 lanes
+__global__ __launch_bounds__(256) void prolog_q_kernel(PrologArgs a)
+{
+    __shared__ __align__(16) uint8_t had[PD * PD * 2]; // hadamard_q, row-major [k][n] bf16
+    __shared__ __align__(16) uint8_t xt[PTOK * XROW];  // the head's tile [token][dim] bf16
+    __shared__ float smax[4][PTOK];
+
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int l16 = lane & 15, g = lane >> 4, l32 = lane & 31, hl = lane >> 5;
+    const int head = blockIdx.x, tok0 = blockIdx.y * PTOK;
+    const int r = a.r;
+
+    for (int i = tid; i < PD * PD * 2 / 16; i += 256)
+        reinterpret_cast<u32x4*>(had)[i] = reinterpret_cast<const u32x4*>(a.had_q)[i];
+
+    // C^T[dim, token] = Wt[dim, :] . q_norm[token, :]: wave w owns dims [32 w, 32 w + 32) x 32 tokens
+    i32x4 acc[2][2];
+#pragma unroll
+    for (int db = 0; db < 2; ++db)
+#pragma unroll
+        for (int tb = 0; tb < 2; ++tb) acc[db][tb] = i32x4{0, 0, 0, 0};
+    const int8_t* wrow[2];
+    const int8_t* qrow[2];
+#pragma unroll
+    for (int db = 0; db < 2; ++db) wrow[db] = a.w_qb_t + ((int64_t)head * PD + 32 * wave + 16 * db + l16) * r + 16 * g;
+#pragma unroll
+    for (int tb = 0; tb < 2; ++tb) qrow[tb] = a.q_norm + (int64_t)min(tok0 + 16 * tb + l16, a.t - 1) * r + 16 * g;
+    for (int k0 = 0; k0 < r; k0 += 64) {
+        i32x4 wf[2], qf[2];
+#pragma unroll
+        for (int db = 0; db < 2; ++db) wf[db] = *reinterpret_cast<const i32x4*>(wrow[db] + k0);
+#pragma unroll
+        for (int tb = 0; tb < 2; ++tb) qf[tb] = *reinterpret_cast<const i32x4*>(qrow[tb] + k0);
+#pragma unroll
+        for (int db = 0; db < 2; ++db)
+#pragma unroll
+            for (int tb = 0; tb < 2; ++tb)
+                acc[db][tb] = __builtin_amdgcn_mfma_i32_16x16x64_i8(wf[db], qf[tb], acc[db][tb], 0, 0, 0);
+    }
+    // register e of acc[db][tb]: dim 32 w + 16 db + 4 g + e, token 16 tb + l16
+    {
+#pragma clang fp contract(off)
+#pragma unroll
+        for (int tb = 0; tb < 2; ++tb) {
+            const int tok = 16 * tb + l16;
+            const float qs = a.q_norm_scale[min(tok0 + tok, a.t - 1)];
+#pragma unroll
+            for (int db = 0; db < 2; ++db) {
+                const int dim = 32 * wave + 16 * db + 4 * g;
+                const f32x4 ws = *reinterpret_cast<const f32x4*>(a.w_qb_scale + (int64_t)head * PD + dim);
+                uint16_t* dst = reinterpret_cast<uint16_t*>(xt + tok * XROW) + dim;
+#pragma unroll
+                for (int e = 0; e < 4; ++e) dst[e] = f32_to_bf16(((float)acc[db][tb][e] * qs) * ws[e]);
+            }
+        }
+    }
+    __syncthreads();
+    rope_tile(xt, a.cos, a.sin, tok0, a.t, tid);
+    __syncthreads();
+
+    // Y^T[n, token] = H^T[n, k] . X^T[k, token]: wave w owns n in [32 w, 32 w + 32).  A (H^T) by transposing reads of
+    // the row-major H: lane jj of 16-lane group G points at row k0 + 4*hl + jj/4 (+ 8), columns 32 w + 16 (G&1) + 4 (jj&3)
+    f32x16 y;
+#pragma unroll
+    for (int e = 0; e < 16; ++e) y[e] = 0.f;
+    {
+        const int jj = lane & 15, mh = (lane >> 4) & 1;
+        const uint8_t* hp = had + (4 * hl + (jj >> 2)) * (PD * 2) + (32 * wave + 16 * mh + 4 * (jj & 3)) * 2;
+        // the transposing reads hand lane half hl the contraction rows {4 hl .. 4 hl + 3} and {8 + 4 hl .. 8 + 4 hl + 3} of
+        // a 16-row step, so the B operand takes the same rows of X: two 8-byte pieces
+        const uint8_t* xp = xt + l32 * XROW + hl * 8;
+#pragma unroll
+        for (int ks = 0; ks < PD / 16; ++ks) {
+            const s16x4 lo = lds_read_tr(hp + ks * 16 * (PD * 2));
+            const s16x4 hi = lds_read_tr(hp + (ks * 16 + 8) * (PD * 2));
+            const bf16x8 av = __builtin_bit_cast(bf16x8, __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
+            const u32x2 b0 = *reinterpret_cast<const u32x2*>(xp + ks * 32);
+            const u32x2 b1 = *reinterpret_cast<const u32x2*>(xp + ks * 32 + 16);
+            const bf16x8 bv = __builtin_bit_cast(bf16x8, u32x4{b0[0], b0[1], b1[0], b1[1]});
+            y = __builtin_amdgcn_mfma_f32_32x32x16_bf16(av, bv, y, 0, 0, 0);
+        }
+    }
+    // register e: n = 32 w + 8 (e/4) + 4 hl + e%4, token l32.  Round to bf16, then per-token absmax over the 128 n
+    float yb[16], mx = 0.f;
+#pragma unroll
+    for (int e = 0; e < 16; ++e) {
+        yb[e] = bf16_to_f32(f32_to_bf16(y[e]));
+        mx = fmaxf(mx, fabsf(yb[e]));
+    }
+    mx = fmaxf(mx, __shfl_xor(mx, 32));
+    if (hl == 0) smax[wave][l32] = mx;
+    __syncthreads();
+    mx = fmaxf(fmaxf(smax[0][l32], smax[1][l32]), fmaxf(smax[2][l32], smax[3][l32]));
+    const float sq = 127.0f / mx;
+    const int gt = tok0 + l32;
+    if (gt < a.t) {
+        int8_t* qo = a.q_int8 + ((int64_t)gt * a.n + head) * PD + 32 * wave + 4 * hl;
+#pragma unroll
+        for (int e4 = 0; e4 < 4; ++e4) {
+            uint32_t pk = 0;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) pk |= ((uint32_t)(int)__builtin_rintf(yb[4 * e4 + e] * sq) & 0xffu) << (8 * e);
+            *reinterpret_cast<uint32_t*>(qo + 8 * e4) = pk;
+        }
+        if (wave == 0 && hl == 0)
+            a.q_scale[(int64_t)gt * a.n + head] = __builtin_bit_cast(uint16_t, (_Float16)(1.0f / sq));
+    }
+}
+
+// ------------------------------------------------------------------------------------------------ x @ [w_k | w_proj]
+// grid (h / 256, token tiles of 32), 256 lanes; partial sums over this workgroup's 256 rows of the weights
+__global__ __launch_bounds__(256) void prolog_xw_kernel(PrologArgs a)
+{
+    extern __shared__ __align__(16) uint8_t wl[]; // [256 k][nw] bf16, nw = 128 + n
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int l32 = lane & 31, hl = lane >> 5;
+    const int split = blockIdx.x, tok0 = blockIdx.y * PTOK;
+    const int nw = PD + a.n, rowb = nw * 2;
+    const int64_t kbase = (int64_t)split * XW_K;
+    // stage the weights: w_k rows then w_proj rows, 16-byte pieces
+    for (int i = tid; i < XW_K * (PD / 8); i += 256) {
+        const int k = i / (PD / 8), c = i % (PD / 8);
+        *reinterpret_cast<u32x4*>(wl + k * rowb + c * 16) =
+            *reinterpret_cast<const u32x4*>(a.w_k + (kbase + k) * PD + c * 8);
+    }
+    for (int i = tid; i < XW_K * (a.n / 8); i += 256) {
+        const int k = i / (a.n / 8), c = i % (a.n / 8);
+        *reinterpret_cast<u32x4*>(wl + k * rowb + PD * 2 + c * 16) =
+            *reinterpret_cast<const u32x4*>(a.w_proj + (kbase + k) * a.n + c * 8);
+    }
+    __syncthreads();
+    const int nblocks = nw / 32; // 32-wide output blocks; wave w takes blocks w, w + 4
+    const int jj = lane & 15, mh = (lane >> 4) & 1;
+    // B operand rows as the transposing reads order them: {4 hl .. + 3} and {8 + 4 hl .. + 3} of every 16-row step
+    const uint16_t* xp = a.x + (int64_t)min(tok0 + l32, a.t - 1) * a.h + kbase + hl * 4;
+    f32x16 acc[2];
+#pragma unroll
+    for (int j = 0; j < 2; ++j)
+#pragma unroll
+        for (int e = 0; e < 16; ++e) acc[j][e] = 0.f;
+    for (int ks = 0; ks < XW_K / 16; ++ks) {
+        const u32x2 b0 = *reinterpret_cast<const u32x2*>(xp + ks * 16);
+        const u32x2 b1 = *reinterpret_cast<const u32x2*>(xp + ks * 16 + 8);
+        const bf16x8 bv = __builtin_bit_cast(bf16x8, u32x4{b0[0], b0[1], b1[0], b1[1]});
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+            const int nb = wave + 4 * j;
+            if (nb < nblocks) {
+                const uint8_t* hp = wl + (ks * 16 + 4 * hl + (jj >> 2)) * rowb + (32 * nb + 16 * mh + 4 * (jj & 3)) * 2;
+                const s16x4 lo = lds_read_tr(hp);
+                const s16x4 hi = lds_read_tr(hp + 8 * rowb);
+                const bf16x8 av = __builtin_bit_cast(bf16x8, __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
+                acc[j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(av, bv, acc[j], 0, 0, 0);
+            }
+        }
+    }
+    // register e of block nb: output 32 nb + 8 (e/4) + 4 hl + e%4, token l32
+    const int gt = tok0 + l32;
+    if (gt < a.t) {
+        float* out = a.xw_part + ((int64_t)split * a.t + gt) * nw;
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+            const int nb = wave + 4 * j;
+            if (nb < nblocks)
+#pragma unroll
+                for (int e4 = 0; e4 < 4; ++e4)
+                    *reinterpret_cast<f32x4*>(out + 32 * nb + 8 * e4 + 4 * hl) =
+                        f32x4{acc[j][4 * e4], acc[j][4 * e4 + 1], acc[j][4 * e4 + 2], acc[j][4 * e4 + 3]};
+        }
+    }
+}
+
+// ------------------------------------------------------------------------------------------------ key path, weights
+__device__ __forceinline__ float block_sum128(float v, float* red)
+{
+#pragma unroll
+    for (int d = 1; d < 64; d <<= 1) v += __shfl_xor(v, d);
+    __syncthreads();
+    if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = v;
+    __syncthreads();
+    return red[0] + red[1];
+}
+__device__ __forceinline__ float block_max128(float v, float* red)
+{
+#pragma unroll
+    for (int d = 1; d < 64; d <<= 1) v = fmaxf(v, __shfl_xor(v, d));
+    __syncthreads();
+    if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = v;
+    __syncthreads();
+    return fmaxf(red[0], red[1]);
+}
+
+// grid (tokens), 128 lanes: lane = output dim
+__global__ __launch_bounds__(128) void prolog_k_kernel(PrologArgs a)
+{
+#pragma clang fp contract(off)
+    __shared__ float red[2];
+    __shared__ float kb[PD];
+    const int tid = threadIdx.x, tok = blockIdx.x;
+    const int nw = PD + a.n;
+    float kv = 0.f, wv = 0.f;
+    for (int s = 0; s < a.ksplits; ++s) {
+        const float* p = a.xw_part + ((int64_t)s * a.t + tok) * nw;
+        kv += p[tid];
+        if (tid < a.n) wv += p[PD + tid];
+    }
+    // LayerNorm in fp32 (biased variance), -> bf16
+    const float mean = block_sum128(kv, red) / (float)PD;
+    const float dlt = kv - mean;
+    const float var = block_sum128(dlt * dlt, red) / (float)PD;
+    float xn = dlt / sqrtf(var + a.eps);
+    xn = xn * bf16_to_f32(a.ln_gamma[tid]) + bf16_to_f32(a.ln_beta[tid]);
+    kb[tid] = bf16_to_f32(f32_to_bf16(xn));
+    __syncthreads();
+    // rotary on the first 64 dims
+    float kr = kb[tid];
+    if (tid < PROPE) {
+        const float c = bf16_to_f32(a.cos[(int64_t)tok * PROPE + tid]), s = bf16_to_f32(a.sin[(int64_t)tok * PROPE + tid]);
+        const float other = tid < 32 ? -kb[tid + 32] : kb[tid - 32];
+        kr = bf16_to_f32(f32_to_bf16(kb[tid] * c + other * s));
+    }
+    __syncthreads();
+    kb[tid] = kr;
+    __syncthreads();
+    // hadamard: y[n] = sum_k kr[k] H[k][n], fp32, -> bf16
+    float y = 0.f;
+    for (int k = 0; k < PD; ++k) y = __builtin_fmaf(kb[k], bf16_to_f32(a.had_k[k * PD + tid]), y);
+    y = bf16_to_f32(f32_to_bf16(y));
+    const float mx = block_max128(fabsf(y), red);
+    const float sq = 127.0f / mx;
+    const int64_t row = a.k_cache_index[tok];
+    if (row >= 0 && row < a.cache_rows) {
+        a.k_cache[row * PD + tid] = (int8_t)(int)__builtin_rintf(y * sq);
+        if (tid == 0) a.k_scale_cache[row] = __builtin_bit_cast(uint16_t, (_Float16)(1.0f / sq));
+    }
+    if (tid < a.n) {
+        const float w = bf16_to_f32(f32_to_bf16(wv));
+        a.weights[(int64_t)tok * a.n + tid] = __builtin_bit_cast(uint16_t, (_Float16)((w * a.wscale_n) * a.wscale_d));
+    }
+}
+
+} // namespace
+
+bool prolog_supported(int64_t h, int64_t r, int64_t n, int64_t d, int64_t rope)
+{
+    return d == PD && rope == PROPE && n > 0 && n % 32 == 0 && n <= 128 && r > 0 && r % 64 == 0 && h > 0 && h % XW_K == 0;
+}
+
+uint64_t prolog_workspace_bytes(int64_t t, int64_t h, int64_t r, int64_t n)
+{
+    const uint64_t wt = (uint64_t)r * n * PD;
+    const uint64_t part = (uint64_t)(h / XW_K) * t * (PD + n) * sizeof(float);
+    return ((wt + 255) & ~(uint64_t)255) + part;
+}
+
+void prolog_bind_workspace(PrologArgs& a, void* ws)
+{
+    uint8_t* p = static_cast<uint8_t*>(ws);
+    a.w_qb_t = reinterpret_cast<int8_t*>(p);
+    p += ((uint64_t)a.r * a.n * PD + 255) & ~(uint64_t)255;
+    a.xw_part = reinterpret_cast<float*>(p);
+}
+
+hipError_t prolog_launch(const PrologArgs& a, hipStream_t stream)
+{
+    if (a.t == 0) return hipSuccess;
+    const int nd = a.n * PD;
+    const int ttiles = (a.t + PTOK - 1) / PTOK;
+    {
+        ScopedKernelTimer tm(KID_PROLOG_TRANSPOSE, stream);
+        hipLaunchKernelGGL(prolog_transpose_kernel, dim3(nd / 64, a.r / 64), dim3(256), 0, stream, a.w_qb, a.w_qb_t, a.r, nd);
+    }
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) return e;
+    {
+        ScopedKernelTimer tm(KID_PROLOG_Q, stream);
+        hipLaunchKernelGGL(prolog_q_kernel, dim3(a.n, ttiles), dim3(256), 0, stream, a);
+    }
+    e = hipGetLastError();
+    if (e != hipSuccess) return e;
+    {
+        const int smem = XW_K * (PD + a.n) * 2;
+        static bool attr_done = false;
+        if (!attr_done) {
+            e = hipFuncSetAttribute(reinterpret_cast<const void*>(prolog_xw_kernel),
+                                    hipFuncAttributeMaxDynamicSharedMemorySize, XW_K * (PD + 128) * 2);
+            if (e != hipSuccess) return e;
+            attr_done = true;
+        }
+        ScopedKernelTimer tm(KID_PROLOG_XW, stream);
+        hipLaunchKernelGGL(prolog_xw_kernel, dim3(a.ksplits, ttiles), dim3(256), smem, stream, a);
+    }
+    e = hipGetLastError();
+    if (e != hipSuccess) return e;
+    {
+        ScopedKernelTimer tm(KID_PROLOG_K, stream);
+        hipLaunchKernelGGL(prolog_k_kernel, dim3(a.t), dim3(128), 0, stream, a);
+    }
+    return hipGetLastError();
+}
+
+} // namespace pto

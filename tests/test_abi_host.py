@@ -58,7 +58,7 @@ def test_tensor_desc_layout_matches_the_reference_abi():
     # framework/include/tile_fwk_bundle/pypto_bundle_api.h:30-35: void* | int32 | int32 | int64[8]
     assert ctypes.sizeof(TensorDesc) == 8 + 4 + 4 + 64
     assert TensorDesc.dataType.offset == 8 and TensorDesc.rank.offset == 12 and TensorDesc.shape.offset == 16
-    assert _runtime._DTYPE_CODE == {torch.int8: 1, torch.int32: 3, torch.float16: 6, torch.float32: 7,
+    assert _runtime._DTYPE_CODE == {torch.int8: 1, torch.int32: 3, torch.int64: 4, torch.float16: 6, torch.float32: 7,
                                     torch.bfloat16: 8}
 
 
