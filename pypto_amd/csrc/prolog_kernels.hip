@@ -122,6 +122,7 @@ __global__ __launch_bounds__(256) void prolog_q_kernel(PrologArgs a)
     for (int db = 0; db < 2; ++db) wrow[db] = a.w_qb_t + ((int64_t)head * PD + 32 * wave + 16 * db + l16) * r + 16 * g;
 #pragma unroll
     for (int tb = 0; tb < 2; ++tb) qrow[tb] = a.q_norm + (int64_t)min(tok0 + 16 * tb + l16, a.t - 1) * r + 16 * g;
+#pragma unroll 6
     for (int k0 = 0; k0 < r; k0 += 64) {
         i32x4 wf[2], qf[2];
 #pragma unroll
@@ -215,11 +216,13 @@ __global__ __launch_bounds__(256) void prolog_xw_kernel(PrologArgs a)
     const int nw = PD + a.n, rowb = nw * 2;
     const int64_t kbase = (int64_t)split * XW_K;
     // stage the weights: w_k rows then w_proj rows, 16-byte pieces
+#pragma unroll 8
     for (int i = tid; i < XW_K * (PD / 8); i += 256) {
         const int k = i / (PD / 8), c = i % (PD / 8);
         *reinterpret_cast<u32x4*>(wl + k * rowb + c * 16) =
             *reinterpret_cast<const u32x4*>(a.w_k + (kbase + k) * PD + c * 8);
     }
+#pragma unroll 8
     for (int i = tid; i < XW_K * (a.n / 8); i += 256) {
         const int k = i / (a.n / 8), c = i % (a.n / 8);
         *reinterpret_cast<u32x4*>(wl + k * rowb + PD * 2 + c * 16) =
@@ -296,6 +299,7 @@ __global__ __launch_bounds__(128) void prolog_k_kernel(PrologArgs a)
     const int tid = threadIdx.x, tok = blockIdx.x;
     const int nw = PD + a.n;
     float kv = 0.f, wv = 0.f;
+#pragma unroll 7
     for (int s = 0; s < a.ksplits; ++s) {
         const float* p = a.xw_part + ((int64_t)s * a.t + tok) * nw;
         kv += p[tid];
@@ -321,6 +325,7 @@ __global__ __launch_bounds__(128) void prolog_k_kernel(PrologArgs a)
     __syncthreads();
     // hadamard: y[n] = sum_k kr[k] H[k][n], fp32, -> bf16
     float y = 0.f;
+#pragma unroll 16
     for (int k = 0; k < PD; ++k) y = __builtin_fmaf(kb[k], bf16_to_f32(a.had_k[k * PD + tid]), y);
     y = bf16_to_f32(f32_to_bf16(y));
     const float mx = block_max128(fabsf(y), red);
