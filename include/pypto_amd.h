@@ -207,6 +207,46 @@ uint64_t pto_indexer_prolog_workspace(const PtoTensorDesc* tensors, uint32_t n_t
 int pto_indexer_prolog_launch(const PtoTensorDesc* tensors, uint32_t n_tensors, const PtoIndexerPrologParams* params,
                               void* workspace, uint64_t workspace_bytes, void* hip_stream);
 
+/* Scalar arguments of mla_prolog_quant_d / mla_prolog_quant_p: the two RmsNorm epsilons and the cache mode
+ * (models/deepseek_v32_exp/mla_prolog_quant_impl.py:866-871; tile_config and rope_cfg hold Ascend tiling knobs). */
+#define PTO_CACHE_PA_BSND 0 /* "PA_BSND": paged caches [block_num, block_size, 1, dim] */
+typedef struct {
+    float epsilon_cq;
+    float epsilon_ckv;
+    int32_t cache_mode;
+} PtoMlaPrologParams;
+
+/*
+ * mla_prolog_quant_d and mla_prolog_quant_p, int8 form (models/deepseek_v32_exp/mla_prolog_quant_impl.py:745-951, compute
+ * :520-727; the decode and the prefill entry of the reference differ in Ascend pass options only).  tensors[21] in the
+ * reference's argument order:
+ *    0 token_x           [t, h]                  BF16   (h a multiple of 256)
+ *    1 w_dq              [h, r]                  BF16   (r a multiple of 128, at most 2048; plain row-major - the
+ *                                                        reference's Ascend NZ tiling is a device format)
+ *    2 w_uq_qr           [r, n*192]              INT8   (n even)
+ *    3 dequant_scale     [n*192, 1]              FP32
+ *    4 w_uk              [n, 128, 512]           BF16
+ *    5 w_dkv_kr          [h, 576]                BF16
+ *    6 gamma_cq          [r]                     BF16
+ *    7 gamma_ckv         [512]                   BF16
+ *    8 cos               [t, 64]                 BF16
+ *    9 sin               [t, 64]                 BF16
+ *   10 cache_index       [t]                     INT64  (flat cache row of each token; rows outside the cache are skipped)
+ *   11 kv_cache          [blocks, bs, 1, 512]    INT8   (updated in place)
+ *   12 kr_cache          [blocks, bs, 1, 64]     BF16   (updated in place)
+ *   13 k_scale_cache     [blocks, bs, 1, 4]      FP32   (updated in place)
+ *   14 q_norm_out        [t, r]                  INT8   (output)
+ *   15 q_norm_scale_out  [t, 1]                  FP32   (output)
+ *   16 query_nope_out    [t, n, 512]             BF16   (output)
+ *   17 query_rope_out    [t, n, 64]              BF16   (output)
+ *   18-20 kv_cache_out, kr_cache_out, k_scale_cache_out: the buffers of 11-13 again
+ * The bf16 form of the reference (empty dequant_scale, BF16 w_uq_qr and kv_cache) is not built and is rejected.
+ */
+uint64_t pto_mla_prolog_quant_workspace(const PtoTensorDesc* tensors, uint32_t n_tensors,
+                                        const PtoMlaPrologParams* params);
+int pto_mla_prolog_quant_launch(const PtoTensorDesc* tensors, uint32_t n_tensors, const PtoMlaPrologParams* params,
+                                void* workspace, uint64_t workspace_bytes, void* hip_stream);
+
 /* Message of the calling thread's most recent failed call ("" if none).  Replaces the message strings
  * the reference's binding layer returns (python/src/bindings/runtime.cpp:270-335). */
 const char* pto_last_error(void);
@@ -218,7 +258,8 @@ const char* pto_last_error(void);
  * events recorded so far for one kernel, returns their summed duration and count, and forgets them.
  * Kernel ids: 0 indexer_score_kernel, 1 indexer_topk_kernel, 2 sfa_decode_kernel, 3 sfa_combine_kernel,
  * 4 indexer_select_kernel, 5 select_experts_kernel, 6 gqa_decode_kernel, 7 gqa_combine_kernel, 8 prolog_transpose_kernel,
- * 9 prolog_q_kernel, 10 prolog_xw_kernel, 11 prolog_k_kernel
+ * 9 prolog_q_kernel, 10 prolog_xw_kernel, 11 prolog_k_kernel, 12 mla_xa_kernel, 13 mla_norm_kernel, 14 mla_qb_kernel,
+ * 15 mla_wuk_kernel
  * (pto_kernel_name returns "" past the last id).
  * Off by default; not for use under graph capture.
  */

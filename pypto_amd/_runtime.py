@@ -53,6 +53,10 @@ class IndexerPrologParams(ctypes.Structure):
     _fields_ = [("eps", ctypes.c_float)]
 
 
+class MlaPrologParams(ctypes.Structure):
+    _fields_ = [("epsilon_cq", ctypes.c_float), ("epsilon_ckv", ctypes.c_float), ("cache_mode", ctypes.c_int32)]
+
+
 _OPS = {
     "sfa_quant": SfaParams,
     "sfa_antiquant": SfaParams,
@@ -60,6 +64,7 @@ _OPS = {
     "select_experts": SelectExpertsParams,
     "gqa_decode": GqaParams,
     "indexer_prolog": IndexerPrologParams,
+    "mla_prolog_quant": MlaPrologParams,
 }
 
 # C status -> Python exception type wrapped by FeError

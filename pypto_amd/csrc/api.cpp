@@ -430,9 +430,109 @@ int plan_prolog(const PtoTensorDesc* ts, uint32_t n, const PtoIndexerPrologParam
     return PTO_OK;
 }
 
+struct MlaPrologPlan {
+    pto::MlaPrologArgs args;
+    uint64_t ws_bytes;
+};
+
+int plan_mla_prolog(const PtoTensorDesc* ts, uint32_t n, const PtoMlaPrologParams* p, MlaPrologPlan* plan)
+{
+    const char* op = "mla_prolog_quant";
+    if (ts == nullptr || n != 21) return fail(PTO_ERR_ARG_COUNT, "%s: expected 21 tensors, got %u", op, n);
+    if (p == nullptr) return fail(PTO_ERR_PARAM, "%s: params is null", op);
+    if (p->cache_mode != PTO_CACHE_PA_BSND)
+        return fail(PTO_ERR_PARAM, "%s: only cache mode PA_BSND (%d) is built, got %d", op, PTO_CACHE_PA_BSND, p->cache_mode);
+    if (ts[3].rank == 0 || ts[3].shape[0] == 0 || ts[2].dataType != PTO_DT_INT8)
+        return fail(PTO_ERR_DTYPE, "%s: only the int8 form (INT8 w_uq_qr with its dequant_scale, INT8 kv_cache) is built", op);
+    static const struct { const char* name; int dtype; int rank; } spec[21] = {
+        {"token_x", PTO_DT_BF16, 2}, {"w_dq", PTO_DT_BF16, 2}, {"w_uq_qr", PTO_DT_INT8, 2}, {"dequant_scale", PTO_DT_FP32, 2},
+        {"w_uk", PTO_DT_BF16, 3}, {"w_dkv_kr", PTO_DT_BF16, 2}, {"gamma_cq", PTO_DT_BF16, 1}, {"gamma_ckv", PTO_DT_BF16, 1},
+        {"cos", PTO_DT_BF16, 2}, {"sin", PTO_DT_BF16, 2}, {"cache_index", PTO_DT_INT64, 1}, {"kv_cache", PTO_DT_INT8, 4},
+        {"kr_cache", PTO_DT_BF16, 4}, {"k_scale_cache", PTO_DT_FP32, 4}, {"q_norm_out", PTO_DT_INT8, 2},
+        {"q_norm_scale_out", PTO_DT_FP32, 2}, {"query_nope_out", PTO_DT_BF16, 3}, {"query_rope_out", PTO_DT_BF16, 3},
+        {"kv_cache_out", PTO_DT_INT8, 4}, {"kr_cache_out", PTO_DT_BF16, 4}, {"k_scale_cache_out", PTO_DT_FP32, 4}};
+    int rc;
+    for (int i = 0; i < 21; ++i)
+        if ((rc = check_tensor(op, ts[i], spec[i].name, spec[i].dtype, spec[i].rank))) return rc;
+    if (!(p->epsilon_cq >= 0.f) || !(p->epsilon_ckv >= 0.f)) return fail(PTO_ERR_PARAM, "%s: epsilons must be non-negative", op);
+    const int64_t t = ts[0].shape[0], h = ts[0].shape[1], r = ts[1].shape[1];
+    const int64_t nh = ts[4].shape[0], dn = ts[4].shape[1], c = ts[4].shape[2], rope = ts[9].shape[1];
+    if (!pto::mla_prolog_supported(h, r, nh, dn, rope, c))
+        return fail(PTO_ERR_SHAPE, "%s: need w_uk [heads, 128, 512] with an even number of heads, rotary dim 64, q_lora_rank a multiple of 128 (at most 2048) and h a multiple of 256; got h %lld r %lld heads %lld nope %lld rotary %lld kv rank %lld",
+                    op, (long long)h, (long long)r, (long long)nh, (long long)dn, (long long)rope, (long long)c);
+    const int64_t nq = nh * (dn + rope);
+    const bool ok = ts[1].shape[0] == h && ts[2].shape[0] == r && ts[2].shape[1] == nq && ts[3].shape[0] == nq &&
+                    ts[3].shape[1] == 1 && ts[5].shape[0] == h && ts[5].shape[1] == c + rope && ts[6].shape[0] == r &&
+                    ts[7].shape[0] == c && ts[8].shape[0] == t && ts[8].shape[1] == rope && ts[9].shape[0] == t &&
+                    ts[10].shape[0] == t && ts[11].shape[2] == 1 && ts[11].shape[3] == c &&
+                    ts[12].shape[0] == ts[11].shape[0] && ts[12].shape[1] == ts[11].shape[1] && ts[12].shape[2] == 1 &&
+                    ts[12].shape[3] == rope && ts[13].shape[0] == ts[11].shape[0] && ts[13].shape[1] == ts[11].shape[1] &&
+                    ts[13].shape[2] == 1 && ts[13].shape[3] == 4 && ts[14].shape[0] == t && ts[14].shape[1] == r &&
+                    ts[15].shape[0] == t && ts[15].shape[1] == 1 && ts[16].shape[0] == t && ts[16].shape[1] == nh &&
+                    ts[16].shape[2] == c && ts[17].shape[0] == t && ts[17].shape[1] == nh && ts[17].shape[2] == rope;
+    if (!ok) return fail(PTO_ERR_SHAPE, "%s: operand shapes do not fit together (t %lld, h %lld, r %lld, heads %lld)", op, (long long)t, (long long)h, (long long)r, (long long)nh);
+    if (ts[18].addr != ts[11].addr || ts[19].addr != ts[12].addr || ts[20].addr != ts[13].addr)
+        return fail(PTO_ERR_PARAM, "%s: kv_cache_out / kr_cache_out / k_scale_cache_out must be the kv_cache / kr_cache / k_scale_cache buffers (the caches are updated in place)", op);
+    if (t > 0x7fffffff / 4096) return fail(PTO_ERR_SHAPE, "%s: too many tokens", op);
+    pto::MlaPrologArgs& a = plan->args;
+    a.x = static_cast<const uint16_t*>(ts[0].addr);
+    a.w_dq = static_cast<const uint16_t*>(ts[1].addr);
+    a.w_uq_qr = static_cast<const int8_t*>(ts[2].addr);
+    a.w_qb_scale = static_cast<const float*>(ts[3].addr);
+    a.w_uk = static_cast<const uint16_t*>(ts[4].addr);
+    a.w_dkv_kr = static_cast<const uint16_t*>(ts[5].addr);
+    a.gamma_cq = static_cast<const uint16_t*>(ts[6].addr);
+    a.gamma_ckv = static_cast<const uint16_t*>(ts[7].addr);
+    a.cos = static_cast<const uint16_t*>(ts[8].addr);
+    a.sin = static_cast<const uint16_t*>(ts[9].addr);
+    a.cache_index = static_cast<const int64_t*>(ts[10].addr);
+    a.kv_cache = static_cast<int8_t*>(ts[11].addr);
+    a.kr_cache = static_cast<uint16_t*>(ts[12].addr);
+    a.k_scale_cache = static_cast<float*>(ts[13].addr);
+    a.q_norm = static_cast<int8_t*>(ts[14].addr);
+    a.q_norm_scale = static_cast<float*>(ts[15].addr);
+    a.q_nope = static_cast<uint16_t*>(ts[16].addr);
+    a.q_rope = static_cast<uint16_t*>(ts[17].addr);
+    a.xa_part = nullptr;
+    a.qb_nope = nullptr;
+    a.cache_rows = ts[11].shape[0] * ts[11].shape[1];
+    a.t = (int32_t)t;
+    a.h = (int32_t)h;
+    a.r = (int32_t)r;
+    a.n = (int32_t)nh;
+    a.ksplits = (int32_t)(h / 256);
+    a.eps_cq = p->epsilon_cq;
+    a.eps_ckv = p->epsilon_ckv;
+    plan->ws_bytes = pto::mla_prolog_workspace_bytes(t, h, r, nh);
+    return PTO_OK;
+}
+
 } // namespace
 
 extern "C" {
+
+uint64_t pto_mla_prolog_quant_workspace(const PtoTensorDesc* tensors, uint32_t n_tensors, const PtoMlaPrologParams* params)
+{
+    MlaPrologPlan plan;
+    return plan_mla_prolog(tensors, n_tensors, params, &plan) == PTO_OK ? plan.ws_bytes : 0;
+}
+
+int pto_mla_prolog_quant_launch(const PtoTensorDesc* tensors, uint32_t n_tensors, const PtoMlaPrologParams* params,
+                                void* workspace, uint64_t workspace_bytes, void* hip_stream)
+{
+    const char* op = "mla_prolog_quant";
+    MlaPrologPlan plan;
+    int rc = plan_mla_prolog(tensors, n_tensors, params, &plan);
+    if (rc) return rc;
+    if (plan.args.t == 0) return PTO_OK;
+    if (workspace == nullptr || workspace_bytes < plan.ws_bytes)
+        return fail(PTO_ERR_WORKSPACE, "%s: workspace of %llu bytes required, got %llu", op,
+                    (unsigned long long)plan.ws_bytes, (unsigned long long)(workspace ? workspace_bytes : 0));
+    pto::mla_prolog_bind_workspace(plan.args, workspace);
+    hipError_t e = pto::mla_prolog_launch(plan.args, static_cast<hipStream_t>(hip_stream));
+    if (e != hipSuccess) return fail(PTO_ERR_HIP, "%s: HIP launch failed: %s", op, hipGetErrorString(e));
+    return PTO_OK;
+}
 
 uint64_t pto_indexer_prolog_workspace(const PtoTensorDesc* tensors, uint32_t n_tensors,
                                       const PtoIndexerPrologParams* params)
@@ -578,7 +678,8 @@ const char* pto_kernel_name(int kernel_id)
     static const char* names[] = {"indexer_score_kernel", "indexer_topk_kernel", "sfa_decode_kernel",
                                   "sfa_combine_kernel", "indexer_select_kernel", "select_experts_kernel",
                                   "gqa_decode_kernel", "gqa_combine_kernel", "prolog_transpose_kernel", "prolog_q_kernel",
-                                  "prolog_xw_kernel", "prolog_k_kernel"};
+                                  "prolog_xw_kernel", "prolog_k_kernel", "mla_xa_kernel", "mla_norm_kernel", "mla_qb_kernel",
+                                  "mla_wuk_kernel"};
     return kernel_id >= 0 && kernel_id < pto::KID_COUNT ? names[kernel_id] : "";
 }
 

@@ -123,4 +123,36 @@ uint64_t prolog_workspace_bytes(int64_t t, int64_t h, int64_t r, int64_t n);
 void prolog_bind_workspace(PrologArgs& a, void* workspace);
 hipError_t prolog_launch(const PrologArgs& a, hipStream_t stream);
 
+// ---------------------------------------------------------------- MLA prolog (int8 form)
+struct MlaPrologArgs {
+    const uint16_t* x;          // [t, h] bf16
+    const uint16_t* w_dq;       // [h, r] bf16
+    const int8_t* w_uq_qr;      // [r, n*192]
+    const float* w_qb_scale;    // [n*192]
+    const uint16_t* w_uk;       // [n, 128, 512] bf16
+    const uint16_t* w_dkv_kr;   // [h, 576] bf16
+    const uint16_t* gamma_cq;   // [r] bf16
+    const uint16_t* gamma_ckv;  // [512] bf16
+    const uint16_t* cos;        // [t, 64] bf16
+    const uint16_t* sin;        // [t, 64] bf16
+    const int64_t* cache_index; // [t]
+    int8_t* kv_cache;           // [cache_rows, 512], updated in place
+    uint16_t* kr_cache;         // [cache_rows, 64] bf16, updated in place
+    float* k_scale_cache;       // [cache_rows, 4], updated in place
+    int8_t* q_norm;             // [t, r]
+    float* q_norm_scale;        // [t]
+    uint16_t* q_nope;           // [t, n, 512] bf16
+    uint16_t* q_rope;           // [t, n, 64] bf16
+    float* xa_part;             // workspace [ksplits, t, r + 576]
+    uint16_t* qb_nope;          // workspace [t, n, 128] bf16
+    int64_t cache_rows;
+    int32_t t, h, r, n, ksplits;
+    float eps_cq, eps_ckv;
+};
+
+bool mla_prolog_supported(int64_t h, int64_t r, int64_t n, int64_t d_nope, int64_t d_rope, int64_t c);
+uint64_t mla_prolog_workspace_bytes(int64_t t, int64_t h, int64_t r, int64_t n);
+void mla_prolog_bind_workspace(MlaPrologArgs& a, void* workspace);
+hipError_t mla_prolog_launch(const MlaPrologArgs& a, hipStream_t stream);
+
 } // namespace pto

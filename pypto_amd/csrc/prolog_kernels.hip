@@ -45,6 +45,8 @@ __device__ __forceinline__ s16x4 lds_read_tr(const uint8_t* p)
     return __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)const_cast<uint8_t*>(p));
 }
 __device__ __forceinline__ float bf16_to_f32(uint16_t v) { return __builtin_bit_cast(float, (uint32_t)v << 16); }
+// The golden's "127 / max": torch evaluates scalar / tensor as reciprocal(tensor) * scalar, two roundings
+__device__ __forceinline__ float quant_scale(float mx) { return (1.0f / mx) * 127.0f; }
 __device__ __forceinline__ uint16_t f32_to_bf16(float f)
 {
     return __builtin_bit_cast(uint16_t, (__bf16)f);
@@ -189,7 +191,7 @@ __global__ __launch_bounds__(256) void prolog_q_kernel(PrologArgs a)
     if (hl == 0) smax[wave][l32] = mx;
     __syncthreads();
     mx = fmaxf(fmaxf(smax[0][l32], smax[1][l32]), fmaxf(smax[2][l32], smax[3][l32]));
-    const float sq = 127.0f / mx;
+    const float sq = quant_scale(mx);
     const int gt = tok0 + l32;
     if (gt < a.t) {
         int8_t* qo = a.q_int8 + ((int64_t)gt * a.n + head) * PD + 32 * wave + 4 * hl;
@@ -329,7 +331,7 @@ __global__ __launch_bounds__(128) void prolog_k_kernel(PrologArgs a)
     for (int k = 0; k < PD; ++k) y = __builtin_fmaf(kb[k], bf16_to_f32(a.had_k[k * PD + tid]), y);
     y = bf16_to_f32(f32_to_bf16(y));
     const float mx = block_max128(fabsf(y), red);
-    const float sq = 127.0f / mx;
+    const float sq = quant_scale(mx);
     const int64_t row = a.k_cache_index[tok];
     if (row >= 0 && row < a.cache_rows) {
         a.k_cache[row * PD + tid] = (int8_t)(int)__builtin_rintf(y * sq);
