@@ -48,7 +48,7 @@ def parse():
     ap.add_argument("--cpu-seqs", type=int, default=8, help="sequences of the workload timed on the CPU oracle")
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--packed", action="store_true", help="use the packed 656-byte-row attention entry point")
-    ap.add_argument("--workload", choices=["v32", "gqa", "select_experts", "indexer_prolog"], default="v32",
+    ap.add_argument("--workload", choices=["v32", "gqa", "select_experts", "indexer_prolog", "mla_prolog"], default="v32",
                     help="v32 (default): the headline DeepSeek-V3.2 indexer + sparse attention decode step; gqa: GLM-4.5 "
                          "paged GQA decode (batch 64, 96/8 heads, contexts U[4096, 32768]); select_experts: GLM-4.5 "
                          "router (8192 tokens x 160 experts)")
@@ -203,28 +203,46 @@ def bench_select_experts(args, torch, lib, dev):
     }))
 
 
+def _paged_rows(torch, dev, g, b, s2, bs):
+    """A random page table for b sequences of s2 tokens and the flat cache row of each sequence's last token."""
+    pages_per_seq = (s2 + bs - 1) // bs
+    n_pages = b * pages_per_seq
+    table = torch.randperm(n_pages, generator=g, device=dev).reshape(b, pages_per_seq)
+    pos = s2 - 1
+    rows = (table[:, pos // bs] * bs + pos % bs).to(torch.int64).contiguous()
+    return n_pages, rows
+
+
 def bench_indexer_prolog(args, torch, lib, dev):
-    """DeepSeek-V3.2 lightning-indexer prolog at decode size: 32 new tokens (batch 32, one each), h 7168, q_lora_rank
-    1536, 64 index heads x 128, a 64K-token paged index cache per sequence; the reference generator's distributions."""
+    """DeepSeek-V3.2 lightning-indexer prolog at decode size: one new token for each of `batch` sequences, h 7168,
+    q_lora_rank 1536, 64 index heads x 128, a 4K-token paged index cache per sequence; the reference generator's
+    distributions (U[-1,1), int8 tensors uniform over their range)."""
     from pypto_amd.deepseek_v32_exp import lightning_indexer_prolog_quant_impl as impl
-    sys.path.insert(0, os.path.join(ROOT, "tests"))
-    from oracle import indexer_prolog as op
-    b = args.batch
-    case = op.make_case(b, 1, 4096, seed=0)
-    d = {k: v.to(dev) for k, v in case.items()}
-    t, n = b, 64
-    tensors = [d["x"], d["q_norm"], d["q_norm_scale"], d["w_qb"], d["w_qb_scale"], d["w_k"], d["w_proj"], d["ln_gamma"],
-               d["ln_beta"], d["cos"], d["sin"], d["hadamard_q"], d["hadamard_k"], d["k_cache"], d["k_scale_cache"],
-               d["k_cache_index"], torch.zeros((t, n, 128), dtype=torch.int8, device=dev),
-               torch.zeros((t, n, 1), dtype=torch.float16, device=dev), d["k_cache"], d["k_scale_cache"],
-               torch.zeros((t, n), dtype=torch.float16, device=dev)]
+    t, n, h, r, d, bs = args.batch, 64, 7168, 1536, 128, 128
+    g = torch.Generator(device=dev).manual_seed(0)
+    bf = torch.bfloat16
+
+    def uni(*shape):
+        return torch.rand(shape, generator=g, device=dev) * 2 - 1
+
+    def i8(*shape):
+        return torch.randint(-128, 128, shape, generator=g, device=dev, dtype=torch.int8)
+
+    n_pages, rows = _paged_rows(torch, dev, g, t, 4096, bs)
+    ang = torch.rand((t, 64), generator=g, device=dev) * 6.2831853
+    k_cache, k_scale_cache = i8(n_pages, bs, 1, d), uni(n_pages, bs, 1, 1).to(torch.float16)
+    tensors = [uni(t, h).to(bf), i8(t, r), uni(t, 1), i8(r, n * d), uni(n * d, 1), uni(h, d).to(bf), uni(h, n).to(bf),
+               torch.ones(d, dtype=bf, device=dev), torch.zeros(d, dtype=bf, device=dev), torch.cos(ang).to(bf),
+               torch.sin(ang).to(bf), uni(d, d).to(bf), uni(d, d).to(bf), k_cache, k_scale_cache, rows,
+               torch.zeros((t, n, d), dtype=torch.int8, device=dev), torch.zeros((t, n, 1), dtype=torch.float16, device=dev),
+               k_cache, k_scale_cache, torch.zeros((t, n), dtype=torch.float16, device=dev)]
     cfg, attrs = impl.IndexerPrologQuantConfigs(), impl.IndexerPrologQuantAttr()
 
     def step(i):
         impl.lightning_indexer_prolog_quant(*tensors, cfg, attrs)
 
     ms, kernels = timed(torch, lib, step, args)
-    work = 1536 * 8192 + 7168 * (128 + 64) * 2 + t * (7168 * 2 + 1536 + 64 * 130 + 64 * 2 + 130)
+    work = r * n * d + h * (d + n) * 2 + t * (h * 2 + r + n * 130 + n * 2 + 130)
     total_us = sum(kernels.values())
     print(json.dumps({
         "metric": "prolog tokens/sec, DeepSeek-V3.2 lightning_indexer_prolog_quant decode", "value": round(t / (ms * 1e-3), 1),
@@ -235,6 +253,55 @@ def bench_indexer_prolog(args, torch, lib, dev):
                      "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(work / total_us / 1e3 / HBM_PEAK_GBS, 4),
                      "traffic": None, "work_per_launch": work, "us_per_launch": round(total_us, 2),
                      "note": "15 MB of weights read once: bound by launch and memory latency at decode sizes"},
+        "kernels": [{"kernel": k, "us": round(u, 2)} for k, u in kernels.items()], "cpu_baseline": None,
+    }))
+
+
+def bench_mla_prolog(args, torch, lib, dev):
+    """DeepSeek-V3.2 MLA prolog (int8 form) at decode size: one new token for each of `batch` sequences, h 7168,
+    q_lora_rank 1536, 128 heads x (128 + 64), kv_lora_rank 512, a 4K-token paged cache per sequence; the reference
+    generator's distributions (x U[-1,1), weights U[-0.1,0.1), w_uq_qr quantised per output channel, cos/sin
+    U[-0.1,0.1))."""
+    from pypto_amd.deepseek_v32_exp import mla_prolog_quant_impl as impl
+    t, n, h, r, c, bs = args.batch, 128, 7168, 1536, 512, 128
+    g = torch.Generator(device=dev).manual_seed(0)
+    bf = torch.bfloat16
+
+    def uni(lo, hi, *shape):
+        return torch.rand(shape, generator=g, device=dev) * (hi - lo) + lo
+
+    w = uni(-0.1, 0.1, r, n * 192)
+    w_scale = (w.abs().amax(0, keepdim=True) / 127)
+    w_uq_qr = torch.round(w / w_scale).to(torch.int8)
+    n_pages, rows = _paged_rows(torch, dev, g, t, 4096, bs)
+    kv = torch.randint(-127, 128, (n_pages, bs, 1, c), generator=g, device=dev, dtype=torch.int8)
+    kr = uni(-1, 1, n_pages, bs, 1, 64).to(bf)
+    ks = uni(0.001, 0.01, n_pages, bs, 1, 4)
+    tensors = [uni(-1, 1, t, h).to(bf), uni(-0.1, 0.1, h, r).to(bf), w_uq_qr, w_scale.reshape(-1, 1).contiguous(),
+               uni(-0.1, 0.1, n, 128, c).to(bf), uni(-0.1, 0.1, h, c + 64).to(bf), uni(-1, 1, r).to(bf), uni(-1, 1, c).to(bf),
+               uni(-0.1, 0.1, t, 64).to(bf), uni(-0.1, 0.1, t, 64).to(bf), rows, kv, kr, ks,
+               torch.zeros((t, r), dtype=torch.int8, device=dev), torch.zeros((t, 1), dtype=torch.float32, device=dev),
+               torch.zeros((t, n, c), dtype=bf, device=dev), torch.zeros((t, n, 64), dtype=bf, device=dev), kv, kr, ks]
+    cfg, rope = impl.MlaTileConfig(), impl.RopeTileShapeConfig([32, 64], [32, 32, 128], [16, 128, 128, 128])
+
+    def step(i):
+        impl.mla_prolog_quant_d(*tensors, 1e-5, 1e-5, "PA_BSND", cfg, rope)
+
+    ms, kernels = timed(torch, lib, step, args)
+    # weights once, plus per token: x, q_norm + scale, q_nope, q_rope, the cache row
+    work = h * r * 2 + r * n * 192 + n * 192 * 4 + n * 128 * c * 2 + h * (c + 64) * 2 + \
+        t * (h * 2 + r + 4 + n * c * 2 + n * 64 * 2 + c + 16 + 128)
+    total_us = sum(kernels.values())
+    print(json.dumps({
+        "metric": "prolog tokens/sec, DeepSeek-V3.2 mla_prolog_quant decode", "value": round(t / (ms * 1e-3), 1),
+        "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms, 4),
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "int8+bf16", "data": "synthetic",
+        "config": {"workload": f"MLA prolog (int8 form), {t} tokens, h 7168, q_lora_rank 1536, 128 heads x 192, "
+                               f"kv_lora_rank 512"},
+        "roofline": {"kernel": "mla prolog (4 kernels)", "bound": "hbm", "achieved": round(work / total_us / 1e3, 1),
+                     "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(work / total_us / 1e3 / HBM_PEAK_GBS, 4),
+                     "traffic": None, "work_per_launch": work, "us_per_launch": round(total_us, 2),
+                     "note": "85 MB of weights read once per call"},
         "kernels": [{"kernel": k, "us": round(u, 2)} for k, u in kernels.items()], "cpu_baseline": None,
     }))
 
@@ -263,6 +330,8 @@ def main():
         return bench_select_experts(args, torch, lib, dev)
     if args.workload == "indexer_prolog":
         return bench_indexer_prolog(args, torch, lib, dev)
+    if args.workload == "mla_prolog":
+        return bench_mla_prolog(args, torch, lib, dev)
     b, ctx, s1 = args.batch, args.ctx, args.s1
     scale = 192 ** -0.5
     nbuf = 3

@@ -247,6 +247,34 @@ uint64_t pto_mla_prolog_quant_workspace(const PtoTensorDesc* tensors, uint32_t n
 int pto_mla_prolog_quant_launch(const PtoTensorDesc* tensors, uint32_t n_tensors, const PtoMlaPrologParams* params,
                                 void* workspace, uint64_t workspace_bytes, void* hip_stream);
 
+/* Scalar arguments of mla_indexer_prolog_quant_d / _p: the MLA prolog's two epsilons and cache mode, and ip_attrs.eps of
+ * the indexer's LayerNorm (models/deepseek_v32_exp/mla_indexer_prolog_quant_impl.py:521-527). */
+typedef struct {
+    float epsilon_cq;
+    float epsilon_ckv;
+    int32_t cache_mode;
+    float indexer_eps;
+} PtoMlaIndexerPrologParams;
+
+/*
+ * mla_indexer_prolog_quant_d and mla_indexer_prolog_quant_p
+ * (models/deepseek_v32_exp/mla_indexer_prolog_quant_impl.py:320-477 and :479-634, compute :45-318): the MLA prolog
+ * followed by the lightning-indexer prolog on the MLA prolog's q_norm / q_norm_scale, which stay internal (workspace), with
+ * token_x, cos, sin and cache_index shared by both.  tensors[34] in the reference's argument order:
+ *    0-13  token_x, mla_w_dq, mla_w_uq_qr, mla_dequant_scale, mla_w_uk, mla_w_dkv_kr, mla_gamma_cq, mla_gamma_ckv, cos, sin,
+ *          cache_index, mla_kv_cache, mla_kr_cache, mla_k_scale_cache             (as tensors 0-13 of pto_mla_prolog_quant_*)
+ *    14-23 ip_w_qb_in, ip_w_qb_scale_in, ip_wk_in, ip_w_proj_in, ip_ln_gamma_k_in, ip_ln_beta_k_in, ip_hadamard_q_in,
+ *          ip_hadamard_k_in, ip_k_cache, ip_k_cache_scale                         (as tensors 3-8, 11-14 of pto_indexer_prolog_*)
+ *    24-28 mla_query_nope_out, mla_query_rope_out, mla_kv_cache_out, mla_kr_cache_out, mla_k_scale_cache_out
+ *    29-33 ip_q_int8_out, ip_q_scale_out, ip_k_int8_out, ip_k_scale_out, ip_weights_out
+ * The cache outputs are the cache inputs themselves (updated in place).  Shape limits are those of the two operators.
+ */
+uint64_t pto_mla_indexer_prolog_quant_workspace(const PtoTensorDesc* tensors, uint32_t n_tensors,
+                                                const PtoMlaIndexerPrologParams* params);
+int pto_mla_indexer_prolog_quant_launch(const PtoTensorDesc* tensors, uint32_t n_tensors,
+                                        const PtoMlaIndexerPrologParams* params, void* workspace,
+                                        uint64_t workspace_bytes, void* hip_stream);
+
 /* Message of the calling thread's most recent failed call ("" if none).  Replaces the message strings
  * the reference's binding layer returns (python/src/bindings/runtime.cpp:270-335). */
 const char* pto_last_error(void);

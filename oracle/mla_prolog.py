@@ -13,8 +13,6 @@ flash attention reads:
           written into the paged caches (kv int8 [.., 512], scale fp32 [.., 4], rope bf16 [.., 64]) at cache_index
 The rotary embedding takes interleaved pairs: element pairs (2i, 2i+1) are first moved to positions (i, 32+i).
 """
-import math
-
 import torch
 
 
@@ -65,6 +63,22 @@ def _scatter(cache, rows, index):
     return out
 
 
+def query_tail(inp, q_norm, q_norm_scale):
+    """The query path downstream of the quantised RmsNorm: q_nope [t, n, 512] and q_rope [t, n, 64] from q_norm,
+    q_norm_scale (tests also call it with the product's own q_norm to check the downstream stages on their own)."""
+    t = q_norm.shape[0]
+    n, d_nope, c = inp["w_uk"].shape
+    d_rope = inp["cos"].shape[1]
+    dt = inp["x"].dtype
+    qb = torch.matmul(q_norm.to(torch.int32), inp["w_uq_qr"].to(torch.int32)).float()          # :205-210
+    qb = (qb * q_norm_scale) * inp["w_qb_scale"].reshape(1, -1)                                # :211-212
+    qb = qb.to(dt).reshape(t, n, d_nope + d_rope)                                              # :216-218
+    q_nope = torch.matmul(qb[:, :, :d_nope].permute(1, 0, 2).float(), inp["w_uk"].float())     # :220-225
+    q_nope = q_nope.to(dt).permute(1, 0, 2).contiguous()                                       # :226-228
+    q_rope = rope_interleaved(qb[:, :, d_nope:], inp["cos"], inp["sin"])                       # :265-272
+    return q_nope, q_rope
+
+
 def mla_prolog(inp, eps_cq=None, eps_ckv=None):
     """inp: the tensors of make_case().  Returns q_norm int8 [t, r], q_norm_scale fp32 [t, 1], q_nope bf16 [t, n, 512],
     q_rope bf16 [t, n, 64] and updated copies kv_cache, kr_cache, k_scale_cache."""
@@ -75,12 +89,7 @@ def mla_prolog(inp, eps_cq=None, eps_ckv=None):
     qa = torch.matmul(x.float(), inp["w_dq"].float()).to(torch.bfloat16)                       # :192-194
     qn = rms_norm(qa, inp["gamma_cq"], eps_cq)                                                 # :196
     q_norm, q_norm_scale = quant(qn, True)                                                     # :204
-    qb = torch.matmul(q_norm.to(torch.int32), inp["w_uq_qr"].to(torch.int32)).float()          # :205-210
-    qb = (qb * q_norm_scale) * inp["w_qb_scale"].reshape(1, -1)                                # :211-212
-    qb = qb.to(x.dtype).reshape(t, n, d_nope + d_rope)                                         # :216-218
-    q_nope = torch.matmul(qb[:, :, :d_nope].permute(1, 0, 2).float(), inp["w_uk"].float())     # :220-225
-    q_nope = q_nope.to(x.dtype).permute(1, 0, 2).contiguous()                                  # :226-228
-    q_rope = rope_interleaved(qb[:, :, d_nope:], inp["cos"], inp["sin"])                       # :265-272
+    q_nope, q_rope = query_tail(inp, q_norm, q_norm_scale)
 
     kv = torch.matmul(x.float(), inp["w_dkv_kr"].float()).to(x.dtype)                          # :243-247
     ckv = rms_norm(kv[:, :c], inp["gamma_ckv"], eps_ckv)                                       # :250-251
@@ -152,3 +161,27 @@ def make_case(b, s1, s2, seed=5, h=7168, q_lora_rank=1536, n=128, d_nope=128, d_
             idx[i, j] = int(table[i, pos // block_size]) * block_size + pos % block_size
     inp["cache_index"] = idx.reshape(t)
     return inp
+
+
+def make_fused_case(b, s1, s2, seed=5, n_idx=64, **kw):
+    """Inputs of the fused MLA + indexer prolog (models/deepseek_v32_exp/deepseekv32_mla_indexer_prolog_quant.py:336-393,
+    :613-800): the MLA prolog's case plus the indexer's own weights and caches; token_x, cos, sin and cache_index are
+    shared.  Returns (mla_case, indexer_case) - the indexer case still lacks q_norm / q_norm_scale, which the MLA
+    prolog produces."""
+    from . import indexer_prolog as ip
+    mla = make_case(b, s1, s2, seed=seed, **kw)
+    h, r = mla["x"].shape[1], mla["w_dq"].shape[1]
+    idx = ip.make_case(b, s1, s2, seed=seed + 1000, h=h, q_lora_rank=r, n=n_idx)
+    for k in ("q_norm", "q_norm_scale", "block_table"):
+        del idx[k]
+    idx.update(x=mla["x"], cos=mla["cos"], sin=mla["sin"], k_cache_index=mla["cache_index"])
+    return mla, idx
+
+
+def mla_indexer_prolog(mla_case, idx_case, eps_cq=None, eps_ckv=None, eps_idx=1e-6):
+    """The fused golden is the composition (fused driver :336-393 and :711-713): the indexer prolog golden runs on the
+    MLA prolog golden's q_norm / q_norm_scale."""
+    from . import indexer_prolog as ip
+    m = mla_prolog(mla_case, eps_cq, eps_ckv)
+    i = ip.indexer_prolog(dict(idx_case, q_norm=m["q_norm"], q_norm_scale=m["q_norm_scale"]), eps=eps_idx)
+    return m, i

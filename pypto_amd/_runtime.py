@@ -57,6 +57,11 @@ class MlaPrologParams(ctypes.Structure):
     _fields_ = [("epsilon_cq", ctypes.c_float), ("epsilon_ckv", ctypes.c_float), ("cache_mode", ctypes.c_int32)]
 
 
+class MlaIndexerPrologParams(ctypes.Structure):
+    _fields_ = [("epsilon_cq", ctypes.c_float), ("epsilon_ckv", ctypes.c_float), ("cache_mode", ctypes.c_int32),
+                ("indexer_eps", ctypes.c_float)]
+
+
 _OPS = {
     "sfa_quant": SfaParams,
     "sfa_antiquant": SfaParams,
@@ -65,6 +70,7 @@ _OPS = {
     "gqa_decode": GqaParams,
     "indexer_prolog": IndexerPrologParams,
     "mla_prolog_quant": MlaPrologParams,
+    "mla_indexer_prolog_quant": MlaIndexerPrologParams,
 }
 
 # C status -> Python exception type wrapped by FeError

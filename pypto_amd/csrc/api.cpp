@@ -507,9 +507,106 @@ int plan_mla_prolog(const PtoTensorDesc* ts, uint32_t n, const PtoMlaPrologParam
     return PTO_OK;
 }
 
+// mla_indexer_prolog_quant: the MLA prolog followed by the lightning-indexer prolog, which reads the MLA prolog's
+// q_norm / q_norm_scale (held in the workspace) and shares token_x, cos, sin and cache_index with it.
+struct FusedPrologPlan {
+    MlaPrologPlan mla;
+    PrologPlan ip;
+    uint64_t off_ip_ws, off_q_norm, off_q_norm_scale, ws_bytes;
+};
+
+uint64_t up256(uint64_t x) { return (x + 255) & ~(uint64_t)255; }
+
+int plan_fused_prolog(const PtoTensorDesc* ts, uint32_t n, const PtoMlaIndexerPrologParams* p, void* ws, FusedPrologPlan* plan)
+{
+    const char* op = "mla_indexer_prolog_quant";
+    if (ts == nullptr || n != 34) return fail(PTO_ERR_ARG_COUNT, "%s: expected 34 tensors, got %u", op, n);
+    if (p == nullptr) return fail(PTO_ERR_PARAM, "%s: params is null", op);
+    if (ts[0].rank != 2 || ts[1].rank != 2) return fail(PTO_ERR_SHAPE, "%s: token_x and mla_w_dq must have rank 2", op);
+    const int64_t t = ts[0].shape[0], r = ts[1].shape[1];
+    if (t < 0 || r <= 0) return fail(PTO_ERR_SHAPE, "%s: bad token count or q_lora_rank", op);
+    // the intermediate tensors; their addresses are placeholders until the workspace is known
+    uint8_t* base = ws ? static_cast<uint8_t*>(ws) : reinterpret_cast<uint8_t*>(uintptr_t(256));
+    PtoTensorDesc qn = {}, qs = {};
+    qn.dataType = PTO_DT_INT8;
+    qn.rank = 2;
+    qn.shape[0] = t;
+    qn.shape[1] = r;
+    qs.dataType = PTO_DT_FP32;
+    qs.rank = 2;
+    qs.shape[0] = t;
+    qs.shape[1] = 1;
+    qn.addr = base;
+    qs.addr = base;
+    PtoTensorDesc m[21], q[21];
+    for (int i = 0; i < 14; ++i) m[i] = ts[i];
+    m[14] = qn;
+    m[15] = qs;
+    for (int i = 0; i < 5; ++i) m[16 + i] = ts[24 + i];
+    const PtoMlaPrologParams mp = {p->epsilon_cq, p->epsilon_ckv, p->cache_mode};
+    int rc = plan_mla_prolog(m, 21, &mp, &plan->mla);
+    if (rc) return rc;
+    q[0] = ts[0];
+    q[1] = qn;
+    q[2] = qs;
+    for (int i = 0; i < 6; ++i) q[3 + i] = ts[14 + i];
+    q[9] = ts[8];
+    q[10] = ts[9];
+    q[11] = ts[20];
+    q[12] = ts[21];
+    q[13] = ts[22];
+    q[14] = ts[23];
+    q[15] = ts[10];
+    for (int i = 0; i < 5; ++i) q[16 + i] = ts[29 + i];
+    const PtoIndexerPrologParams ipp = {p->indexer_eps};
+    rc = plan_prolog(q, 21, &ipp, &plan->ip);
+    if (rc) return rc;
+    plan->off_ip_ws = up256(plan->mla.ws_bytes);
+    plan->off_q_norm = plan->off_ip_ws + up256(plan->ip.ws_bytes);
+    plan->off_q_norm_scale = plan->off_q_norm + up256((uint64_t)t * r);
+    plan->ws_bytes = plan->off_q_norm_scale + up256((uint64_t)t * 4);
+    if (ws) {
+        plan->mla.args.q_norm = reinterpret_cast<int8_t*>(base + plan->off_q_norm);
+        plan->mla.args.q_norm_scale = reinterpret_cast<float*>(base + plan->off_q_norm_scale);
+        plan->ip.args.q_norm = plan->mla.args.q_norm;
+        plan->ip.args.q_norm_scale = plan->mla.args.q_norm_scale;
+    }
+    return PTO_OK;
+}
+
 } // namespace
 
 extern "C" {
+
+uint64_t pto_mla_indexer_prolog_quant_workspace(const PtoTensorDesc* tensors, uint32_t n_tensors,
+                                                const PtoMlaIndexerPrologParams* params)
+{
+    FusedPrologPlan plan;
+    return plan_fused_prolog(tensors, n_tensors, params, nullptr, &plan) == PTO_OK ? plan.ws_bytes : 0;
+}
+
+int pto_mla_indexer_prolog_quant_launch(const PtoTensorDesc* tensors, uint32_t n_tensors,
+                                        const PtoMlaIndexerPrologParams* params, void* workspace,
+                                        uint64_t workspace_bytes, void* hip_stream)
+{
+    const char* op = "mla_indexer_prolog_quant";
+    FusedPrologPlan plan;
+    int rc = plan_fused_prolog(tensors, n_tensors, params, nullptr, &plan);
+    if (rc) return rc;
+    if (plan.mla.args.t == 0) return PTO_OK;
+    if (workspace == nullptr || workspace_bytes < plan.ws_bytes)
+        return fail(PTO_ERR_WORKSPACE, "%s: workspace of %llu bytes required, got %llu", op,
+                    (unsigned long long)plan.ws_bytes, (unsigned long long)(workspace ? workspace_bytes : 0));
+    if ((rc = plan_fused_prolog(tensors, n_tensors, params, workspace, &plan))) return rc;
+    uint8_t* base = static_cast<uint8_t*>(workspace);
+    pto::mla_prolog_bind_workspace(plan.mla.args, base);
+    pto::prolog_bind_workspace(plan.ip.args, base + plan.off_ip_ws);
+    hipStream_t stream = static_cast<hipStream_t>(hip_stream);
+    hipError_t e = pto::mla_prolog_launch(plan.mla.args, stream);
+    if (e == hipSuccess) e = pto::prolog_launch(plan.ip.args, stream);
+    if (e != hipSuccess) return fail(PTO_ERR_HIP, "%s: HIP launch failed: %s", op, hipGetErrorString(e));
+    return PTO_OK;
+}
 
 uint64_t pto_mla_prolog_quant_workspace(const PtoTensorDesc* tensors, uint32_t n_tensors, const PtoMlaPrologParams* params)
 {

@@ -6,8 +6,11 @@ atol 2.5e-5 and the rope cache with rtol 0.0078125 / atol 1e-4.  Every stage her
 points; what differs from the oracle is the summation order of the fp32 matmuls and of the RmsNorm sums, which now and
 then moves a value across a bf16 rounding boundary.  So, against the oracle evaluated with the operator's epsilons:
 int8 values within 1 everywhere and equal in at least 98 % of the places; scales within one bf16 step (2^-7 relative)
-and bit-equal in most rows; bf16 outputs within the reference's tolerances everywhere and bit-equal in at least 90 %
-of the places (a flipped q_norm value moves the 24576 products of its token by up to one int8 step of that token).
+and bit-equal in most rows.  A flipped q_norm value moves the 24576 products of its token by up to one int8 step of
+that token, which takes a few of that token's q_nope values out of the tight tolerance - the reference's comparator
+allows 0.5 % of such outliers (utils/compare.py:16, max_error_ratio); here at most 0.1 % of the elements and none
+beyond 3 x the tolerance.  The downstream stages are also checked on their own: from the product's own q_norm /
+q_norm_scale the oracle's q_nope and q_rope must be met with no outlier at all.
 """
 import pytest
 import torch
@@ -53,17 +56,21 @@ def check(case, got, eps=EPS):
         assert ((a - b).abs() <= 2.0 ** -7 * b.abs() + 1e-8).all(), f"{name}: {float(((a - b).abs() / b.abs()).max())}"
         assert (a == b).float().mean() >= min_equal, f"{name}: only {(a == b).float().mean():.3f} bit-equal"
 
-    def floats(a, b, name, rtol, atol, min_equal):
+    def floats(a, b, name, rtol, atol, min_equal, outliers=0.0):
         a, b = a.float(), b.float()
         assert torch.isfinite(a).all(), name
-        bad = (a - b).abs() > atol + rtol * b.abs()
-        assert not bad.any(), f"{name}: {int(bad.sum())} values outside rtol {rtol} atol {atol}, worst {float((a - b).abs().max())}"
+        ratio = (a - b).abs() / (atol + rtol * b.abs())
+        assert (ratio > 1).float().mean() <= outliers and ratio.max() <= 3, \
+            f"{name}: {int((ratio > 1).sum())} values outside rtol {rtol} atol {atol}, worst {float(ratio.max())} x"
         assert (a == b).float().mean() >= min_equal, f"{name}: only {(a == b).float().mean():.3f} bit-equal"
 
     ints(got["q_norm"], gold["q_norm"], "q_norm")
     scales(got["q_norm_scale"], gold["q_norm_scale"], "q_norm_scale", 0.80)
-    floats(got["q_nope"], gold["q_nope"], "q_nope", 0.0078125, 0.005, 0.90)
-    floats(got["q_rope"], gold["q_rope"], "q_rope", 0.0078125, 0.005, 0.90)
+    floats(got["q_nope"], gold["q_nope"], "q_nope", 0.0078125, 0.005, 0.85, outliers=1e-3)
+    floats(got["q_rope"], gold["q_rope"], "q_rope", 0.0078125, 0.005, 0.85, outliers=1e-3)
+    tail_nope, tail_rope = op.query_tail(case, got["q_norm"], got["q_norm_scale"])
+    floats(got["q_nope"], tail_nope, "q_nope from the product's q_norm", 0.0078125, 0.005, 0.99)
+    floats(got["q_rope"], tail_rope, "q_rope from the product's q_norm", 0.0078125, 0.005, 0.99)
     ints(got["kv_cache"].view(-1, 512)[rows], gold["kv_cache"].view(-1, 512)[rows], "kv_cache")
     scales(got["k_scale_cache"].view(-1, 4)[rows], gold["k_scale_cache"].view(-1, 4)[rows], "k_scale_cache", 0.80)
     floats(got["kr_cache"].view(-1, 64)[rows], gold["kr_cache"].view(-1, 64)[rows], "kr_cache", 0.0078125, 1e-4, 0.95)
@@ -98,6 +105,28 @@ def test_small_sizes_and_ragged_token_tiles(cuda):
 def test_decode_batch_model_sizes(cuda):
     case = op.make_case(32, 1, 512, seed=15)
     check(case, run(case, cuda))
+
+
+def test_prolog_feeds_sparse_flash_attention(cuda):
+    """Stage chaining: the query the prolog writes and the cache rows it adds are, as they are, what sparse flash
+    attention reads (int8 kv rows with four fp32 scales, bf16 rope rows, q_nope | q_rope)."""
+    from _cases import run_sfa
+    from test_gpu_sfa import full_check
+    b, s1, s2 = 3, 2, 300
+    case = op.make_case(b, s1, s2, seed=16)
+    got = run(case, cuda)
+    rows = case["cache_index"]
+    # the reference generator leaves the old cache rows in whatever range; attention needs them plausible, which they are
+    # (int8 rows with positive scales from quant()).  Every position of a sequence is attended, the new ones included.
+    tk = torch.zeros((b * s1, 2048), dtype=torch.int32)
+    tk[:, :s2] = torch.arange(s2, dtype=torch.int32)
+    ca = {"b": b, "s1": s1, "nq": 128, "topk": 2048, "block_size": 128, "softmax_scale": 192 ** -0.5,
+          "act_seq": [s2] * b, "q": torch.cat([got["q_nope"], got["q_rope"]], dim=-1).reshape(b, s1, 128, 576),
+          "kn": got["kv_cache"].view(-1, 512), "kr": got["kr_cache"].view(-1, 64),
+          "kn_scales": got["k_scale_cache"].view(-1, 4), "topk_indices": tk, "block_table": case["block_table"]}
+    assert (ca["kn_scales"][rows] > 0).all()
+    out = run_sfa(ca, cuda)   # the attention takes the caches as 2-D views [rows, dim], like the reference's driver
+    full_check(out, ca, "prolog -> attention")
 
 
 def test_errors(cuda):
