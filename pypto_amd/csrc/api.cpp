@@ -500,7 +500,7 @@ int plan_mla_prolog(const PtoTensorDesc* ts, uint32_t n, const PtoMlaPrologParam
     a.h = (int32_t)h;
     a.r = (int32_t)r;
     a.n = (int32_t)nh;
-    a.ksplits = (int32_t)(h / 256);
+    a.ksplits = (int32_t)((h + 1023) / 1024);
     a.eps_cq = p->epsilon_cq;
     a.eps_ckv = p->epsilon_ckv;
     plan->ws_bytes = pto::mla_prolog_workspace_bytes(t, h, r, nh);

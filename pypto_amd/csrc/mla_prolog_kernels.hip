@@ -16,7 +16,7 @@
 // At decode sizes the operator streams 85 MB of weights once (w_dq 22, w_uq_qr 38, w_uk 17, w_dkv_kr 8) and is bound
 // by that read.  All four weight matrices are stored with the output dimension contiguous, the opposite of what the
 // MFMA operands want (contraction contiguous per lane), so every weight tile goes through LDS and is read back
-// transposed: bf16 tiles with ds_read_b64_tr_b16, the int8 tile byte by byte.
+// transposed: bf16 tiles with ds_read_b64_tr_b16, the int8 tile with ds_read_b64_tr_b8.
 //   mla_xa_kernel    x @ [w_dq | w_dkv_kr], 256 contraction rows x 128 outputs per workgroup, fp32 partials
 //   mla_norm_kernel  one workgroup per token: fixed-order sum of the partials, both RmsNorms, the quantisations, the
 //                    key's rotary embedding, the three cache writes, q_norm / q_norm_scale
@@ -35,11 +35,16 @@ namespace {
 
 constexpr int MTOK = 32;          // tokens per workgroup tile
 constexpr int MNOPE = 128, MROPE = 64, MQH = MNOPE + MROPE, MC = 512, MKV = MC + MROPE;
-constexpr int XA_K = 256;         // contraction rows per workgroup of mla_xa_kernel
+constexpr int MAX_R = 2048;       // largest q_lora_rank (LDS of mla_norm_kernel, registers of mla_qb_kernel)
+constexpr int XA_K = 256;         // contraction rows per stage of mla_xa_kernel
+constexpr int XA_SPLIT = 1024;    // contraction rows per workgroup of mla_xa_kernel (one fp32 partial sum each)
+constexpr int XROW2 = 64 * 2 + 16; // bytes per LDS row of a [k][64] bf16 weight tile (padded against bank conflicts)
 constexpr int TROW = 128 * 2 + 32; // bytes per LDS row of a [k][128] bf16 weight tile (padded against bank conflicts)
 constexpr int QB_K = 128;         // contraction rows per stage of mla_qb_kernel
-constexpr int QROW = 132;         // bytes per LDS row of a [k][128] int8 weight tile (padded)
-constexpr int MAX_R = 2048;       // largest q_lora_rank mla_norm_kernel holds in LDS
+constexpr int QROW = 136;         // bytes per LDS row of a [k][128] int8 weight tile (padded, 8-byte aligned)
+constexpr int QB_GROUPS = 4;      // wavefront quads of mla_qb_kernel, each with its own stages in flight
+constexpr int QB_MAXS = MAX_R / QB_K / QB_GROUPS; // stages per group at the largest q_lora_rank
+constexpr int QB_QP = MTOK * (MAX_R / 16) / 1024; // 16-byte pieces of the q_norm tile per lane at the largest q_lora_rank
 
 typedef short s16x4 __attribute__((ext_vector_type(4)));
 typedef __attribute__((address_space(3))) s16x4 lds_s16x4;
@@ -47,71 +52,109 @@ __device__ __forceinline__ s16x4 lds_read_tr(const uint8_t* p)
 {
     return __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)const_cast<uint8_t*>(p));
 }
+typedef int v2i __attribute__((ext_vector_type(2)));
+typedef __attribute__((address_space(3))) v2i lds_v2i;
+__device__ __forceinline__ v2i lds_read_tr8(const uint8_t* p)
+{
+    return __builtin_amdgcn_ds_read_tr8_b64_v2i32((lds_v2i*)const_cast<uint8_t*>(p));
+}
 __device__ __forceinline__ float bf16_to_f32(uint16_t v) { return __builtin_bit_cast(float, (uint32_t)v << 16); }
 // The golden's "127 / max": torch evaluates scalar / tensor as reciprocal(tensor) * scalar, two roundings
 __device__ __forceinline__ float quant_scale(float mx) { return (1.0f / mx) * 127.0f; }
 __device__ __forceinline__ uint16_t f32_to_bf16(float f) { return __builtin_bit_cast(uint16_t, (__bf16)f); }
 __device__ __forceinline__ float round_bf16(float f) { return bf16_to_f32(f32_to_bf16(f)); }
 
-// 32 outputs x 32 tokens += W[k0 .. k0 + 16 steps, outputs]^T . X[tokens, k]: A by transposing reads of the [k][n] tile
-// in LDS (lane jj of a 16-lane group points at row 4 hl + jj / 4 (+ 8) of the step, columns 16 mh + 4 (jj & 3)), which
-// hand lane half hl the contraction rows {4 hl .. 4 hl + 3} and {8 + 4 hl .. + 3}; B takes the same rows of X as two
-// 8-byte pieces.  Register e of the result: output 8 (e / 4) + 4 hl + e % 4, token lane % 32.
+// 32 outputs x 32 tokens += W[KSTEPS steps of 16 rows, outputs]^T . X[tokens, k]: A by transposing reads of the [k][n]
+// tile in LDS, rows of ROWB bytes (lane jj of a 16-lane group points at row 4 hl + jj / 4 (+ 8) of the step, columns
+// 16 mh + 4 (jj & 3)), which hand lane half hl the contraction rows {4 hl .. 4 hl + 3} and {8 + 4 hl .. + 3}; B takes the
+// same rows of X as two 8-byte pieces.  Register e of the result: output 8 (e / 4) + 4 hl + e % 4, token lane % 32.
+// The B operand is loaded by its own call so that a caller can put these loads ahead of a prefetch in program order:
+// memory operations complete in order, and a wait for loads issued after a prefetch would wait for the prefetch too.
 template <int KSTEPS>
-__device__ __forceinline__ void gemm_tr_tile(f32x16& acc, const uint8_t* wtile, int ncol0, const uint16_t* xrow, int lane)
+__device__ __forceinline__ void load_b_rows(u32x2 (&b)[2 * KSTEPS], const uint16_t* xrow, int lane)
 {
-    const int jj = lane & 15, mh = (lane >> 4) & 1, hl = lane >> 5;
-    const uint8_t* hp = wtile + (4 * hl + (jj >> 2)) * TROW + (ncol0 + 16 * mh + 4 * (jj & 3)) * 2;
-    const uint16_t* xp = xrow + hl * 4;
+    const uint16_t* xp = xrow + (lane >> 5) * 4;
 #pragma unroll
     for (int ks = 0; ks < KSTEPS; ++ks) {
-        const u32x2 b0 = *reinterpret_cast<const u32x2*>(xp + ks * 16);
-        const u32x2 b1 = *reinterpret_cast<const u32x2*>(xp + ks * 16 + 8);
-        const bf16x8 bv = __builtin_bit_cast(bf16x8, u32x4{b0[0], b0[1], b1[0], b1[1]});
-        const s16x4 lo = lds_read_tr(hp + ks * 16 * TROW);
-        const s16x4 hi = lds_read_tr(hp + (ks * 16 + 8) * TROW);
+        b[2 * ks] = *reinterpret_cast<const u32x2*>(xp + ks * 16);
+        b[2 * ks + 1] = *reinterpret_cast<const u32x2*>(xp + ks * 16 + 8);
+    }
+}
+template <int KSTEPS, int ROWB>
+__device__ __forceinline__ void gemm_tr_tile(f32x16& acc, const uint8_t* wtile, int ncol0, const u32x2 (&b)[2 * KSTEPS], int lane)
+{
+    const int jj = lane & 15, mh = (lane >> 4) & 1, hl = lane >> 5;
+    const uint8_t* hp = wtile + (4 * hl + (jj >> 2)) * ROWB + (ncol0 + 16 * mh + 4 * (jj & 3)) * 2;
+#pragma unroll
+    for (int ks = 0; ks < KSTEPS; ++ks) {
+        const bf16x8 bv = __builtin_bit_cast(bf16x8, u32x4{b[2 * ks][0], b[2 * ks][1], b[2 * ks + 1][0], b[2 * ks + 1][1]});
+        const s16x4 lo = lds_read_tr(hp + ks * 16 * ROWB);
+        const s16x4 hi = lds_read_tr(hp + (ks * 16 + 8) * ROWB);
         const bf16x8 av = __builtin_bit_cast(bf16x8, __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
         acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(av, bv, acc, 0, 0, 0);
     }
 }
 
 // ------------------------------------------------------------------------------------------------ x @ [w_dq | w_dkv_kr]
-// grid (h / 256, output tiles of 128, token tiles of 32), 256 lanes
-__global__ __launch_bounds__(256) void mla_xa_kernel(MlaPrologArgs a)
+// grid (ceil(h / 1024), output tiles of 64, token tiles of 32), 1024 lanes = 4 groups of 4 wavefronts.  Group g takes rows
+// [256 g, 256 g + 256) of the workgroup's 1024 contraction rows: 256 rows x 64 outputs of weights, loaded in one go (every
+// load of the workgroup is in flight at once - at decode sizes the kernel is a single pass over the weights and its
+// duration is one memory latency plus the transfer), transposed through the group's LDS buffer.  Within a group wave w
+// owns the 32 outputs of block w & 1 over rows [128 (w >> 1), + 128).  The eight partial sums of an output are added
+// through LDS in a fixed order; fp32 partial sums per 1024-row split go to the workspace.
+__global__ __launch_bounds__(1024) void mla_xa_kernel(MlaPrologArgs a)
 {
-    extern __shared__ __align__(16) uint8_t wl[]; // [256 k][128 n] bf16, rows of TROW bytes
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    extern __shared__ __align__(16) uint8_t xa_lds[]; // [4 groups][256 k][64 n] bf16, rows of XROW2 bytes
+    const int tid = threadIdx.x & 255, grp = threadIdx.x >> 8, lane = tid & 63, wave = tid >> 6;
     const int l32 = lane & 31, hl = lane >> 5;
     const int split = blockIdx.x, tile = blockIdx.y, tok0 = blockIdx.z * MTOK;
-    const int64_t kbase = (int64_t)split * XA_K;
-    const int qtiles = a.r / 128;
+    const int stages = min(XA_SPLIT, a.h - split * XA_SPLIT) / XA_K; // 256-row stages of this split (4 but for the last)
+    const int sg = min(grp, stages - 1);                              // idle groups re-read the last stage and drop it
+    const int64_t kbase = (int64_t)split * XA_SPLIT + sg * XA_K;
+    const int qtiles = a.r / 64;
     const uint16_t* src;
-    int ld, width;
+    int ld;
     if (tile < qtiles) {
-        src = a.w_dq + tile * 128;
+        src = a.w_dq + tile * 64;
         ld = a.r;
-        width = 128;
     } else {
-        const int c0 = (tile - qtiles) * 128;
-        src = a.w_dkv_kr + c0;
+        src = a.w_dkv_kr + (tile - qtiles) * 64;
         ld = MKV;
-        width = min(128, MKV - c0);
     }
-    const int pieces = width / 8; // 16-byte pieces per row
-#pragma unroll 8
-    for (int i = tid; i < XA_K * pieces; i += 256) {
-        const int k = i / pieces, c = i % pieces;
-        *reinterpret_cast<u32x4*>(wl + k * TROW + c * 16) = *reinterpret_cast<const u32x4*>(src + (kbase + k) * ld + c * 8);
-    }
+    uint8_t* wl = xa_lds + grp * (XA_K * XROW2);
+    const int nb = wave & 1, kh = wave >> 1;
+    // the B operand first, then the weights (memory operations complete in order)
+    u32x2 bx[16];
+    load_b_rows<8>(bx, a.x + (int64_t)min(tok0 + l32, a.t - 1) * a.h + kbase + 128 * kh, lane);
+    // 256 rows x 128 bytes = 8 pieces of 16 bytes per lane (rows tid/8 + 32 i, piece tid%8)
+    const int srow = tid >> 3, spc = tid & 7;
+    const uint16_t* sp = src + (kbase + srow) * ld + 8 * spc;
+    u32x4 stg[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) stg[i] = *reinterpret_cast<const u32x4*>(sp + (int64_t)(32 * i) * ld);
+#pragma unroll
+    for (int i = 0; i < 8; ++i) *reinterpret_cast<u32x4*>(wl + (srow + 32 * i) * XROW2 + 16 * spc) = stg[i];
     __syncthreads();
-    if (32 * wave >= width) return;
     f32x16 acc;
 #pragma unroll
     for (int e = 0; e < 16; ++e) acc[e] = 0.f;
-    gemm_tr_tile<XA_K / 16>(acc, wl, 32 * wave, a.x + (int64_t)min(tok0 + l32, a.t - 1) * a.h + kbase, lane);
+    gemm_tr_tile<8, XROW2>(acc, wl + 128 * kh * XROW2, 32 * nb, bx, lane);
+    __syncthreads();
+    // partial sums of (group, row half) -> LDS; the two collecting waves add them in the order of the rows
+    float* red = reinterpret_cast<float*>(xa_lds);
+    const int part = 2 * grp + kh;
+    if (part > 0 && grp < stages) {
+#pragma unroll
+        for (int e = 0; e < 16; ++e) red[((part * 2 + nb) * 16 + e) * 64 + lane] = acc[e];
+    }
+    __syncthreads();
+    if (part > 0) return;
+    for (int pp = 1; pp < 2 * stages; ++pp)
+#pragma unroll
+        for (int e = 0; e < 16; ++e) acc[e] += red[((pp * 2 + nb) * 16 + e) * 64 + lane];
     const int gt = tok0 + l32;
     if (gt < a.t) {
-        float* out = a.xa_part + ((int64_t)split * a.t + gt) * (a.r + MKV) + tile * 128 + 32 * wave + 4 * hl;
+        float* out = a.xa_part + ((int64_t)split * a.t + gt) * (a.r + MKV) + tile * 64 + 32 * nb + 4 * hl;
 #pragma unroll
         for (int e4 = 0; e4 < 4; ++e4)
             *reinterpret_cast<f32x4*>(out + 8 * e4) = f32x4{acc[4 * e4], acc[4 * e4 + 1], acc[4 * e4 + 2], acc[4 * e4 + 3]};
@@ -140,12 +183,42 @@ __global__ __launch_bounds__(256) void mla_norm_kernel(MlaPrologArgs a)
     __shared__ float red[8];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, tok = blockIdx.x;
     const int r = a.r, ncols = r + MKV;
-    // q_a and kv: partial sums in a fixed order, rounded to bf16
-    for (int c = tid; c < ncols; c += 256) {
-        float s = 0.f;
-#pragma unroll 7
-        for (int sp = 0; sp < a.ksplits; ++sp) s += a.xa_part[((int64_t)sp * a.t + tok) * ncols + c];
-        buf[c] = round_bf16(s);
+    // everything that does not depend on the sums is loaded first, so that its latency hides behind them
+    const int64_t row = a.cache_index[tok];
+    const bool row_ok = row >= 0 && row < a.cache_rows;
+    constexpr int NQ = MAX_R / 256;
+    uint16_t gq[NQ];
+#pragma unroll
+    for (int j = 0; j < NQ; ++j) gq[j] = 256 * j + tid < r ? a.gamma_cq[256 * j + tid] : (uint16_t)0;
+    const uint16_t gk0 = a.gamma_ckv[tid], gk1 = a.gamma_ckv[256 + tid];
+    const int ri = tid & 31;
+    const float rc0 = bf16_to_f32(a.cos[(int64_t)tok * MROPE + ri]), rc1 = bf16_to_f32(a.cos[(int64_t)tok * MROPE + ri + 32]);
+    const float rs0 = bf16_to_f32(a.sin[(int64_t)tok * MROPE + ri]), rs1 = bf16_to_f32(a.sin[(int64_t)tok * MROPE + ri + 32]);
+    // q_a and kv: partial sums in a fixed order, rounded to bf16 (lane: columns tid + 256 j; all of a split's loads in
+    // flight together)
+    {
+        constexpr int NJ = (MAX_R + MKV + 255) / 256;
+        // every load is unconditional (columns past the end re-read the last one and are dropped below): a load under
+        // a condition makes the compiler wait for it on the spot, one memory round trip per load
+        int cj[NJ];
+        float sum[NJ];
+#pragma unroll
+        for (int j = 0; j < NJ; ++j) {
+            cj[j] = min(256 * j + tid, ncols - 1);
+            sum[j] = 0.f;
+        }
+#pragma unroll 4
+        for (int sp = 0; sp < a.ksplits; ++sp) {
+            const float* p = a.xa_part + ((int64_t)sp * a.t + tok) * ncols;
+            float v[NJ];
+#pragma unroll
+            for (int j = 0; j < NJ; ++j) v[j] = p[cj[j]];
+#pragma unroll
+            for (int j = 0; j < NJ; ++j) sum[j] += v[j];
+        }
+#pragma unroll
+        for (int j = 0; j < NJ; ++j)
+            if (256 * j + tid < ncols) buf[256 * j + tid] = round_bf16(sum[j]);
     }
     __syncthreads();
     // query: RmsNorm over r, then per-token quantisation
@@ -158,10 +231,14 @@ __global__ __launch_bounds__(256) void mla_norm_kernel(MlaPrologArgs a)
         __syncthreads();
         const float y = 1.0f / sqrtf(((red[0] + red[1]) + (red[2] + red[3])) + a.eps_cq);
         float mx = 0.f;
-        for (int c = tid; c < r; c += 256) {
-            const float v = round_bf16(bf16_to_f32(a.gamma_cq[c]) * (buf[c] * y));
-            buf[c] = v;
-            mx = fmaxf(mx, fabsf(v));
+#pragma unroll
+        for (int j = 0; j < NQ; ++j) {
+            const int c = 256 * j + tid;
+            if (c < r) {
+                const float v = round_bf16(bf16_to_f32(gq[j]) * (buf[c] * y));
+                buf[c] = v;
+                mx = fmaxf(mx, fabsf(v));
+            }
         }
         mx = wave_max(mx);
         if (lane == 0) red[4 + wave] = mx;
@@ -178,8 +255,6 @@ __global__ __launch_bounds__(256) void mla_norm_kernel(MlaPrologArgs a)
         if (tid == 0) a.q_norm_scale[tok] = 1.0f / sq;
     }
     __syncthreads();
-    const int64_t row = a.cache_index[tok];
-    const bool row_ok = row >= 0 && row < a.cache_rows;
     // key: RmsNorm over 512 (lane: elements tid and tid + 256), groups of 128 quantised on their own
     {
         const float x0 = buf[r + tid], x1 = buf[r + 256 + tid];
@@ -187,8 +262,8 @@ __global__ __launch_bounds__(256) void mla_norm_kernel(MlaPrologArgs a)
         if (lane == 0) red[wave] = ss;
         __syncthreads();
         const float y = 1.0f / sqrtf(((red[0] + red[1]) + (red[2] + red[3])) + a.eps_ckv);
-        const float v0 = round_bf16(bf16_to_f32(a.gamma_ckv[tid]) * (x0 * y));
-        const float v1 = round_bf16(bf16_to_f32(a.gamma_ckv[256 + tid]) * (x1 * y));
+        const float v0 = round_bf16(bf16_to_f32(gk0) * (x0 * y));
+        const float v1 = round_bf16(bf16_to_f32(gk1) * (x1 * y));
         // waves 0, 1 hold group 0 (v0) and group 2 (v1); waves 2, 3 groups 1 and 3
         const float m0 = wave_max(fabsf(v0)), m1 = wave_max(fabsf(v1));
         __syncthreads();
@@ -212,83 +287,116 @@ __global__ __launch_bounds__(256) void mla_norm_kernel(MlaPrologArgs a)
     // key rotary: pair i = elements (2i, 2i+1) -> positions (i, 32 + i)
     if (tid < MROPE / 2 && row_ok) {
         const float xe = buf[r + MC + 2 * tid], xo = buf[r + MC + 2 * tid + 1];
-        const uint16_t* cp = a.cos + (int64_t)tok * MROPE;
-        const uint16_t* sp = a.sin + (int64_t)tok * MROPE;
-        const float o1 = xe * bf16_to_f32(cp[tid]) + (-xo) * bf16_to_f32(sp[tid]);
-        const float o2 = xo * bf16_to_f32(cp[tid + 32]) + xe * bf16_to_f32(sp[tid + 32]);
+        const float o1 = xe * rc0 + (-xo) * rs0;
+        const float o2 = xo * rc1 + xe * rs1;
         a.kr_cache[row * MROPE + tid] = f32_to_bf16(o1);
         a.kr_cache[row * MROPE + 32 + tid] = f32_to_bf16(o2);
     }
 }
 
 // ------------------------------------------------------------------------------------------------ q_norm @ w_uq_qr
-// grid (n * 192 / 128, token tiles of 32), 256 lanes: wave w owns outputs [32 w, 32 w + 32) of the tile
-__global__ __launch_bounds__(256) void mla_qb_kernel(MlaPrologArgs a)
+// grid (n * 192 / 128, token tiles of 32), 1024 lanes = 4 groups of 4 wavefronts.  Group g takes the contraction stages
+// g, g + 4, ... (128 rows x 128 outputs each) and issues the loads of all of them at once (registers), so that the
+// whole tile of weights is in flight together; a stage then goes through the group's LDS buffer to be read back byte-
+// transposed.  The token tile of q_norm sits in LDS (loaded ahead of the weights: memory operations complete in
+// order).  Within a group wave w owns outputs [32 w, 32 w + 32) of the tile.  The groups' int32 sums are added through LDS
+// at the end (exact, so the result does not depend on the split).
+__global__ __launch_bounds__(1024) void mla_qb_kernel(MlaPrologArgs a)
 {
 #pragma clang fp contract(off)
-    __shared__ __align__(16) uint8_t wl[2][QB_K * QROW];
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    extern __shared__ __align__(16) uint8_t qb_lds[]; // [QB_GROUPS][QB_K * QROW] weights | [32][r + 16] q_norm
+    const int tid = threadIdx.x & 255, grp = threadIdx.x >> 8, lane = tid & 63, wave = tid >> 6;
     const int l16 = lane & 15, g = lane >> 4;
     const int col0 = blockIdx.x * 128, tok0 = blockIdx.y * MTOK;
-    const int r = a.r;
+    const int r = a.r, qrowb = r + 16; // padded against bank conflicts (r is a multiple of 128)
     const int64_t nq = (int64_t)a.n * MQH;
+    uint8_t* wl = qb_lds + grp * (QB_K * QROW);
+    uint8_t* ql = qb_lds + QB_GROUPS * (QB_K * QROW);
 
-    // staging: 128 rows x 128 bytes per stage = 4 pieces of 16 bytes per lane (rows tid/8 + 32 i, piece tid%8)
+    // q_norm tile: 32 rows of r bytes, 16-byte pieces over the 1024 lanes (at most QB_QP per lane)
+    const int qpieces = MTOK * (r / 16);
+    u32x4 qst[QB_QP];
+#pragma unroll
+    for (int i = 0; i < QB_QP; ++i) {
+        const int pc = min((int)threadIdx.x + 1024 * i, qpieces - 1);
+        const int row = pc / (r / 16), c = pc % (r / 16);
+        qst[i] = *reinterpret_cast<const u32x4*>(a.q_norm + (int64_t)min(tok0 + row, a.t - 1) * r + 16 * c);
+    }
+    // weights: every stage of this group, 128 rows x 128 bytes = 4 pieces of 16 bytes per lane (rows tid/8 + 32 i, piece
+    // tid%8); stages past the end re-read the last one and are dropped
+    const int stages = r / QB_K;
     const int srow = tid >> 3, spc = tid & 7;
     const int8_t* sp = a.w_uq_qr + (int64_t)srow * nq + col0 + 16 * spc;
-    u32x4 stg[4];
-    auto stage_load = [&](int s) {
+    u32x4 stg[QB_MAXS][4];
 #pragma unroll
-        for (int i = 0; i < 4; ++i) stg[i] = *reinterpret_cast<const u32x4*>(sp + ((int64_t)s * QB_K + 32 * i) * nq);
-    };
-    auto stage_store = [&](int bufi) {
+    for (int j = 0; j < QB_MAXS; ++j) {
+        const int s = min(grp + QB_GROUPS * j, stages - 1);
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            uint32_t* d = reinterpret_cast<uint32_t*>(&wl[bufi][(srow + 32 * i) * QROW + 16 * spc]);
-            d[0] = stg[i][0];
-            d[1] = stg[i][1];
-            d[2] = stg[i][2];
-            d[3] = stg[i][3];
-        }
-    };
+        for (int i = 0; i < 4; ++i) stg[j][i] = *reinterpret_cast<const u32x4*>(sp + ((int64_t)s * QB_K + 32 * i) * nq);
+    }
+#pragma unroll
+    for (int i = 0; i < QB_QP; ++i) {
+        const int pc = (int)threadIdx.x + 1024 * i;
+        if (pc < qpieces) *reinterpret_cast<u32x4*>(ql + (pc / (r / 16)) * qrowb + 16 * (pc % (r / 16))) = qst[i];
+    }
     i32x4 acc[2][2];
 #pragma unroll
     for (int nb = 0; nb < 2; ++nb)
 #pragma unroll
         for (int tb = 0; tb < 2; ++tb) acc[nb][tb] = i32x4{0, 0, 0, 0};
-    const int8_t* qrow[2];
 #pragma unroll
-    for (int tb = 0; tb < 2; ++tb) qrow[tb] = a.q_norm + (int64_t)min(tok0 + 16 * tb + l16, a.t - 1) * r + 16 * g;
-
-    const int stages = r / QB_K;
-    stage_load(0);
-    stage_store(0);
-    __syncthreads();
-    for (int s = 0; s < stages; ++s) {
-        if (s + 1 < stages) stage_load(s + 1);
-        const uint8_t* wb = wl[s & 1];
+    for (int j = 0; j < QB_MAXS; ++j) {
+        const int s = grp + QB_GROUPS * j;
 #pragma unroll
-        for (int ks = 0; ks < QB_K / 64; ++ks) {
-            i32x4 qf[2], wf[2];
+        for (int i = 0; i < 4; ++i) {
+            u32x2* d = reinterpret_cast<u32x2*>(wl + (srow + 32 * i) * QROW + 16 * spc);
+            d[0] = u32x2{stg[j][i][0], stg[j][i][1]};
+            d[1] = u32x2{stg[j][i][2], stg[j][i][3]};
+        }
+        __syncthreads();
+        if (s < stages) {
 #pragma unroll
-            for (int tb = 0; tb < 2; ++tb) qf[tb] = *reinterpret_cast<const i32x4*>(qrow[tb] + s * QB_K + ks * 64);
-            // A operand: output 32 w + 16 nb + l16, contraction bytes 16 g .. 16 g + 15 of the step - one byte per row
-#pragma unroll
-            for (int nb = 0; nb < 2; ++nb) {
-                const uint8_t* p = wb + (ks * 64 + 16 * g) * QROW + 32 * wave + 16 * nb + l16;
-#pragma unroll
-                for (int q4 = 0; q4 < 4; ++q4)
-                    wf[nb][q4] = (int)((uint32_t)p[(4 * q4) * QROW] | ((uint32_t)p[(4 * q4 + 1) * QROW] << 8) |
-                                       ((uint32_t)p[(4 * q4 + 2) * QROW] << 16) | ((uint32_t)p[(4 * q4 + 3) * QROW] << 24));
-            }
-#pragma unroll
-            for (int nb = 0; nb < 2; ++nb)
+            for (int ks = 0; ks < QB_K / 64; ++ks) {
+                i32x4 qf[2], wf[2];
 #pragma unroll
                 for (int tb = 0; tb < 2; ++tb)
-                    acc[nb][tb] = __builtin_amdgcn_mfma_i32_16x16x64_i8(wf[nb], qf[tb], acc[nb][tb], 0, 0, 0);
+                    qf[tb] = *reinterpret_cast<const i32x4*>(ql + (16 * tb + l16) * qrowb + s * QB_K + ks * 64 + 16 * g);
+                // A operand: output 32 w + 16 nb + l16, contraction bytes 16 g .. 16 g + 15 of the step.  An 8-bit
+                // transposing read hands lane i of a 16-lane group byte i % 8 of the chunks addressed by lanes
+                // i / 8, i / 8 + 2, ..., i / 8 + 14: with lane i pointing at row i / 2, column half i % 2, lane i gets
+                // output column i over rows 0 .. 7 - eight of its sixteen contraction bytes per read
+#pragma unroll
+                for (int nb = 0; nb < 2; ++nb) {
+                    const uint8_t* p = wl + (ks * 64 + 16 * g + (l16 >> 1)) * QROW + 32 * wave + 16 * nb + 8 * (l16 & 1);
+                    const v2i lo = lds_read_tr8(p), hi = lds_read_tr8(p + 8 * QROW);
+                    wf[nb] = i32x4{lo[0], lo[1], hi[0], hi[1]};
+                }
+#pragma unroll
+                for (int nb = 0; nb < 2; ++nb)
+#pragma unroll
+                    for (int tb = 0; tb < 2; ++tb)
+                        acc[nb][tb] = __builtin_amdgcn_mfma_i32_16x16x64_i8(wf[nb], qf[tb], acc[nb][tb], 0, 0, 0);
+            }
         }
-        if (s + 1 < stages) stage_store((s + 1) & 1);
         __syncthreads();
+    }
+    // add the groups' sums: groups 1.. leave theirs in their own (now idle) first buffer, group 0 collects
+    if (grp > 0) {
+        i32x4* red = reinterpret_cast<i32x4*>(wl);
+#pragma unroll
+        for (int nb = 0; nb < 2; ++nb)
+#pragma unroll
+            for (int tb = 0; tb < 2; ++tb) red[(2 * nb + tb) * 256 + tid] = acc[nb][tb];
+    }
+    __syncthreads();
+    if (grp > 0) return;
+#pragma unroll
+    for (int og = 1; og < QB_GROUPS; ++og) {
+        const i32x4* red = reinterpret_cast<const i32x4*>(qb_lds + og * (QB_K * QROW));
+#pragma unroll
+        for (int nb = 0; nb < 2; ++nb)
+#pragma unroll
+            for (int tb = 0; tb < 2; ++tb) acc[nb][tb] += red[(2 * nb + tb) * 256 + tid];
     }
     // register e of acc[nb][tb]: output col0 + 32 w + 16 nb + 4 g + e, token 16 tb + l16
 #pragma unroll
@@ -334,6 +442,9 @@ __global__ __launch_bounds__(256) void mla_wuk_kernel(MlaPrologArgs a)
     const int l32 = lane & 31, hl = lane >> 5;
     const int head = blockIdx.x, ct = blockIdx.y, tok0 = blockIdx.z * MTOK;
     const uint16_t* src = a.w_uk + (int64_t)head * MNOPE * MC + ct * 128;
+    const int gt = tok0 + l32;
+    u32x2 bx[2 * (MNOPE / 16)];
+    load_b_rows<MNOPE / 16>(bx, a.qb_nope + ((int64_t)min(gt, a.t - 1) * a.n + head) * MNOPE, lane);
 #pragma unroll
     for (int i = tid; i < MNOPE * 16; i += 256) {
         const int k = i >> 4, c = i & 15;
@@ -343,8 +454,7 @@ __global__ __launch_bounds__(256) void mla_wuk_kernel(MlaPrologArgs a)
     f32x16 acc;
 #pragma unroll
     for (int e = 0; e < 16; ++e) acc[e] = 0.f;
-    const int gt = tok0 + l32;
-    gemm_tr_tile<MNOPE / 16>(acc, wl, 32 * wave, a.qb_nope + ((int64_t)min(gt, a.t - 1) * a.n + head) * MNOPE, lane);
+    gemm_tr_tile<MNOPE / 16, TROW>(acc, wl, 32 * wave, bx, lane);
     if (gt < a.t) {
         uint16_t* out = a.q_nope + ((int64_t)gt * a.n + head) * MC + ct * 128 + 32 * wave + 4 * hl;
 #pragma unroll
@@ -368,7 +478,7 @@ static uint64_t up256(uint64_t x) { return (x + 255) & ~(uint64_t)255; }
 
 uint64_t mla_prolog_workspace_bytes(int64_t t, int64_t h, int64_t r, int64_t n)
 {
-    return up256((uint64_t)(h / XA_K) * t * (r + MKV) * sizeof(float)) + up256((uint64_t)t * n * MNOPE * 2);
+    return up256((uint64_t)((h + XA_SPLIT - 1) / XA_SPLIT) * t * (r + MKV) * sizeof(float)) + up256((uint64_t)t * n * MNOPE * 2);
 }
 
 void mla_prolog_bind_workspace(MlaPrologArgs& a, void* ws)
@@ -385,16 +495,16 @@ hipError_t mla_prolog_launch(const MlaPrologArgs& a, hipStream_t stream)
     const int ttiles = (a.t + MTOK - 1) / MTOK;
     hipError_t e;
     {
-        const int smem = XA_K * TROW;
+        const int smem = 4 * XA_K * XROW2;
         static bool attr_done = false;
         if (!attr_done) {
             e = hipFuncSetAttribute(reinterpret_cast<const void*>(mla_xa_kernel), hipFuncAttributeMaxDynamicSharedMemorySize, smem);
             if (e != hipSuccess) return e;
             attr_done = true;
         }
-        const int tiles = a.r / 128 + (MKV + 127) / 128;
+        const int tiles = (a.r + MKV) / 64;
         ScopedKernelTimer tm(KID_MLA_XA, stream);
-        hipLaunchKernelGGL(mla_xa_kernel, dim3(a.ksplits, tiles, ttiles), dim3(256), smem, stream, a);
+        hipLaunchKernelGGL(mla_xa_kernel, dim3(a.ksplits, tiles, ttiles), dim3(1024), smem, stream, a);
     }
     if ((e = hipGetLastError()) != hipSuccess) return e;
     {
@@ -403,8 +513,16 @@ hipError_t mla_prolog_launch(const MlaPrologArgs& a, hipStream_t stream)
     }
     if ((e = hipGetLastError()) != hipSuccess) return e;
     {
+        const int smem = QB_GROUPS * QB_K * QROW + MTOK * (a.r + 16);
+        static bool attr_done = false;
+        if (!attr_done) {
+            e = hipFuncSetAttribute(reinterpret_cast<const void*>(mla_qb_kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                    QB_GROUPS * QB_K * QROW + MTOK * (MAX_R + 16));
+            if (e != hipSuccess) return e;
+            attr_done = true;
+        }
         ScopedKernelTimer tm(KID_MLA_QB, stream);
-        hipLaunchKernelGGL(mla_qb_kernel, dim3(a.n * MQH / 128, ttiles), dim3(256), 0, stream, a);
+        hipLaunchKernelGGL(mla_qb_kernel, dim3(a.n * MQH / 128, ttiles), dim3(1024), smem, stream, a);
     }
     if ((e = hipGetLastError()) != hipSuccess) return e;
     {
