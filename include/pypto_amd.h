@@ -181,7 +181,7 @@ typedef struct {
  * lightning_indexer_prolog_quant (models/deepseek_v32_exp/lightning_indexer_prolog_quant_impl.py:203-243; tensors in the
  * order of IndexerPrologQuantInput :63-80 followed by IndexerPrologQuantOutput :83-89).  tensors[21], in order:
  *    0 x              [t, h]                 BF16   (h a multiple of 256)
- *    1 q_norm         [t, r]                 INT8   (r a multiple of 64)
+ *    1 q_norm         [t, r]                 INT8   (r a multiple of 128, at most 2048)
  *    2 q_norm_scale   [t, 1]                 FP32
  *    3 w_qb           [r, n*128]             INT8   (plain row-major; the reference's Ascend NZ tiling is a device format)
  *    4 w_qb_scale     [n*128, 1]             FP32
@@ -285,7 +285,7 @@ const char* pto_last_error(void);
  * is bracketed by a HIP event pair recorded on the launch stream; pto_kernel_timing_read waits for the
  * events recorded so far for one kernel, returns their summed duration and count, and forgets them.
  * Kernel ids: 0 indexer_score_kernel, 1 indexer_topk_kernel, 2 sfa_decode_kernel, 3 sfa_combine_kernel,
- * 4 indexer_select_kernel, 5 select_experts_kernel, 6 gqa_decode_kernel, 7 gqa_combine_kernel, 8 prolog_transpose_kernel,
+ * 4 indexer_select_kernel, 5 select_experts_kernel, 6 gqa_decode_kernel, 7 gqa_combine_kernel, 8 (unused),
  * 9 prolog_q_kernel, 10 prolog_xw_kernel, 11 prolog_k_kernel, 12 mla_xa_kernel, 13 mla_norm_kernel, 14 mla_qb_kernel,
  * 15 mla_wuk_kernel
  * (pto_kernel_name returns "" past the last id).

@@ -17,6 +17,7 @@ reference checkout):
   topk.py     top-k ordering rule              framework/src/interface/interpreter/calculator/calc_torch.cpp:2481-2494,2734-2749
   compare.py  tolerance comparators            models/deepseek_v32_exp/utils/compare.py:16-125
   indexer_prolog.py  lightning-indexer prolog  models/deepseek_v32_exp/deepseekv32_lightning_indexer_prolog_quant.py:30-288
+  mla_prolog.py      MLA prolog (int8 form) and the fused MLA + indexer prolog  models/deepseek_v32_exp/deepseekv32_mla_prolog_quant.py:32-441, deepseekv32_mla_indexer_prolog_quant.py:336-393,711-713
   select_experts.py  grouped expert selection  models/glm_v4_5/glm_select_experts.py:274-313
                                                python/tests/ut/interpreter/_ops/moe_gating_topk.py:223-287
   gqa.py      paged GQA decode goldens         models/glm_v4_5/glm_attention.py:1374-1483

@@ -380,7 +380,7 @@ int plan_prolog(const PtoTensorDesc* ts, uint32_t n, const PtoIndexerPrologParam
     const int64_t t = ts[0].shape[0], h = ts[0].shape[1], r = ts[1].shape[1], nd = ts[3].shape[1];
     const int64_t d = ts[11].shape[0], rope = ts[9].shape[1], nh = ts[6].shape[1];
     if (d != 128 || nd != nh * d || !pto::prolog_supported(h, r, nh, d, rope))
-        return fail(PTO_ERR_SHAPE, "%s: need head dim 128, rotary dim 64, heads a multiple of 32 (at most 128), w_qb [r, heads*128] with r a multiple of 64 and h a multiple of 256; got h %lld r %lld heads %lld dim %lld rotary %lld w_qb cols %lld",
+        return fail(PTO_ERR_SHAPE, "%s: need head dim 128, rotary dim 64, heads a multiple of 32 (at most 128), w_qb [r, heads*128] with r a multiple of 128 (at most 2048) and h a multiple of 256; got h %lld r %lld heads %lld dim %lld rotary %lld w_qb cols %lld",
                     op, (long long)h, (long long)r, (long long)nh, (long long)d, (long long)rope, (long long)nd);
     const bool ok = ts[1].shape[0] == t && ts[2].shape[0] == t && ts[2].shape[1] == 1 && ts[3].shape[0] == r &&
                     ts[4].shape[0] == nd && ts[4].shape[1] == 1 && ts[5].shape[0] == h && ts[5].shape[1] == d &&
@@ -415,7 +415,6 @@ int plan_prolog(const PtoTensorDesc* ts, uint32_t n, const PtoIndexerPrologParam
     a.q_int8 = static_cast<int8_t*>(ts[16].addr);
     a.q_scale = static_cast<uint16_t*>(ts[17].addr);
     a.weights = static_cast<uint16_t*>(ts[20].addr);
-    a.w_qb_t = nullptr;
     a.xw_part = nullptr;
     a.cache_rows = ts[13].shape[0] * ts[13].shape[1];
     a.t = (int32_t)t;

@@ -111,7 +111,6 @@ struct PrologArgs {
     int8_t* q_int8;            // [t, n, 128]
     uint16_t* q_scale;         // [t, n] fp16
     uint16_t* weights;         // [t, n] fp16
-    int8_t* w_qb_t;            // workspace [n*128, r]
     float* xw_part;            // workspace [ksplits, t, 128 + n]
     int64_t cache_rows;
     int32_t t, h, r, n, ksplits;

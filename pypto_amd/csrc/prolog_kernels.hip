@@ -12,11 +12,12 @@
 //
 // At decode sizes (tens of tokens) the operator streams 15 MB of weights once and is bound by that read and by launch
 // latency, not by the matrix cores; the kernels are laid out for coalesced weight reads:
-//   prolog_transpose_kernel  w_qb [r, n d] -> [n d, r] in the workspace, so that both operands of the int8 GEMM are
-//                            contiguous along the contraction (16 bytes per lane straight into the MFMA operand layout)
-//   prolog_q_kernel          one workgroup per (head, 32 tokens): int8 MFMA GEMM over r, scale and round to bf16 into
-//                            LDS, rotary in LDS, hadamard as a bf16 MFMA (matrix read with transposing LDS reads),
-//                            quantisation
+//   prolog_q_kernel          one workgroup of 1024 lanes per (head, 32 tokens): int8 MFMA GEMM over r - w_qb has the
+//                            output dimension contiguous, so its tile (r x 128 bytes, every load issued at once) goes
+//                            through LDS and is read back with 8-bit transposing reads; four wave groups split the
+//                            contraction and add their int32 sums through LDS - then, on the first group, scale and
+//                            round to bf16 into LDS, rotary in LDS, hadamard as a bf16 MFMA (matrix read with 16-bit
+//                            transposing LDS reads), quantisation
 //   prolog_xw_kernel         x @ [w_k | w_proj] split over the contraction (256 rows of the weights per workgroup, staged
 //                            in LDS and read with transposing reads); fp32 partials to the workspace
 //   prolog_k_kernel          one workgroup per token: sums the partials in a fixed order, LayerNorm, rotary, hadamard,
@@ -36,6 +37,12 @@ constexpr int PROPE = 64;    // rotary dims
 constexpr int PTOK = 32;     // tokens per workgroup tile
 constexpr int XW_K = 256;    // contraction rows per workgroup of prolog_xw_kernel
 constexpr int XROW = PD * 2 + 16; // bytes per LDS row of the 32 x 128 bf16 tile (padded)
+constexpr int QK = 128;      // contraction rows per stage of prolog_q_kernel
+constexpr int QROW = 136;    // bytes per LDS row of a [k][128] int8 weight stage (padded, 8-byte aligned)
+constexpr int QGROUPS = 4;   // wave groups of prolog_q_kernel, each with its own stages
+constexpr int QMAX_R = 2048; // largest q_lora_rank
+constexpr int QMAXS = QMAX_R / QK / QGROUPS;   // stages per group at the largest q_lora_rank
+constexpr int QQP = PTOK * (QMAX_R / 16) / 1024; // 16-byte pieces of the q_norm tile per lane at the largest q_lora_rank
 
 typedef short s16x4 __attribute__((ext_vector_type(4)));
 typedef short s16x8 __attribute__((ext_vector_type(8)));
@@ -44,35 +51,18 @@ __device__ __forceinline__ s16x4 lds_read_tr(const uint8_t* p)
 {
     return __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)const_cast<uint8_t*>(p));
 }
+typedef int v2i __attribute__((ext_vector_type(2)));
+typedef __attribute__((address_space(3))) v2i lds_v2i;
+__device__ __forceinline__ v2i lds_read_tr8(const uint8_t* p)
+{
+    return __builtin_amdgcn_ds_read_tr8_b64_v2i32((lds_v2i*)const_cast<uint8_t*>(p));
+}
 __device__ __forceinline__ float bf16_to_f32(uint16_t v) { return __builtin_bit_cast(float, (uint32_t)v << 16); }
 // The golden's "127 / max": torch evaluates scalar / tensor as reciprocal(tensor) * scalar, two roundings
 __device__ __forceinline__ float quant_scale(float mx) { return (1.0f / mx) * 127.0f; }
 __device__ __forceinline__ uint16_t f32_to_bf16(float f)
 {
     return __builtin_bit_cast(uint16_t, (__bf16)f);
-}
-
-// ------------------------------------------------------------------------------------------------ transpose
-__global__ __launch_bounds__(256) void prolog_transpose_kernel(const int8_t* __restrict__ w, int8_t* __restrict__ wt,
-                                                               int r, int nd)
-{
-    __shared__ uint8_t tile[64][68];
-    const int n0 = blockIdx.x * 64, r0 = blockIdx.y * 64;
-    const int tx = threadIdx.x & 15, ty = threadIdx.x >> 4;
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-        const int row = ty + 16 * i;
-        const uint32_t v = *reinterpret_cast<const uint32_t*>(w + (int64_t)(r0 + row) * nd + n0 + 4 * tx);
-        *reinterpret_cast<uint32_t*>(&tile[row][4 * tx]) = v;
-    }
-    __syncthreads();
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-        const int nn = ty + 16 * i;
-        const uint32_t v = (uint32_t)tile[4 * tx][nn] | ((uint32_t)tile[4 * tx + 1][nn] << 8) |
-                           ((uint32_t)tile[4 * tx + 2][nn] << 16) | ((uint32_t)tile[4 * tx + 3][nn] << 24);
-        *reinterpret_cast<uint32_t*>(wt + (int64_t)(n0 + nn) * r + r0 + 4 * tx) = v;
-    }
 }
 
 // Rotary embedding of the first 64 dims of the 32 x 128 bf16 tile in LDS, fp32 arithmetic with every product and sum
@@ -97,46 +87,119 @@ __device__ __forceinline__ void rope_tile(uint8_t* xt, const uint16_t* cosp, con
 }
 
 // ------------------------------------------------------------------------------------------------ query path
-// grid (heads, token tiles of 32), 256 lanes
-__global__ __launch_bounds__(256) void prolog_q_kernel(PrologArgs a)
+// grid (heads, token tiles of 32), 1024 lanes = 4 groups of 4 wavefronts
+__global__ __launch_bounds__(1024) void prolog_q_kernel(PrologArgs a)
 {
-    __shared__ __align__(16) uint8_t had[PD * PD * 2]; // hadamard_q, row-major [k][n] bf16
-    __shared__ __align__(16) uint8_t xt[PTOK * XROW];  // the head's tile [token][dim] bf16
-    __shared__ float smax[4][PTOK];
+    // LDS: [4 groups][QK x QROW] weight stages | [32][r + 16] q_norm tile.  Once the GEMM is done the first region is
+    // reused for hadamard_q [128][128] bf16, the head's bf16 tile [32][XROW] and the per-wave maxima.
+    extern __shared__ __align__(16) uint8_t plds[];
+    uint8_t* had = plds;
+    uint8_t* xt = plds + PD * PD * 2;
+    float(*smax)[PTOK] = reinterpret_cast<float(*)[PTOK]>(plds + PD * PD * 2 + PTOK * XROW);
 
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int tid = threadIdx.x & 255, grp = threadIdx.x >> 8, lane = tid & 63, wave = tid >> 6;
     const int l16 = lane & 15, g = lane >> 4, l32 = lane & 31, hl = lane >> 5;
     const int head = blockIdx.x, tok0 = blockIdx.y * PTOK;
-    const int r = a.r;
+    const int r = a.r, qrowb = r + 16;
+    const int64_t nd = (int64_t)a.n * PD;
+    uint8_t* wl = plds + grp * (QK * QROW);
+    uint8_t* ql = plds + QGROUPS * (QK * QROW);
 
-    for (int i = tid; i < PD * PD * 2 / 16; i += 256)
-        reinterpret_cast<u32x4*>(had)[i] = reinterpret_cast<const u32x4*>(a.had_q)[i];
-
-    // C^T[dim, token] = Wt[dim, :] . q_norm[token, :]: wave w owns dims [32 w, 32 w + 32) x 32 tokens
+    // loads in the order they are needed: hadamard_q (parked in registers until the GEMM is over), the q_norm tile,
+    // then every weight stage of this group - all in flight together
+    u32x4 hst[2];
+#pragma unroll
+    for (int i = 0; i < 2; ++i) hst[i] = reinterpret_cast<const u32x4*>(a.had_q)[threadIdx.x + 1024 * i];
+    const int qpieces = PTOK * (r / 16);
+    u32x4 qst[QQP];
+#pragma unroll
+    for (int i = 0; i < QQP; ++i) {
+        const int pc = min((int)threadIdx.x + 1024 * i, qpieces - 1);
+        const int row = pc / (r / 16), c = pc % (r / 16);
+        qst[i] = *reinterpret_cast<const u32x4*>(a.q_norm + (int64_t)min(tok0 + row, a.t - 1) * r + 16 * c);
+    }
+    const int stages = r / QK;
+    const int srow = tid >> 3, spc = tid & 7;
+    const int8_t* sp = a.w_qb + (int64_t)srow * nd + head * PD + 16 * spc;
+    u32x4 stg[QMAXS][4];
+#pragma unroll
+    for (int j = 0; j < QMAXS; ++j) {
+        const int s = min(grp + QGROUPS * j, stages - 1); // past the end: the last stage again, dropped below
+#pragma unroll
+        for (int i = 0; i < 4; ++i) stg[j][i] = *reinterpret_cast<const u32x4*>(sp + ((int64_t)s * QK + 32 * i) * nd);
+    }
+#pragma unroll
+    for (int i = 0; i < QQP; ++i) {
+        const int pc = (int)threadIdx.x + 1024 * i;
+        if (pc < qpieces) *reinterpret_cast<u32x4*>(ql + (pc / (r / 16)) * qrowb + 16 * (pc % (r / 16))) = qst[i];
+    }
+    // C^T[dim, token] = W^T[dim, :] . q_norm[token, :]: wave w owns dims [32 w, 32 w + 32) x 32 tokens
     i32x4 acc[2][2];
 #pragma unroll
     for (int db = 0; db < 2; ++db)
 #pragma unroll
         for (int tb = 0; tb < 2; ++tb) acc[db][tb] = i32x4{0, 0, 0, 0};
-    const int8_t* wrow[2];
-    const int8_t* qrow[2];
 #pragma unroll
-    for (int db = 0; db < 2; ++db) wrow[db] = a.w_qb_t + ((int64_t)head * PD + 32 * wave + 16 * db + l16) * r + 16 * g;
+    for (int j = 0; j < QMAXS; ++j) {
+        const int s = grp + QGROUPS * j;
 #pragma unroll
-    for (int tb = 0; tb < 2; ++tb) qrow[tb] = a.q_norm + (int64_t)min(tok0 + 16 * tb + l16, a.t - 1) * r + 16 * g;
-#pragma unroll 6
-    for (int k0 = 0; k0 < r; k0 += 64) {
-        i32x4 wf[2], qf[2];
+        for (int i = 0; i < 4; ++i) {
+            u32x2* d = reinterpret_cast<u32x2*>(wl + (srow + 32 * i) * QROW + 16 * spc);
+            d[0] = u32x2{stg[j][i][0], stg[j][i][1]};
+            d[1] = u32x2{stg[j][i][2], stg[j][i][3]};
+        }
+        __syncthreads();
+        if (s < stages) {
 #pragma unroll
-        for (int db = 0; db < 2; ++db) wf[db] = *reinterpret_cast<const i32x4*>(wrow[db] + k0);
+            for (int ks = 0; ks < QK / 64; ++ks) {
+                i32x4 qf[2], wf[2];
 #pragma unroll
-        for (int tb = 0; tb < 2; ++tb) qf[tb] = *reinterpret_cast<const i32x4*>(qrow[tb] + k0);
+                for (int tb = 0; tb < 2; ++tb)
+                    qf[tb] = *reinterpret_cast<const i32x4*>(ql + (16 * tb + l16) * qrowb + s * QK + ks * 64 + 16 * g);
+                // A operand: dim 32 w + 16 db + l16, contraction bytes 16 g .. 16 g + 15 of the step.  An 8-bit
+                // transposing read hands lane i of a 16-lane group byte i % 8 of the chunks addressed by lanes
+                // i / 8, i / 8 + 2, ..., i / 8 + 14: with lane i pointing at row i / 2, column half i % 2, lane i gets
+                // column i over rows 0 .. 7 - eight of its sixteen contraction bytes per read
+#pragma unroll
+                for (int db = 0; db < 2; ++db) {
+                    const uint8_t* p = wl + (ks * 64 + 16 * g + (l16 >> 1)) * QROW + 32 * wave + 16 * db + 8 * (l16 & 1);
+                    const v2i lo = lds_read_tr8(p), hi = lds_read_tr8(p + 8 * QROW);
+                    wf[db] = i32x4{lo[0], lo[1], hi[0], hi[1]};
+                }
+#pragma unroll
+                for (int db = 0; db < 2; ++db)
+#pragma unroll
+                    for (int tb = 0; tb < 2; ++tb)
+                        acc[db][tb] = __builtin_amdgcn_mfma_i32_16x16x64_i8(wf[db], qf[tb], acc[db][tb], 0, 0, 0);
+            }
+        }
+        __syncthreads();
+    }
+    // add the groups' int32 sums (exact): groups 1.. leave theirs in their own stage buffer, group 0 collects
+    if (grp > 0) {
+        i32x4* red = reinterpret_cast<i32x4*>(wl);
 #pragma unroll
         for (int db = 0; db < 2; ++db)
 #pragma unroll
-            for (int tb = 0; tb < 2; ++tb)
-                acc[db][tb] = __builtin_amdgcn_mfma_i32_16x16x64_i8(wf[db], qf[tb], acc[db][tb], 0, 0, 0);
+            for (int tb = 0; tb < 2; ++tb) red[(2 * db + tb) * 256 + tid] = acc[db][tb];
     }
+    __syncthreads();
+    if (grp == 0) {
+#pragma unroll
+        for (int og = 1; og < QGROUPS; ++og) {
+            const i32x4* red = reinterpret_cast<const i32x4*>(plds + og * (QK * QROW));
+#pragma unroll
+            for (int db = 0; db < 2; ++db)
+#pragma unroll
+                for (int tb = 0; tb < 2; ++tb) acc[db][tb] += red[(2 * db + tb) * 256 + tid];
+        }
+    }
+    __syncthreads();
+    // the stage buffers are free now: hadamard_q moves in
+#pragma unroll
+    for (int i = 0; i < 2; ++i) reinterpret_cast<u32x4*>(had)[threadIdx.x + 1024 * i] = hst[i];
+    __syncthreads();
+    if (grp > 0) return; // the barriers below are among the first group's waves (a finished wave does not count)
     // register e of acc[db][tb]: dim 32 w + 16 db + 4 g + e, token 16 tb + l16
     {
 #pragma clang fp contract(off)
@@ -300,39 +363,48 @@ __global__ __launch_bounds__(128) void prolog_k_kernel(PrologArgs a)
     __shared__ float kb[PD];
     const int tid = threadIdx.x, tok = blockIdx.x;
     const int nw = PD + a.n;
+    // everything that does not depend on the sums is loaded first (its latency hides behind them), and no load sits
+    // under a condition (the compiler would wait for it on the spot)
+    const int64_t row = a.k_cache_index[tok];
+    const float gam = bf16_to_f32(a.ln_gamma[tid]), bet = bf16_to_f32(a.ln_beta[tid]);
+    const int ri = tid & (PROPE - 1);
+    const float rc = bf16_to_f32(a.cos[(int64_t)tok * PROPE + ri]), rs = bf16_to_f32(a.sin[(int64_t)tok * PROPE + ri]);
+    uint16_t hk[PD]; // this lane's column of hadamard_k
+#pragma unroll
+    for (int k = 0; k < PD; ++k) hk[k] = a.had_k[k * PD + tid];
     float kv = 0.f, wv = 0.f;
-#pragma unroll 7
+    const int wcol = PD + min(tid, a.n - 1);
+#pragma unroll 4
     for (int s = 0; s < a.ksplits; ++s) {
         const float* p = a.xw_part + ((int64_t)s * a.t + tok) * nw;
-        kv += p[tid];
-        if (tid < a.n) wv += p[PD + tid];
+        const float v0 = p[tid], v1 = p[wcol];
+        kv += v0;
+        wv += v1;
     }
     // LayerNorm in fp32 (biased variance), -> bf16
     const float mean = block_sum128(kv, red) / (float)PD;
     const float dlt = kv - mean;
     const float var = block_sum128(dlt * dlt, red) / (float)PD;
     float xn = dlt / sqrtf(var + a.eps);
-    xn = xn * bf16_to_f32(a.ln_gamma[tid]) + bf16_to_f32(a.ln_beta[tid]);
+    xn = xn * gam + bet;
     kb[tid] = bf16_to_f32(f32_to_bf16(xn));
     __syncthreads();
     // rotary on the first 64 dims
     float kr = kb[tid];
     if (tid < PROPE) {
-        const float c = bf16_to_f32(a.cos[(int64_t)tok * PROPE + tid]), s = bf16_to_f32(a.sin[(int64_t)tok * PROPE + tid]);
         const float other = tid < 32 ? -kb[tid + 32] : kb[tid - 32];
-        kr = bf16_to_f32(f32_to_bf16(kb[tid] * c + other * s));
+        kr = bf16_to_f32(f32_to_bf16(kb[tid] * rc + other * rs));
     }
     __syncthreads();
     kb[tid] = kr;
     __syncthreads();
     // hadamard: y[n] = sum_k kr[k] H[k][n], fp32, -> bf16
     float y = 0.f;
-#pragma unroll 16
-    for (int k = 0; k < PD; ++k) y = __builtin_fmaf(kb[k], bf16_to_f32(a.had_k[k * PD + tid]), y);
+#pragma unroll
+    for (int k = 0; k < PD; ++k) y = __builtin_fmaf(kb[k], bf16_to_f32(hk[k]), y);
     y = bf16_to_f32(f32_to_bf16(y));
     const float mx = block_max128(fabsf(y), red);
     const float sq = quant_scale(mx);
-    const int64_t row = a.k_cache_index[tok];
     if (row >= 0 && row < a.cache_rows) {
         a.k_cache[row * PD + tid] = (int8_t)(int)__builtin_rintf(y * sq);
         if (tid == 0) a.k_scale_cache[row] = __builtin_bit_cast(uint16_t, (_Float16)(1.0f / sq));
@@ -347,55 +419,44 @@ __global__ __launch_bounds__(128) void prolog_k_kernel(PrologArgs a)
 
 bool prolog_supported(int64_t h, int64_t r, int64_t n, int64_t d, int64_t rope)
 {
-    return d == PD && rope == PROPE && n > 0 && n % 32 == 0 && n <= 128 && r > 0 && r % 64 == 0 && h > 0 && h % XW_K == 0;
+    return d == PD && rope == PROPE && n > 0 && n % 32 == 0 && n <= 128 && r > 0 && r % QK == 0 && r <= QMAX_R && h > 0 &&
+           h % XW_K == 0;
 }
 
 uint64_t prolog_workspace_bytes(int64_t t, int64_t h, int64_t r, int64_t n)
 {
-    const uint64_t wt = (uint64_t)r * n * PD;
-    const uint64_t part = (uint64_t)(h / XW_K) * t * (PD + n) * sizeof(float);
-    return ((wt + 255) & ~(uint64_t)255) + part;
+    (void)r;
+    return (uint64_t)(h / XW_K) * t * (PD + n) * sizeof(float);
 }
 
-void prolog_bind_workspace(PrologArgs& a, void* ws)
-{
-    uint8_t* p = static_cast<uint8_t*>(ws);
-    a.w_qb_t = reinterpret_cast<int8_t*>(p);
-    p += ((uint64_t)a.r * a.n * PD + 255) & ~(uint64_t)255;
-    a.xw_part = reinterpret_cast<float*>(p);
-}
+void prolog_bind_workspace(PrologArgs& a, void* ws) { a.xw_part = static_cast<float*>(ws); }
 
 hipError_t prolog_launch(const PrologArgs& a, hipStream_t stream)
 {
     if (a.t == 0) return hipSuccess;
-    const int nd = a.n * PD;
     const int ttiles = (a.t + PTOK - 1) / PTOK;
-    {
-        ScopedKernelTimer tm(KID_PROLOG_TRANSPOSE, stream);
-        hipLaunchKernelGGL(prolog_transpose_kernel, dim3(nd / 64, a.r / 64), dim3(256), 0, stream, a.w_qb, a.w_qb_t, a.r, nd);
+    hipError_t e;
+    static bool attr_done = false;
+    if (!attr_done) {
+        e = hipFuncSetAttribute(reinterpret_cast<const void*>(prolog_q_kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                QGROUPS * QK * QROW + PTOK * (QMAX_R + 16));
+        if (e != hipSuccess) return e;
+        e = hipFuncSetAttribute(reinterpret_cast<const void*>(prolog_xw_kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                XW_K * (PD + 128) * 2);
+        if (e != hipSuccess) return e;
+        attr_done = true;
     }
-    hipError_t e = hipGetLastError();
-    if (e != hipSuccess) return e;
     {
+        static_assert(QGROUPS * QK * QROW >= PD * PD * 2 + PTOK * XROW + 4 * PTOK * 4, "epilogue fits in the stage buffers");
         ScopedKernelTimer tm(KID_PROLOG_Q, stream);
-        hipLaunchKernelGGL(prolog_q_kernel, dim3(a.n, ttiles), dim3(256), 0, stream, a);
+        hipLaunchKernelGGL(prolog_q_kernel, dim3(a.n, ttiles), dim3(1024), QGROUPS * QK * QROW + PTOK * (a.r + 16), stream, a);
     }
-    e = hipGetLastError();
-    if (e != hipSuccess) return e;
+    if ((e = hipGetLastError()) != hipSuccess) return e;
     {
-        const int smem = XW_K * (PD + a.n) * 2;
-        static bool attr_done = false;
-        if (!attr_done) {
-            e = hipFuncSetAttribute(reinterpret_cast<const void*>(prolog_xw_kernel),
-                                    hipFuncAttributeMaxDynamicSharedMemorySize, XW_K * (PD + 128) * 2);
-            if (e != hipSuccess) return e;
-            attr_done = true;
-        }
         ScopedKernelTimer tm(KID_PROLOG_XW, stream);
-        hipLaunchKernelGGL(prolog_xw_kernel, dim3(a.ksplits, ttiles), dim3(256), smem, stream, a);
+        hipLaunchKernelGGL(prolog_xw_kernel, dim3(a.ksplits, ttiles), dim3(256), XW_K * (PD + a.n) * 2, stream, a);
     }
-    e = hipGetLastError();
-    if (e != hipSuccess) return e;
+    if ((e = hipGetLastError()) != hipSuccess) return e;
     {
         ScopedKernelTimer tm(KID_PROLOG_K, stream);
         hipLaunchKernelGGL(prolog_k_kernel, dim3(a.t), dim3(128), 0, stream, a);

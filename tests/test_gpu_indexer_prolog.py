@@ -102,7 +102,7 @@ def test_prolog_feeds_the_indexer(cuda):
 
 def test_errors(cuda):
     from pypto_amd.error import FeError
-    case = op.make_case(2, 1, 256, seed=1, h=512, q_lora_rank=64, n=32)
+    case = op.make_case(2, 1, 256, seed=1, h=512, q_lora_rank=128, n=32)
     bad = dict(case, k_cache_index=case["k_cache_index"].int())
     with pytest.raises(FeError, match="int64"):
         run(bad, cuda)
