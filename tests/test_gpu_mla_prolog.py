@@ -107,6 +107,12 @@ def test_decode_batch_model_sizes(cuda):
     check(case, run(case, cuda))
 
 
+def test_reference_prefill_case_t128(cuda):
+    # the reference's (skipped, "large shape") prefill test test_b128_s4k4_pa_nd_bf16_quantb_p: 128 tokens, model sizes
+    case = op.make_case(128, 1, 1024, seed=17)
+    check(case, run(case, cuda, entry="mla_prolog_quant_p"))
+
+
 def test_prolog_feeds_sparse_flash_attention(cuda):
     """Stage chaining: the query the prolog writes and the cache rows it adds are, as they are, what sparse flash
     attention reads (int8 kv rows with four fp32 scales, bf16 rope rows, q_nope | q_rope)."""

@@ -171,6 +171,25 @@ def test_full_size_config5_mtp(cuda):
     full_check(run_sfa(case, cuda, packed=True, entry="d_950"), case, "config5 mtp")
 
 
+def test_reference_prefill_case_b1_s256(cuda):
+    """The reference's (skipped, "large test case") prefill test sfa_bf16_b1_s256_seq64K_int8_p: one sequence of 65536
+    cached tokens, 256 query tokens, 128 heads, through the prefill entry.  The full output is produced on the GPU; the
+    oracle checks a sample of the query tokens (every token attends exactly topk rows here, so a token's result depends on
+    its own query and top-k row only) and every token is checked for finiteness and for lying inside the convex hull of
+    the dequantised values it attends."""
+    case = osfa.make_case(1, 128, 256, [65536], seed=23)
+    out = run_sfa(case, cuda, entry="p")
+    assert torch.isfinite(out.float()).all()
+    sel = [0, 1, 100, 255]
+    sub = dict(case, s1=len(sel), q=case["q"][:, sel].contiguous(),
+               topk_indices=case["topk_indices"].reshape(1, 256, -1)[:, sel].reshape(len(sel), -1).contiguous())
+    full_check(out[:, sel].contiguous(), sub, "prefill b1 s256 (sampled tokens)")
+    kn = osfa.dequant_nope(case["kn"], case["kn_scales"]).float()
+    lo, hi = kn.min(0).values, kn.max(0).values
+    o = out.float().reshape(-1, 512)
+    assert (o >= lo - 0.02).all() and (o <= hi + 0.02).all()
+
+
 def test_bad_calls_raise_before_launch(cuda):
     from pypto_amd.deepseek_v32_exp import sparse_flash_attention_quant_impl as impl
     from pypto_amd.error import FeError
