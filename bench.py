@@ -48,7 +48,7 @@ def parse():
     ap.add_argument("--cpu-seqs", type=int, default=8, help="sequences of the workload timed on the CPU oracle")
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--packed", action="store_true", help="use the packed 656-byte-row attention entry point")
-    ap.add_argument("--workload", choices=["v32", "gqa", "select_experts", "indexer_prolog", "mla_prolog"], default="v32",
+    ap.add_argument("--workload", choices=["v32", "gqa", "select_experts", "indexer_prolog", "mla_prolog", "mla_indexer_prolog"], default="v32",
                     help="v32 (default): the headline DeepSeek-V3.2 indexer + sparse attention decode step; gqa: GLM-4.5 "
                          "paged GQA decode (batch 64, 96/8 heads, contexts U[4096, 32768]); select_experts: GLM-4.5 "
                          "router (8192 tokens x 160 experts)")
@@ -306,6 +306,60 @@ def bench_mla_prolog(args, torch, lib, dev):
     }))
 
 
+def bench_mla_indexer_prolog(args, torch, lib, dev):
+    """DeepSeek-V3.2 fused MLA + lightning-indexer prolog at decode size: the two workloads above in one call (shared
+    token_x, cos, sin, cache_index; q_norm handed over inside the workspace)."""
+    from pypto_amd.deepseek_v32_exp import mla_indexer_prolog_quant_impl as impl
+    t, n, ni, h, r, c, d, bs = args.batch, 128, 64, 7168, 1536, 512, 128, 128
+    g = torch.Generator(device=dev).manual_seed(0)
+    bf = torch.bfloat16
+
+    def uni(lo, hi, *shape):
+        return torch.rand(shape, generator=g, device=dev) * (hi - lo) + lo
+
+    def i8(*shape):
+        return torch.randint(-128, 128, shape, generator=g, device=dev, dtype=torch.int8)
+
+    w = uni(-0.1, 0.1, r, n * 192)
+    w_scale = (w.abs().amax(0, keepdim=True) / 127)
+    n_pages, rows = _paged_rows(torch, dev, g, t, 4096, bs)
+    kv = torch.randint(-127, 128, (n_pages, bs, 1, c), generator=g, device=dev, dtype=torch.int8)
+    kr, ks = uni(-1, 1, n_pages, bs, 1, 64).to(bf), uni(0.001, 0.01, n_pages, bs, 1, 4)
+    ik, iks = i8(n_pages, bs, 1, d), uni(-1, 1, n_pages, bs, 1, 1).to(torch.float16)
+    tensors = [uni(-1, 1, t, h).to(bf), uni(-0.1, 0.1, h, r).to(bf), torch.round(w / w_scale).to(torch.int8),
+               w_scale.reshape(-1, 1).contiguous(), uni(-0.1, 0.1, n, 128, c).to(bf), uni(-0.1, 0.1, h, c + 64).to(bf),
+               uni(-1, 1, r).to(bf), uni(-1, 1, c).to(bf), uni(-0.1, 0.1, t, 64).to(bf), uni(-0.1, 0.1, t, 64).to(bf), rows,
+               kv, kr, ks,
+               i8(r, ni * d), uni(-1, 1, ni * d, 1), uni(-1, 1, h, d).to(bf), uni(-1, 1, h, ni).to(bf),
+               torch.ones(d, dtype=bf, device=dev), torch.zeros(d, dtype=bf, device=dev), uni(-1, 1, d, d).to(bf),
+               uni(-1, 1, d, d).to(bf), ik, iks,
+               torch.zeros((t, n, c), dtype=bf, device=dev), torch.zeros((t, n, 64), dtype=bf, device=dev), kv, kr, ks,
+               torch.zeros((t, ni, d), dtype=torch.int8, device=dev), torch.zeros((t, ni, 1), dtype=torch.float16, device=dev),
+               ik, iks, torch.zeros((t, ni), dtype=torch.float16, device=dev)]
+    scal = (1e-5, 1e-5, "PA_BSND", impl.MlaTileConfig(), impl.IndexerPrologQuantAttr(), impl.IndexerPrologQuantConfigs(),
+            impl.RopeTileShapeConfig([32, 64], [32, 32, 128], [16, 128, 128, 128]))
+
+    def step(i):
+        impl.mla_indexer_prolog_quant_d(*tensors, *scal)
+
+    ms, kernels = timed(torch, lib, step, args)
+    work = h * r * 2 + r * n * 192 + n * 192 * 4 + n * 128 * c * 2 + h * (c + 64) * 2 + r * ni * d + h * (d + ni) * 2 + \
+        t * (h * 2 + n * c * 2 + n * 64 * 2 + c + 16 + 128 + ni * 130 + ni * 2 + 130)
+    total_us = sum(kernels.values())
+    print(json.dumps({
+        "metric": "prolog tokens/sec, DeepSeek-V3.2 mla_indexer_prolog_quant decode", "value": round(t / (ms * 1e-3), 1),
+        "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms, 4),
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "int8+bf16", "data": "synthetic",
+        "config": {"workload": f"fused MLA + lightning-indexer prolog, {t} tokens, h 7168, q_lora_rank 1536, 128 heads x 192, "
+                               f"kv_lora_rank 512, 64 x 128 index heads"},
+        "roofline": {"kernel": "fused prolog (4 kernels)", "bound": "hbm", "achieved": round(work / total_us / 1e3, 1),
+                     "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(work / total_us / 1e3 / HBM_PEAK_GBS, 4),
+                     "traffic": None, "work_per_launch": work, "us_per_launch": round(total_us, 2),
+                     "note": "100 MB of weights read once per call"},
+        "kernels": [{"kernel": k, "us": round(u, 2)} for k, u in kernels.items()], "cpu_baseline": None,
+    }))
+
+
 def main():
     args = parse()
     if args.gpus != 1:
@@ -332,6 +386,8 @@ def main():
         return bench_indexer_prolog(args, torch, lib, dev)
     if args.workload == "mla_prolog":
         return bench_mla_prolog(args, torch, lib, dev)
+    if args.workload == "mla_indexer_prolog":
+        return bench_mla_indexer_prolog(args, torch, lib, dev)
     b, ctx, s1 = args.batch, args.ctx, args.s1
     scale = 192 ** -0.5
     nbuf = 3

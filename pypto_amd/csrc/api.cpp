@@ -494,6 +494,10 @@ int plan_mla_prolog(const PtoTensorDesc* ts, uint32_t n, const PtoMlaPrologParam
     a.q_rope = static_cast<uint16_t*>(ts[17].addr);
     a.xa_part = nullptr;
     a.qb_nope = nullptr;
+    a.w_k = nullptr;
+    a.w_proj = nullptr;
+    a.n_idx = 0;
+    a.ncols = (int32_t)(r + c + rope);
     a.cache_rows = ts[11].shape[0] * ts[11].shape[1];
     a.t = (int32_t)t;
     a.h = (int32_t)h;
@@ -502,7 +506,7 @@ int plan_mla_prolog(const PtoTensorDesc* ts, uint32_t n, const PtoMlaPrologParam
     a.ksplits = (int32_t)((h + 1023) / 1024);
     a.eps_cq = p->epsilon_cq;
     a.eps_ckv = p->epsilon_ckv;
-    plan->ws_bytes = pto::mla_prolog_workspace_bytes(t, h, r, nh);
+    plan->ws_bytes = pto::mla_prolog_workspace_bytes(t, h, r, nh, 0);
     return PTO_OK;
 }
 
@@ -512,6 +516,7 @@ struct FusedPrologPlan {
     MlaPrologPlan mla;
     PrologPlan ip;
     uint64_t off_ip_ws, off_q_norm, off_q_norm_scale, ws_bytes;
+    bool fused; // four launches (the two operators' kernels side by side) instead of seven
 };
 
 uint64_t up256(uint64_t x) { return (x + 255) & ~(uint64_t)255; }
@@ -560,6 +565,11 @@ int plan_fused_prolog(const PtoTensorDesc* ts, uint32_t n, const PtoMlaIndexerPr
     const PtoIndexerPrologParams ipp = {p->indexer_eps};
     rc = plan_prolog(q, 21, &ipp, &plan->ip);
     if (rc) return rc;
+    plan->fused = pto::fused_prolog_supported(plan->ip.args.n);
+    if (plan->fused) { // the indexer's partial sums live inside the MLA prolog's: no workspace of its own
+        plan->mla.ws_bytes = pto::mla_prolog_workspace_bytes(t, plan->mla.args.h, r, plan->mla.args.n, plan->ip.args.n);
+        plan->ip.ws_bytes = 0;
+    }
     plan->off_ip_ws = up256(plan->mla.ws_bytes);
     plan->off_q_norm = plan->off_ip_ws + up256(plan->ip.ws_bytes);
     plan->off_q_norm_scale = plan->off_q_norm + up256((uint64_t)t * r);
@@ -598,11 +608,17 @@ int pto_mla_indexer_prolog_quant_launch(const PtoTensorDesc* tensors, uint32_t n
                     (unsigned long long)plan.ws_bytes, (unsigned long long)(workspace ? workspace_bytes : 0));
     if ((rc = plan_fused_prolog(tensors, n_tensors, params, workspace, &plan))) return rc;
     uint8_t* base = static_cast<uint8_t*>(workspace);
-    pto::mla_prolog_bind_workspace(plan.mla.args, base);
-    pto::prolog_bind_workspace(plan.ip.args, base + plan.off_ip_ws);
     hipStream_t stream = static_cast<hipStream_t>(hip_stream);
-    hipError_t e = pto::mla_prolog_launch(plan.mla.args, stream);
-    if (e == hipSuccess) e = pto::prolog_launch(plan.ip.args, stream);
+    hipError_t e;
+    if (plan.fused) {
+        pto::fused_prolog_bind(plan.mla.args, plan.ip.args, base);
+        e = pto::fused_prolog_launch(plan.mla.args, plan.ip.args, stream);
+    } else {
+        pto::mla_prolog_bind_workspace(plan.mla.args, base);
+        pto::prolog_bind_workspace(plan.ip.args, base + plan.off_ip_ws);
+        e = pto::mla_prolog_launch(plan.mla.args, stream);
+        if (e == hipSuccess) e = pto::prolog_launch(plan.ip.args, stream);
+    }
     if (e != hipSuccess) return fail(PTO_ERR_HIP, "%s: HIP launch failed: %s", op, hipGetErrorString(e));
     return PTO_OK;
 }

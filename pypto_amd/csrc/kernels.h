@@ -111,7 +111,9 @@ struct PrologArgs {
     int8_t* q_int8;            // [t, n, 128]
     uint16_t* q_scale;         // [t, n] fp16
     uint16_t* weights;         // [t, n] fp16
-    float* xw_part;            // workspace [ksplits, t, 128 + n]
+    float* xw_part;            // fp32 partial sums of x @ [w_k | w_proj]: element (split, token, col) at
+                               // xw_part[(split * t + token) * xw_stride + xw_col0 + col]
+    int32_t xw_stride, xw_col0;
     int64_t cache_rows;
     int32_t t, h, r, n, ksplits;
     float eps, wscale_n, wscale_d;
@@ -142,16 +144,24 @@ struct MlaPrologArgs {
     float* q_norm_scale;        // [t]
     uint16_t* q_nope;           // [t, n, 512] bf16
     uint16_t* q_rope;           // [t, n, 64] bf16
-    float* xa_part;             // workspace [ksplits, t, r + 576]
+    const uint16_t* w_k;        // fused with the indexer prolog only: its [h, 128] and [h, n_idx] bf16 weights, whose
+    const uint16_t* w_proj;     // products with x ride along in the first kernel
+    float* xa_part;             // workspace [ksplits, t, ncols]
     uint16_t* qb_nope;          // workspace [t, n, 128] bf16
     int64_t cache_rows;
     int32_t t, h, r, n, ksplits;
+    int32_t n_idx, ncols;       // index heads (0: not fused); columns of a partial-sum row: r + 576 (+ 128 + n_idx)
     float eps_cq, eps_ckv;
 };
 
 bool mla_prolog_supported(int64_t h, int64_t r, int64_t n, int64_t d_nope, int64_t d_rope, int64_t c);
-uint64_t mla_prolog_workspace_bytes(int64_t t, int64_t h, int64_t r, int64_t n);
+uint64_t mla_prolog_workspace_bytes(int64_t t, int64_t h, int64_t r, int64_t n, int64_t n_idx);
 void mla_prolog_bind_workspace(MlaPrologArgs& a, void* workspace);
 hipError_t mla_prolog_launch(const MlaPrologArgs& a, hipStream_t stream);
+// The fused MLA + indexer prolog as four launches (needs n_idx a multiple of 64); fused_prolog_bind points the indexer's
+// partial sums into the MLA prolog's and sizes are those of mla_prolog_workspace_bytes(.., n_idx).
+bool fused_prolog_supported(int64_t n_idx);
+void fused_prolog_bind(MlaPrologArgs& m, PrologArgs& p, void* workspace);
+hipError_t fused_prolog_launch(const MlaPrologArgs& m, const PrologArgs& p, hipStream_t stream);
 
 } // namespace pto

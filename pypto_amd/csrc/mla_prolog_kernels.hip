@@ -28,6 +28,8 @@
 
 #include "common.h"
 #include "kernels.h"
+#include "prolog_common.h"
+#include "prolog_device.h"
 #include "timing.h"
 
 namespace pto {
@@ -41,28 +43,11 @@ constexpr int XA_SPLIT = 1024;    // contraction rows per workgroup of mla_xa_ke
 constexpr int XROW2 = 64 * 2 + 16; // bytes per LDS row of a [k][64] bf16 weight tile (padded against bank conflicts)
 constexpr int TROW = 128 * 2 + 32; // bytes per LDS row of a [k][128] bf16 weight tile (padded against bank conflicts)
 constexpr int QB_K = 128;         // contraction rows per stage of mla_qb_kernel
-constexpr int QROW = 136;         // bytes per LDS row of a [k][128] int8 weight tile (padded, 8-byte aligned)
+constexpr int MQROW = 136;         // bytes per LDS row of a [k][128] int8 weight tile (padded, 8-byte aligned)
 constexpr int QB_GROUPS = 4;      // wavefront quads of mla_qb_kernel, each with its own stages in flight
 constexpr int QB_MAXS = MAX_R / QB_K / QB_GROUPS; // stages per group at the largest q_lora_rank
 constexpr int QB_QP = MTOK * (MAX_R / 16) / 1024; // 16-byte pieces of the q_norm tile per lane at the largest q_lora_rank
 
-typedef short s16x4 __attribute__((ext_vector_type(4)));
-typedef __attribute__((address_space(3))) s16x4 lds_s16x4;
-__device__ __forceinline__ s16x4 lds_read_tr(const uint8_t* p)
-{
-    return __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)const_cast<uint8_t*>(p));
-}
-typedef int v2i __attribute__((ext_vector_type(2)));
-typedef __attribute__((address_space(3))) v2i lds_v2i;
-__device__ __forceinline__ v2i lds_read_tr8(const uint8_t* p)
-{
-    return __builtin_amdgcn_ds_read_tr8_b64_v2i32((lds_v2i*)const_cast<uint8_t*>(p));
-}
-__device__ __forceinline__ float bf16_to_f32(uint16_t v) { return __builtin_bit_cast(float, (uint32_t)v << 16); }
-// The golden's "127 / max": torch evaluates scalar / tensor as reciprocal(tensor) * scalar, two roundings
-__device__ __forceinline__ float quant_scale(float mx) { return (1.0f / mx) * 127.0f; }
-__device__ __forceinline__ uint16_t f32_to_bf16(float f) { return __builtin_bit_cast(uint16_t, (__bf16)f); }
-__device__ __forceinline__ float round_bf16(float f) { return bf16_to_f32(f32_to_bf16(f)); }
 
 // 32 outputs x 32 tokens += W[KSTEPS steps of 16 rows, outputs]^T . X[tokens, k]: A by transposing reads of the [k][n]
 // tile in LDS, rows of ROWB bytes (lane jj of a 16-lane group points at row 4 hl + jj / 4 (+ 8) of the step, columns
@@ -117,9 +102,15 @@ __global__ __launch_bounds__(1024) void mla_xa_kernel(MlaPrologArgs a)
     if (tile < qtiles) {
         src = a.w_dq + tile * 64;
         ld = a.r;
-    } else {
+    } else if (tile < qtiles + MKV / 64) {
         src = a.w_dkv_kr + (tile - qtiles) * 64;
         ld = MKV;
+    } else if (tile < qtiles + MKV / 64 + PD / 64) { // fused with the indexer prolog: its x @ [w_k | w_proj] rides along
+        src = a.w_k + (tile - qtiles - MKV / 64) * 64;
+        ld = PD;
+    } else {
+        src = a.w_proj + (tile - qtiles - MKV / 64 - PD / 64) * 64;
+        ld = a.n_idx;
     }
     uint8_t* wl = xa_lds + grp * (XA_K * XROW2);
     const int nb = wave & 1, kh = wave >> 1;
@@ -154,7 +145,7 @@ __global__ __launch_bounds__(1024) void mla_xa_kernel(MlaPrologArgs a)
         for (int e = 0; e < 16; ++e) acc[e] += red[((pp * 2 + nb) * 16 + e) * 64 + lane];
     const int gt = tok0 + l32;
     if (gt < a.t) {
-        float* out = a.xa_part + ((int64_t)split * a.t + gt) * (a.r + MKV) + tile * 64 + 32 * nb + 4 * hl;
+        float* out = a.xa_part + ((int64_t)split * a.t + gt) * a.ncols + tile * 64 + 32 * nb + 4 * hl;
 #pragma unroll
         for (int e4 = 0; e4 < 4; ++e4)
             *reinterpret_cast<f32x4*>(out + 8 * e4) = f32x4{acc[4 * e4], acc[4 * e4 + 1], acc[4 * e4 + 2], acc[4 * e4 + 3]};
@@ -175,13 +166,13 @@ __device__ __forceinline__ float wave_max(float v)
     return v;
 }
 
-// grid (tokens), 256 lanes
-__global__ __launch_bounds__(256) void mla_norm_kernel(MlaPrologArgs a)
+// one workgroup of 256 lanes per token
+__device__ __forceinline__ void mla_norm_body(const MlaPrologArgs& a, int tok)
 {
 #pragma clang fp contract(off)
     __shared__ float buf[MAX_R + MKV];
     __shared__ float red[8];
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, tok = blockIdx.x;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int r = a.r, ncols = r + MKV;
     // everything that does not depend on the sums is loaded first, so that its latency hides behind them
     const int64_t row = a.cache_index[tok];
@@ -209,7 +200,7 @@ __global__ __launch_bounds__(256) void mla_norm_kernel(MlaPrologArgs a)
         }
 #pragma unroll 4
         for (int sp = 0; sp < a.ksplits; ++sp) {
-            const float* p = a.xa_part + ((int64_t)sp * a.t + tok) * ncols;
+            const float* p = a.xa_part + ((int64_t)sp * a.t + tok) * a.ncols;
             float v[NJ];
 #pragma unroll
             for (int j = 0; j < NJ; ++j) v[j] = p[cj[j]];
@@ -301,17 +292,17 @@ __global__ __launch_bounds__(256) void mla_norm_kernel(MlaPrologArgs a)
 // transposed.  The token tile of q_norm sits in LDS (loaded ahead of the weights: memory operations complete in
 // order).  Within a group wave w owns outputs [32 w, 32 w + 32) of the tile.  The groups' int32 sums are added through LDS
 // at the end (exact, so the result does not depend on the split).
-__global__ __launch_bounds__(1024) void mla_qb_kernel(MlaPrologArgs a)
+__host__ __device__ constexpr int mla_qb_lds_bytes(int r) { return QB_GROUPS * QB_K * MQROW + MTOK * (r + 16); }
+// qb_lds: [QB_GROUPS][QB_K * MQROW] weights | [32][r + 16] q_norm
+__device__ __forceinline__ void mla_qb_body(const MlaPrologArgs& a, int col0, int tok0, uint8_t* qb_lds)
 {
 #pragma clang fp contract(off)
-    extern __shared__ __align__(16) uint8_t qb_lds[]; // [QB_GROUPS][QB_K * QROW] weights | [32][r + 16] q_norm
     const int tid = threadIdx.x & 255, grp = threadIdx.x >> 8, lane = tid & 63, wave = tid >> 6;
     const int l16 = lane & 15, g = lane >> 4;
-    const int col0 = blockIdx.x * 128, tok0 = blockIdx.y * MTOK;
     const int r = a.r, qrowb = r + 16; // padded against bank conflicts (r is a multiple of 128)
     const int64_t nq = (int64_t)a.n * MQH;
-    uint8_t* wl = qb_lds + grp * (QB_K * QROW);
-    uint8_t* ql = qb_lds + QB_GROUPS * (QB_K * QROW);
+    uint8_t* wl = qb_lds + grp * (QB_K * MQROW);
+    uint8_t* ql = qb_lds + QB_GROUPS * (QB_K * MQROW);
 
     // q_norm tile: 32 rows of r bytes, 16-byte pieces over the 1024 lanes (at most QB_QP per lane)
     const int qpieces = MTOK * (r / 16);
@@ -349,7 +340,7 @@ __global__ __launch_bounds__(1024) void mla_qb_kernel(MlaPrologArgs a)
         const int s = grp + QB_GROUPS * j;
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
-            u32x2* d = reinterpret_cast<u32x2*>(wl + (srow + 32 * i) * QROW + 16 * spc);
+            u32x2* d = reinterpret_cast<u32x2*>(wl + (srow + 32 * i) * MQROW + 16 * spc);
             d[0] = u32x2{stg[j][i][0], stg[j][i][1]};
             d[1] = u32x2{stg[j][i][2], stg[j][i][3]};
         }
@@ -367,8 +358,8 @@ __global__ __launch_bounds__(1024) void mla_qb_kernel(MlaPrologArgs a)
                 // output column i over rows 0 .. 7 - eight of its sixteen contraction bytes per read
 #pragma unroll
                 for (int nb = 0; nb < 2; ++nb) {
-                    const uint8_t* p = wl + (ks * 64 + 16 * g + (l16 >> 1)) * QROW + 32 * wave + 16 * nb + 8 * (l16 & 1);
-                    const v2i lo = lds_read_tr8(p), hi = lds_read_tr8(p + 8 * QROW);
+                    const uint8_t* p = wl + (ks * 64 + 16 * g + (l16 >> 1)) * MQROW + 32 * wave + 16 * nb + 8 * (l16 & 1);
+                    const v2i lo = lds_read_tr8(p), hi = lds_read_tr8(p + 8 * MQROW);
                     wf[nb] = i32x4{lo[0], lo[1], hi[0], hi[1]};
                 }
 #pragma unroll
@@ -392,7 +383,7 @@ __global__ __launch_bounds__(1024) void mla_qb_kernel(MlaPrologArgs a)
     if (grp > 0) return;
 #pragma unroll
     for (int og = 1; og < QB_GROUPS; ++og) {
-        const i32x4* red = reinterpret_cast<const i32x4*>(qb_lds + og * (QB_K * QROW));
+        const i32x4* red = reinterpret_cast<const i32x4*>(qb_lds + og * (QB_K * MQROW));
 #pragma unroll
         for (int nb = 0; nb < 2; ++nb)
 #pragma unroll
@@ -431,6 +422,42 @@ __global__ __launch_bounds__(1024) void mla_qb_kernel(MlaPrologArgs a)
             }
         }
     }
+}
+
+// grid (tokens), 256 lanes
+__global__ __launch_bounds__(256) void mla_norm_kernel(MlaPrologArgs a) { mla_norm_body(a, blockIdx.x); }
+
+// grid (n * 192 / 128, token tiles of 32), 1024 lanes
+__global__ __launch_bounds__(1024) void mla_qb_kernel(MlaPrologArgs a)
+{
+    extern __shared__ __align__(16) uint8_t qb_lds[];
+    mla_qb_body(a, blockIdx.x * 128, blockIdx.y * MTOK, qb_lds);
+}
+
+// ------------------------------------------------------------------------------------------------ fused with the indexer prolog
+// The fused operator runs the two prologs' per-token kernels side by side in one launch, and likewise the two int8
+// GEMMs on q_norm (192 + 64 workgroups at model sizes: one per compute unit); the indexer's x @ [w_k | w_proj] rides along
+// in mla_xa_kernel as three more output tiles.
+// grid (tokens, 2), 256 lanes: y = 0 the MLA norms and cache rows, y = 1 the indexer's key path and weights (128 lanes)
+__global__ __launch_bounds__(256) void fused_norm_kernel(MlaPrologArgs m, PrologArgs p)
+{
+    if (blockIdx.y == 0) {
+        mla_norm_body(m, blockIdx.x);
+    } else {
+        if (threadIdx.x >= 128) return; // the barriers inside are among the two remaining waves
+        prolog_k_body(p, blockIdx.x);
+    }
+}
+
+// grid (n * 192 / 128 + index heads, token tiles of 32), 1024 lanes
+__global__ __launch_bounds__(1024) void fused_qb_kernel(MlaPrologArgs m, PrologArgs p)
+{
+    extern __shared__ __align__(16) uint8_t fq_lds[];
+    const int nqb = m.n * MQH / 128;
+    if ((int)blockIdx.x < nqb)
+        mla_qb_body(m, blockIdx.x * 128, blockIdx.y * MTOK, fq_lds);
+    else
+        prolog_q_body(p, blockIdx.x - nqb, blockIdx.y * PTOK, fq_lds);
 }
 
 // ------------------------------------------------------------------------------------------------ q_b[:, head, :128] @ w_uk[head]
@@ -476,53 +503,84 @@ bool mla_prolog_supported(int64_t h, int64_t r, int64_t n, int64_t d_nope, int64
 
 static uint64_t up256(uint64_t x) { return (x + 255) & ~(uint64_t)255; }
 
-uint64_t mla_prolog_workspace_bytes(int64_t t, int64_t h, int64_t r, int64_t n)
+static uint64_t xa_part_bytes(int64_t t, int64_t h, int64_t ncols)
 {
-    return up256((uint64_t)((h + XA_SPLIT - 1) / XA_SPLIT) * t * (r + MKV) * sizeof(float)) + up256((uint64_t)t * n * MNOPE * 2);
+    return up256((uint64_t)((h + XA_SPLIT - 1) / XA_SPLIT) * t * ncols * sizeof(float));
+}
+
+uint64_t mla_prolog_workspace_bytes(int64_t t, int64_t h, int64_t r, int64_t n, int64_t n_idx)
+{
+    return xa_part_bytes(t, h, r + MKV + (n_idx ? PD + n_idx : 0)) + up256((uint64_t)t * n * MNOPE * 2);
 }
 
 void mla_prolog_bind_workspace(MlaPrologArgs& a, void* ws)
 {
     uint8_t* p = static_cast<uint8_t*>(ws);
     a.xa_part = reinterpret_cast<float*>(p);
-    p += up256((uint64_t)a.ksplits * a.t * (a.r + MKV) * sizeof(float));
+    p += xa_part_bytes(a.t, a.h, a.ncols);
     a.qb_nope = reinterpret_cast<uint16_t*>(p);
 }
 
-hipError_t mla_prolog_launch(const MlaPrologArgs& a, hipStream_t stream)
+bool fused_prolog_supported(int64_t n_idx) { return n_idx % 64 == 0; }
+
+void fused_prolog_bind(MlaPrologArgs& m, PrologArgs& p, void* ws)
+{
+    m.w_k = p.w_k;
+    m.w_proj = p.w_proj;
+    m.n_idx = p.n;
+    m.ncols = m.r + MKV + PD + p.n;
+    mla_prolog_bind_workspace(m, ws);
+    p.xw_part = m.xa_part;
+    p.xw_stride = m.ncols;
+    p.xw_col0 = m.r + MKV;
+    p.ksplits = m.ksplits;
+}
+
+static hipError_t set_lds_limits()
+{
+    static bool done = false;
+    if (done) return hipSuccess;
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(mla_xa_kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                       4 * XA_K * XROW2);
+    if (e != hipSuccess) return e;
+    e = hipFuncSetAttribute(reinterpret_cast<const void*>(mla_qb_kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
+                            mla_qb_lds_bytes(MAX_R));
+    if (e != hipSuccess) return e;
+    e = hipFuncSetAttribute(reinterpret_cast<const void*>(fused_qb_kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
+                            mla_qb_lds_bytes(MAX_R) > prolog_q_lds_bytes(QMAX_R) ? mla_qb_lds_bytes(MAX_R) : prolog_q_lds_bytes(QMAX_R));
+    if (e != hipSuccess) return e;
+    done = true;
+    return hipSuccess;
+}
+
+// p == nullptr: the MLA prolog on its own; otherwise the fused operator (m and p bound by fused_prolog_bind)
+static hipError_t launch_prologs(const MlaPrologArgs& a, const PrologArgs* p, hipStream_t stream)
 {
     if (a.t == 0) return hipSuccess;
     const int ttiles = (a.t + MTOK - 1) / MTOK;
-    hipError_t e;
+    hipError_t e = set_lds_limits();
+    if (e != hipSuccess) return e;
     {
-        const int smem = 4 * XA_K * XROW2;
-        static bool attr_done = false;
-        if (!attr_done) {
-            e = hipFuncSetAttribute(reinterpret_cast<const void*>(mla_xa_kernel), hipFuncAttributeMaxDynamicSharedMemorySize, smem);
-            if (e != hipSuccess) return e;
-            attr_done = true;
-        }
-        const int tiles = (a.r + MKV) / 64;
         ScopedKernelTimer tm(KID_MLA_XA, stream);
-        hipLaunchKernelGGL(mla_xa_kernel, dim3(a.ksplits, tiles, ttiles), dim3(1024), smem, stream, a);
+        hipLaunchKernelGGL(mla_xa_kernel, dim3(a.ksplits, a.ncols / 64, ttiles), dim3(1024), 4 * XA_K * XROW2, stream, a);
     }
     if ((e = hipGetLastError()) != hipSuccess) return e;
     {
         ScopedKernelTimer tm(KID_MLA_NORM, stream);
-        hipLaunchKernelGGL(mla_norm_kernel, dim3(a.t), dim3(256), 0, stream, a);
+        if (p)
+            hipLaunchKernelGGL(fused_norm_kernel, dim3(a.t, 2), dim3(256), 0, stream, a, *p);
+        else
+            hipLaunchKernelGGL(mla_norm_kernel, dim3(a.t), dim3(256), 0, stream, a);
     }
     if ((e = hipGetLastError()) != hipSuccess) return e;
     {
-        const int smem = QB_GROUPS * QB_K * QROW + MTOK * (a.r + 16);
-        static bool attr_done = false;
-        if (!attr_done) {
-            e = hipFuncSetAttribute(reinterpret_cast<const void*>(mla_qb_kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
-                                    QB_GROUPS * QB_K * QROW + MTOK * (MAX_R + 16));
-            if (e != hipSuccess) return e;
-            attr_done = true;
-        }
         ScopedKernelTimer tm(KID_MLA_QB, stream);
-        hipLaunchKernelGGL(mla_qb_kernel, dim3(a.n * MQH / 128, ttiles), dim3(1024), smem, stream, a);
+        if (p) {
+            const int smem = mla_qb_lds_bytes(a.r) > prolog_q_lds_bytes(a.r) ? mla_qb_lds_bytes(a.r) : prolog_q_lds_bytes(a.r);
+            hipLaunchKernelGGL(fused_qb_kernel, dim3(a.n * MQH / 128 + p->n, ttiles), dim3(1024), smem, stream, a, *p);
+        } else {
+            hipLaunchKernelGGL(mla_qb_kernel, dim3(a.n * MQH / 128, ttiles), dim3(1024), mla_qb_lds_bytes(a.r), stream, a);
+        }
     }
     if ((e = hipGetLastError()) != hipSuccess) return e;
     {
@@ -530,6 +588,13 @@ hipError_t mla_prolog_launch(const MlaPrologArgs& a, hipStream_t stream)
         hipLaunchKernelGGL(mla_wuk_kernel, dim3(a.n, MC / 128, ttiles), dim3(256), 0, stream, a);
     }
     return hipGetLastError();
+}
+
+hipError_t mla_prolog_launch(const MlaPrologArgs& a, hipStream_t stream) { return launch_prologs(a, nullptr, stream); }
+
+hipError_t fused_prolog_launch(const MlaPrologArgs& m, const PrologArgs& p, hipStream_t stream)
+{
+    return launch_prologs(m, &p, stream);
 }
 
 } // namespace pto

@@ -1,7 +1,10 @@
 """GPU parity: fused MLA prolog + lightning-indexer prolog (HIP, through the C ABI).
 
-Two bars.  (1) Plumbing: the fused call must give, bit for bit, what the two operators give when called one after the
-other with the MLA prolog's q_norm / q_norm_scale handed over by the caller.  (2) Against the oracle's composition of
+Two bars.  (1) Plumbing: the fused call must give what the two operators give when called one after the other with the
+MLA prolog's q_norm / q_norm_scale handed over by the caller - bit for bit for every MLA output and for the indexer's
+query (integer GEMM, same epilogue); the indexer's key path and weights sum x @ [w_k | w_proj] in a different order when
+fused (the product rides along in the MLA prolog's first kernel), so there: int8 within 1, fp16 within one bf16 step.
+(2) Against the oracle's composition of
 the two goldens: the MLA outputs as in test_gpu_mla_prolog; the indexer outputs inherit the (rare, one-step) q_norm
 differences of the MLA stage, which is why the reference widens q_int8's tolerance to 2 here
 (deepseekv32_mla_indexer_prolog_quant.py:824): int8 within 2 everywhere and equal in at least 95 % of the places, scales
@@ -94,7 +97,20 @@ def check_against_oracle(mla_case, idx_case, got):
     close(got["q_scale"], gi["q_scale"], "q_scale")
     ints(got["k_cache"].view(-1, 128)[rows], gi["k_cache"].view(-1, 128)[rows], "idx k_int8", 1, 0.98)
     close(got["idx_k_scale_cache"].view(-1)[rows], gi["k_scale_cache"].view(-1)[rows], "idx k_scale")
-    close(got["weights"], gi["weights"], "weights")
+    close(got["weights"], gi["weights"], "weights", atol=2e-6)
+
+
+def same_as_separate(fused, sep):
+    for k, v in fused.items():
+        if k in ("k_cache", "idx_k_scale_cache", "weights"):
+            continue
+        assert torch.equal(v, sep[k]), f"{k}: fused and separate calls differ"
+    assert (fused["k_cache"].int() - sep["k_cache"].int()).abs().max() <= 1
+    assert (fused["k_cache"] == sep["k_cache"]).float().mean() >= 0.999
+    for k in ("idx_k_scale_cache", "weights"):
+        a, b = fused[k].float(), sep[k].float()
+        # weights near zero are sums that cancel: there the summation order shows at the fp32 level of the 7168 terms
+        assert ((a - b).abs() <= 2.0 ** -7 * b.abs() + 2e-6).all(), k
 
 
 def test_reference_case_b4_s2_fused_equals_separate_and_oracle(cuda):
@@ -102,18 +118,25 @@ def test_reference_case_b4_s2_fused_equals_separate_and_oracle(cuda):
     mla_case, idx_case = op.make_fused_case(4, 2, 1024, seed=21)
     fused = run_fused(mla_case, idx_case, cuda)
     sep = run_separate(mla_case, idx_case, cuda)
-    for k, v in fused.items():
-        assert torch.equal(v, sep[k]), f"{k}: fused and separate calls differ"
+    same_as_separate(fused, sep)
     check_against_oracle(mla_case, idx_case, fused)
 
 
 def test_prefill_entry_ragged_tiles_small_sizes(cuda):
-    mla_case, idx_case = op.make_fused_case(37, 1, 300, seed=22, n_idx=32, h=512, q_lora_rank=256, n=4)
+    mla_case, idx_case = op.make_fused_case(37, 1, 300, seed=22, n_idx=64, h=512, q_lora_rank=256, n=4)
     fused = run_fused(mla_case, idx_case, cuda, entry="mla_indexer_prolog_quant_p")
+    sep = run_separate(mla_case, idx_case, cuda)
+    same_as_separate(fused, sep)
+    check_against_oracle(mla_case, idx_case, fused)
+
+
+def test_index_head_counts_without_the_side_by_side_kernels(cuda):
+    # 32 index heads: x @ w_proj is half an output tile wide, so the fused entry runs the two operators back to back
+    mla_case, idx_case = op.make_fused_case(5, 1, 300, seed=23, n_idx=32, h=512, q_lora_rank=256, n=4)
+    fused = run_fused(mla_case, idx_case, cuda)
     sep = run_separate(mla_case, idx_case, cuda)
     for k, v in fused.items():
         assert torch.equal(v, sep[k]), f"{k}: fused and separate calls differ"
-    check_against_oracle(mla_case, idx_case, fused)
 
 
 def test_errors(cuda):
