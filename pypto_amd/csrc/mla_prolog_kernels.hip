@@ -198,14 +198,19 @@ __device__ __forceinline__ void mla_norm_body(const MlaPrologArgs& a, int tok)
             cj[j] = min(256 * j + tid, ncols - 1);
             sum[j] = 0.f;
         }
-#pragma unroll 4
-        for (int sp = 0; sp < a.ksplits; ++sp) {
-            const float* p = a.xa_part + ((int64_t)sp * a.t + tok) * a.ncols;
-            float v[NJ];
+        // four splits' loads in flight together (a split past the end re-reads the last one and adds zero)
+        for (int s0 = 0; s0 < a.ksplits; s0 += 4) {
+            float v[4][NJ];
 #pragma unroll
-            for (int j = 0; j < NJ; ++j) v[j] = p[cj[j]];
+            for (int i = 0; i < 4; ++i) {
+                const float* p = a.xa_part + ((int64_t)min(s0 + i, a.ksplits - 1) * a.t + tok) * a.ncols;
 #pragma unroll
-            for (int j = 0; j < NJ; ++j) sum[j] += v[j];
+                for (int j = 0; j < NJ; ++j) v[i][j] = p[cj[j]];
+            }
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+#pragma unroll
+                for (int j = 0; j < NJ; ++j) sum[j] += s0 + i < a.ksplits ? v[i][j] : 0.f;
         }
 #pragma unroll
         for (int j = 0; j < NJ; ++j)

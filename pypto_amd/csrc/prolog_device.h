@@ -265,12 +265,21 @@ __device__ __forceinline__ void prolog_k_body(const PrologArgs& a, int tok)
     for (int k = 0; k < PD; ++k) hk[k] = a.had_k[k * PD + tid];
     float kv = 0.f, wv = 0.f;
     const int wcol = PD + min(tid, a.n - 1);
-#pragma unroll 4
-    for (int s = 0; s < a.ksplits; ++s) {
-        const float* p = a.xw_part + ((int64_t)s * a.t + tok) * a.xw_stride + a.xw_col0;
-        const float v0 = p[tid], v1 = p[wcol];
-        kv += v0;
-        wv += v1;
+    // sixteen splits' loads in flight together (a split past the end re-reads the last one and adds zero); the order
+    // of the additions is the order of the splits
+    for (int s0 = 0; s0 < a.ksplits; s0 += 16) {
+        float v0[16], v1[16];
+#pragma unroll
+        for (int j = 0; j < 16; ++j) {
+            const float* p = a.xw_part + ((int64_t)min(s0 + j, a.ksplits - 1) * a.t + tok) * a.xw_stride + a.xw_col0;
+            v0[j] = p[tid];
+            v1[j] = p[wcol];
+        }
+#pragma unroll
+        for (int j = 0; j < 16; ++j) {
+            kv += s0 + j < a.ksplits ? v0[j] : 0.f;
+            wv += s0 + j < a.ksplits ? v1[j] : 0.f;
+        }
     }
     // LayerNorm in fp32 (biased variance), -> bf16
     const float mean = block_sum128(kv, red) / (float)PD;

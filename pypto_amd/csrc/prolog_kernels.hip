@@ -12,13 +12,13 @@
 //
 // At decode sizes (tens of tokens) the operator streams 15 MB of weights once and is bound by that read and by launch
 // latency, not by the matrix cores; the kernels are laid out for coalesced weight reads:
-//   prolog_q_kernel          one workgroup of 1024 lanes per (head, 32 tokens): int8 MFMA GEMM over r - w_qb has the
+//   prolog_qx_kernel         one workgroup of 1024 lanes per (head, 32 tokens): int8 MFMA GEMM over r - w_qb has the
 //                            output dimension contiguous, so its tile (r x 128 bytes, every load issued at once) goes
 //                            through LDS and is read back with 8-bit transposing reads; four wave groups split the
 //                            contraction and add their int32 sums through LDS - then, on the first group, scale and
 //                            round to bf16 into LDS, rotary in LDS, hadamard as a bf16 MFMA (matrix read with 16-bit
 //                            transposing LDS reads), quantisation
-//   prolog_xw_kernel         x @ [w_k | w_proj] split over the contraction (256 rows of the weights per workgroup, staged
+//   (same launch)            x @ [w_k | w_proj] split over the contraction (256 rows of the weights per workgroup, staged
 //                            in LDS and read with transposing reads); fp32 partials to the workspace
 //   prolog_k_kernel          one workgroup per token: sums the partials in a fixed order, LayerNorm, rotary, hadamard,
 //                            quantisation, cache write, weights
@@ -33,24 +33,17 @@
 namespace pto {
 namespace {
 
-// grid (heads, token tiles of 32), 1024 lanes
-__global__ __launch_bounds__(1024) void prolog_q_kernel(PrologArgs a)
-{
-    extern __shared__ __align__(16) uint8_t plds[];
-    prolog_q_body(a, blockIdx.x, blockIdx.y * PTOK, plds);
-}
 
 // grid (tokens), 128 lanes
 __global__ __launch_bounds__(128) void prolog_k_kernel(PrologArgs a) { prolog_k_body(a, blockIdx.x); }
 
 // ------------------------------------------------------------------------------------------------ x @ [w_k | w_proj]
-// grid (h / 256, token tiles of 32), 256 lanes; partial sums over this workgroup's 256 rows of the weights
-__global__ __launch_bounds__(256) void prolog_xw_kernel(PrologArgs a)
+// 256 lanes per (256 rows of the weights, token tile of 32): partial sums over those rows; wl is [256 k][nw] bf16,
+// nw = 128 + n
+__device__ __forceinline__ void prolog_xw_body(const PrologArgs& a, int split, int tok0, uint8_t* wl)
 {
-    extern __shared__ __align__(16) uint8_t wl[]; // [256 k][nw] bf16, nw = 128 + n
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int l32 = lane & 31, hl = lane >> 5;
-    const int split = blockIdx.x, tok0 = blockIdx.y * PTOK;
     const int nw = PD + a.n, rowb = nw * 2;
     const int64_t kbase = (int64_t)split * XW_K;
     // stage the weights: w_k rows then w_proj rows, 16-byte pieces
@@ -108,6 +101,19 @@ __global__ __launch_bounds__(256) void prolog_xw_kernel(PrologArgs a)
     }
 }
 
+// The query path and x @ [w_k | w_proj] do not depend on each other: one launch runs them side by side.
+// grid (heads + h / 256, token tiles of 32), 1024 lanes (the workgroups of the second kind use their first 256)
+__global__ __launch_bounds__(1024) void prolog_qx_kernel(PrologArgs a)
+{
+    extern __shared__ __align__(16) uint8_t plds[];
+    if ((int)blockIdx.x < a.n) {
+        prolog_q_body(a, blockIdx.x, blockIdx.y * PTOK, plds);
+    } else {
+        if (threadIdx.x >= 256) return; // the barrier inside is among the remaining four waves
+        prolog_xw_body(a, blockIdx.x - a.n, blockIdx.y * PTOK, plds);
+    }
+}
+
 } // namespace
 
 bool prolog_supported(int64_t h, int64_t r, int64_t n, int64_t d, int64_t rope)
@@ -135,23 +141,18 @@ hipError_t prolog_launch(const PrologArgs& a, hipStream_t stream)
     const int ttiles = (a.t + PTOK - 1) / PTOK;
     hipError_t e;
     static bool attr_done = false;
+    constexpr int xw_lds_max = XW_K * (PD + 128) * 2;
     if (!attr_done) {
-        e = hipFuncSetAttribute(reinterpret_cast<const void*>(prolog_q_kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
-                                prolog_q_lds_bytes(QMAX_R));
-        if (e != hipSuccess) return e;
-        e = hipFuncSetAttribute(reinterpret_cast<const void*>(prolog_xw_kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
-                                XW_K * (PD + 128) * 2);
+        e = hipFuncSetAttribute(reinterpret_cast<const void*>(prolog_qx_kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                prolog_q_lds_bytes(QMAX_R) > xw_lds_max ? prolog_q_lds_bytes(QMAX_R) : xw_lds_max);
         if (e != hipSuccess) return e;
         attr_done = true;
     }
     {
+        const int xw_lds = XW_K * (PD + a.n) * 2;
+        const int smem = prolog_q_lds_bytes(a.r) > xw_lds ? prolog_q_lds_bytes(a.r) : xw_lds;
         ScopedKernelTimer tm(KID_PROLOG_Q, stream);
-        hipLaunchKernelGGL(prolog_q_kernel, dim3(a.n, ttiles), dim3(1024), prolog_q_lds_bytes(a.r), stream, a);
-    }
-    if ((e = hipGetLastError()) != hipSuccess) return e;
-    {
-        ScopedKernelTimer tm(KID_PROLOG_XW, stream);
-        hipLaunchKernelGGL(prolog_xw_kernel, dim3(a.ksplits, ttiles), dim3(256), XW_K * (PD + a.n) * 2, stream, a);
+        hipLaunchKernelGGL(prolog_qx_kernel, dim3(a.n + a.ksplits, ttiles), dim3(1024), smem, stream, a);
     }
     if ((e = hipGetLastError()) != hipSuccess) return e;
     {
