@@ -285,9 +285,9 @@ const char* pto_last_error(void);
  * is bracketed by a HIP event pair recorded on the launch stream; pto_kernel_timing_read waits for the
  * events recorded so far for one kernel, returns their summed duration and count, and forgets them.
  * Kernel ids: 0 indexer_score_kernel, 1 indexer_topk_kernel, 2 sfa_decode_kernel, 3 sfa_combine_kernel,
- * 4 indexer_select_kernel, 5 select_experts_kernel, 6 gqa_decode_kernel, 7 gqa_combine_kernel, 8 (unused),
- * 9 prolog_q_kernel, 10 prolog_xw_kernel, 11 prolog_k_kernel, 12 mla_xa_kernel, 13 mla_norm_kernel, 14 mla_qb_kernel,
- * 15 mla_wuk_kernel
+ * 4 indexer_select_kernel, 5 select_experts_kernel, 6 gqa_decode_kernel, 7 gqa_combine_kernel, 8 unused,
+ * 9 prolog_qx_kernel, 10 unused, 11 prolog_k_kernel, 12 mla_xa_kernel, 13 mla_norm_kernel (fused_norm_kernel in the fused
+ * prolog), 14 mla_qb_kernel (fused_qb_kernel in the fused prolog), 15 mla_wuk_kernel
  * (pto_kernel_name returns "" past the last id).
  * Off by default; not for use under graph capture.
  */

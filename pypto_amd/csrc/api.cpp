@@ -789,8 +789,8 @@ const char* pto_kernel_name(int kernel_id)
 {
     static const char* names[] = {"indexer_score_kernel", "indexer_topk_kernel", "sfa_decode_kernel",
                                   "sfa_combine_kernel", "indexer_select_kernel", "select_experts_kernel",
-                                  "gqa_decode_kernel", "gqa_combine_kernel", "prolog_transpose_kernel", "prolog_q_kernel",
-                                  "prolog_xw_kernel", "prolog_k_kernel", "mla_xa_kernel", "mla_norm_kernel", "mla_qb_kernel",
+                                  "gqa_decode_kernel", "gqa_combine_kernel", "unused", "prolog_qx_kernel", "unused",
+                                  "prolog_k_kernel", "mla_xa_kernel", "mla_norm_kernel", "mla_qb_kernel",
                                   "mla_wuk_kernel"};
     return kernel_id >= 0 && kernel_id < pto::KID_COUNT ? names[kernel_id] : "";
 }
