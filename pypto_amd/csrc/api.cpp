@@ -660,6 +660,7 @@ int pto_indexer_prolog_launch(const PtoTensorDesc* tensors, uint32_t n_tensors, 
     PrologPlan plan;
     int rc = plan_prolog(tensors, n_tensors, params, &plan);
     if (rc) return rc;
+    if (plan.args.t == 0) return PTO_OK;
     if (workspace == nullptr || workspace_bytes < plan.ws_bytes)
         return fail(PTO_ERR_WORKSPACE, "%s: workspace of %llu bytes required, got %llu", op,
                     (unsigned long long)plan.ws_bytes, (unsigned long long)(workspace ? workspace_bytes : 0));

@@ -139,6 +139,22 @@ def test_index_head_counts_without_the_side_by_side_kernels(cuda):
         assert torch.equal(v, sep[k]), f"{k}: fused and separate calls differ"
 
 
+def test_no_tokens_is_a_no_op(cuda):
+    """An empty batch (t = 0) is accepted by all three prolog entries and touches nothing."""
+    mla_case, idx_case = op.make_fused_case(2, 1, 256, seed=24, n_idx=64, h=512, q_lora_rank=256, n=4)
+    for k in ("x", "cos", "sin", "cache_index"):
+        mla_case[k] = mla_case[k][:0].contiguous()
+    idx_case.update(x=mla_case["x"], cos=mla_case["cos"], sin=mla_case["sin"], k_cache_index=mla_case["cache_index"])
+    fused = run_fused(mla_case, idx_case, cuda)
+    sep = run_separate(mla_case, idx_case, cuda)
+    for got in (fused, sep):
+        assert torch.equal(got["kv_cache"], mla_case["kv_cache"]) and torch.equal(got["kr_cache"], mla_case["kr_cache"])
+        assert torch.equal(got["k_scale_cache"], mla_case["k_scale_cache"])
+        assert torch.equal(got["k_cache"], idx_case["k_cache"])
+        assert torch.equal(got["idx_k_scale_cache"], idx_case["k_scale_cache"])
+        assert got["q_nope"].shape == (0, 4, 512) and got["q_int8"].shape == (0, 64, 128)
+
+
 def test_errors(cuda):
     from pypto_amd.error import FeError
     mla_case, idx_case = op.make_fused_case(2, 1, 256, seed=1, n_idx=32, h=512, q_lora_rank=256, n=4)
