@@ -217,9 +217,9 @@ typedef struct {
 } PtoMlaPrologParams;
 
 /*
- * mla_prolog_quant_d and mla_prolog_quant_p, int8 form (models/deepseek_v32_exp/mla_prolog_quant_impl.py:745-951, compute
- * :520-727; the decode and the prefill entry of the reference differ in Ascend pass options only).  tensors[21] in the
- * reference's argument order:
+ * mla_prolog_quant_d and mla_prolog_quant_p (models/deepseek_v32_exp/mla_prolog_quant_impl.py:745-951, compute :520-727;
+ * the decode and the prefill entry of the reference differ in Ascend pass options only).  tensors[21] in the reference's
+ * argument order, int8 form:
  *    0 token_x           [t, h]                  BF16   (h a multiple of 256)
  *    1 w_dq              [h, r]                  BF16   (r a multiple of 128, at most 2048; plain row-major - the
  *                                                        reference's Ascend NZ tiling is a device format)
@@ -240,7 +240,9 @@ typedef struct {
  *   16 query_nope_out    [t, n, 512]             BF16   (output)
  *   17 query_rope_out    [t, n, 64]              BF16   (output)
  *   18-20 kv_cache_out, kr_cache_out, k_scale_cache_out: the buffers of 11-13 again
- * The bf16 form of the reference (empty dequant_scale, BF16 w_uq_qr and kv_cache) is not built and is rejected.
+ * bf16 form (the reference's "is_quant" False, :578-581): dequant_scale with no elements (rank 1 or 2), and w_uq_qr,
+ * kv_cache, q_norm_out, kv_cache_out all BF16 - no quantisation anywhere: q_norm_out is the RmsNorm output, the kv cache row
+ * the normalised key; k_scale_cache and q_norm_scale_out are not touched; q_lora_rank must then be a multiple of 256.
  */
 uint64_t pto_mla_prolog_quant_workspace(const PtoTensorDesc* tensors, uint32_t n_tensors,
                                         const PtoMlaPrologParams* params);

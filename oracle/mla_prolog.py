@@ -1,8 +1,10 @@
-"""CPU restatement of the reference's MLA prolog golden, int8 ("quant_b") form (test infrastructure only).
+"""CPU restatement of the reference's MLA prolog golden (test infrastructure only).
 
 Follows ``mla_prolog_quant_v32_compute`` and its helpers in models/deepseek_v32_exp/deepseekv32_mla_prolog_quant.py
-(:32-124 helpers, :131-283 compute, :285-441 generators) with is_quant_a False, is_quant_b True, no smoothing - the
-configuration of the reference's quantised tests (:700-812).  The operator turns hidden states into everything sparse
+(:32-124 helpers, :131-283 compute, :285-441 generators) with is_quant_a False, no smoothing, and is_quant_b True (the
+int8 form of the reference's quantised tests, :700-812, described below) or False (the bf16 form of its tests
+:815-938: no quantisation anywhere - q_norm is the RmsNorm output itself, w_uq_qr is bf16, the kv cache holds the
+normalised key in bf16 and the scale tensors are not touched).  The operator turns hidden states into everything sparse
 flash attention reads:
   query : x @ w_dq (fp32 -> bf16) -> RmsNorm(gamma_cq) -> per-token int8 quantisation (q_norm, q_norm_scale: also the
           inputs of the lightning-indexer prolog) -> int8 GEMM with w_uq_qr (exact int32) * token scale * channel scale
@@ -64,14 +66,18 @@ def _scatter(cache, rows, index):
 
 
 def query_tail(inp, q_norm, q_norm_scale):
-    """The query path downstream of the quantised RmsNorm: q_nope [t, n, 512] and q_rope [t, n, 64] from q_norm,
-    q_norm_scale (tests also call it with the product's own q_norm to check the downstream stages on their own)."""
+    """The query path downstream of the (quantised) RmsNorm: q_nope [t, n, 512] and q_rope [t, n, 64] from q_norm,
+    q_norm_scale (tests also call it with the product's own q_norm to check the downstream stages on their own).
+    q_norm_scale None: the bf16 form."""
     t = q_norm.shape[0]
     n, d_nope, c = inp["w_uk"].shape
     d_rope = inp["cos"].shape[1]
     dt = inp["x"].dtype
-    qb = torch.matmul(q_norm.to(torch.int32), inp["w_uq_qr"].to(torch.int32)).float()          # :205-210
-    qb = (qb * q_norm_scale) * inp["w_qb_scale"].reshape(1, -1)                                # :211-212
+    if q_norm_scale is None:
+        qb = torch.matmul(q_norm.float(), inp["w_uq_qr"].float())                              # :214
+    else:
+        qb = torch.matmul(q_norm.to(torch.int32), inp["w_uq_qr"].to(torch.int32)).float()      # :205-210
+        qb = (qb * q_norm_scale) * inp["w_qb_scale"].reshape(1, -1)                            # :211-212
     qb = qb.to(dt).reshape(t, n, d_nope + d_rope)                                              # :216-218
     q_nope = torch.matmul(qb[:, :, :d_nope].permute(1, 0, 2).float(), inp["w_uk"].float())     # :220-225
     q_nope = q_nope.to(dt).permute(1, 0, 2).contiguous()                                       # :226-228
@@ -86,21 +92,26 @@ def mla_prolog(inp, eps_cq=None, eps_ckv=None):
     t = x.shape[0]
     n, d_nope, c = inp["w_uk"].shape
     d_rope = inp["cos"].shape[1]
+    quant_b = inp["w_uq_qr"].dtype == torch.int8
     qa = torch.matmul(x.float(), inp["w_dq"].float()).to(torch.bfloat16)                       # :192-194
     qn = rms_norm(qa, inp["gamma_cq"], eps_cq)                                                 # :196
-    q_norm, q_norm_scale = quant(qn, True)                                                     # :204
+    q_norm, q_norm_scale = quant(qn, True) if quant_b else (qn, None)                          # :204
     q_nope, q_rope = query_tail(inp, q_norm, q_norm_scale)
 
     kv = torch.matmul(x.float(), inp["w_dkv_kr"].float()).to(x.dtype)                          # :243-247
     ckv = rms_norm(kv[:, :c], inp["gamma_ckv"], eps_ckv)                                       # :250-251
-    k_nope, k_scale = quant(ckv.reshape(t, 4, c // 4), True)                                   # :254-256
+    if quant_b:
+        k_nope, k_scale = quant(ckv.reshape(t, 4, c // 4), True)                               # :254-256
+    else:
+        k_nope, k_scale = ckv, None
     k_rope = rope_interleaved(kv[:, c:].reshape(t, 1, d_rope), inp["cos"], inp["sin"]).reshape(t, d_rope)
     idx = inp["cache_index"]
     return {
         "q_norm": q_norm, "q_norm_scale": q_norm_scale, "q_nope": q_nope, "q_rope": q_rope,
         "kv_cache": _scatter(inp["kv_cache"], k_nope.reshape(t, c), idx),                      # :275-276
         "kr_cache": _scatter(inp["kr_cache"], k_rope, idx),                                    # :279-280
-        "k_scale_cache": _scatter(inp["k_scale_cache"], k_scale.reshape(t, 4), idx),           # :282-287
+        "k_scale_cache": (_scatter(inp["k_scale_cache"], k_scale.reshape(t, 4), idx)           # :282-287
+                          if quant_b else inp["k_scale_cache"].clone()),
     }
 
 
@@ -113,15 +124,19 @@ def intermediates(inp, eps_cq=None, eps_ckv=None):
     n, d_nope, c = inp["w_uk"].shape
     qa = torch.matmul(x.float(), inp["w_dq"].float()).to(torch.bfloat16)
     qn = rms_norm(qa, inp["gamma_cq"], eps_cq)
-    q_norm, q_norm_scale = quant(qn, True)
-    qb = torch.matmul(q_norm.to(torch.int32), inp["w_uq_qr"].to(torch.int32)).float()
-    qb = ((qb * q_norm_scale) * inp["w_qb_scale"].reshape(1, -1)).to(x.dtype).reshape(t, n, -1)
+    if inp["w_uq_qr"].dtype == torch.int8:
+        q_norm, q_norm_scale = quant(qn, True)
+        qb = torch.matmul(q_norm.to(torch.int32), inp["w_uq_qr"].to(torch.int32)).float()
+        qb = ((qb * q_norm_scale) * inp["w_qb_scale"].reshape(1, -1)).to(x.dtype).reshape(t, n, -1)
+    else:
+        qb = torch.matmul(qn.float(), inp["w_uq_qr"].float()).to(x.dtype).reshape(t, n, -1)
     kv = torch.matmul(x.float(), inp["w_dkv_kr"].float()).to(x.dtype)
     ckv = rms_norm(kv[:, :c], inp["gamma_ckv"], eps_ckv)
     return {"q_a": qa, "q_rms": qn, "q_b": qb, "kv": kv, "kv_rms": ckv}
 
 
-def make_case(b, s1, s2, seed=5, h=7168, q_lora_rank=1536, n=128, d_nope=128, d_rope=64, c=512, block_size=128):
+def make_case(b, s1, s2, seed=5, h=7168, q_lora_rank=1536, n=128, d_nope=128, d_rope=64, c=512, block_size=128,
+              quant_b=True):
     """The reference generator's distributions (:331-441): x U[-1,1), weights U[-0.1,0.1) (w_uq_qr then quantised per
     output channel), gammas U[-1,1), cos/sin U[-0.1,0.1), caches filled from U[-1,1) data (the kv part quantised per
     group of 128); the last s1 positions of each length-s2 sequence are the new tokens (:299-313)."""
@@ -132,7 +147,10 @@ def make_case(b, s1, s2, seed=5, h=7168, q_lora_rank=1536, n=128, d_nope=128, d_
     def uni(lo, hi, *shape):
         return torch.rand(shape, generator=g) * (hi - lo) + lo
 
-    w_uq_qr, w_qb_scale = quant(uni(-0.1, 0.1, q_lora_rank, n * (d_nope + d_rope)).to(bf), False)
+    w_uq_qr = uni(-0.1, 0.1, q_lora_rank, n * (d_nope + d_rope)).to(bf)
+    w_qb_scale = torch.zeros((0,), dtype=torch.float32)          # the bf16 form passes an empty dequant_scale (:613)
+    if quant_b:
+        w_uq_qr, w_qb_scale = quant(w_uq_qr, False)
     inp = {
         "x": uni(-1, 1, t, h).to(bf),
         "w_dq": uni(-0.1, 0.1, h, q_lora_rank).to(bf),
@@ -150,9 +168,13 @@ def make_case(b, s1, s2, seed=5, h=7168, q_lora_rank=1536, n=128, d_nope=128, d_
     table = torch.randperm(n_pages, generator=g).to(torch.int32).reshape(b, pages_per_seq)
     inp["block_table"] = table
     kv_old = uni(-1, 1, n_pages * block_size, 4, c // 4).to(bf)
-    kv_q, kv_s = quant(kv_old, True)
-    inp["kv_cache"] = kv_q.reshape(n_pages, block_size, 1, c)
-    inp["k_scale_cache"] = kv_s.reshape(n_pages, block_size, 1, 4).contiguous()
+    if quant_b:
+        kv_q, kv_s = quant(kv_old, True)
+        inp["kv_cache"] = kv_q.reshape(n_pages, block_size, 1, c)
+        inp["k_scale_cache"] = kv_s.reshape(n_pages, block_size, 1, 4).contiguous()
+    else:
+        inp["kv_cache"] = kv_old.reshape(n_pages, block_size, 1, c).contiguous()
+        inp["k_scale_cache"] = torch.zeros((n_pages, block_size, 1, 4), dtype=torch.float32)          # :603-606
     inp["kr_cache"] = uni(-1, 1, n_pages, block_size, 1, d_rope).to(bf)
     idx = torch.empty((b, s1), dtype=torch.int64)
     for i in range(b):

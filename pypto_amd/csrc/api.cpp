@@ -441,15 +441,22 @@ int plan_mla_prolog(const PtoTensorDesc* ts, uint32_t n, const PtoMlaPrologParam
     if (p == nullptr) return fail(PTO_ERR_PARAM, "%s: params is null", op);
     if (p->cache_mode != PTO_CACHE_PA_BSND)
         return fail(PTO_ERR_PARAM, "%s: only cache mode PA_BSND (%d) is built, got %d", op, PTO_CACHE_PA_BSND, p->cache_mode);
-    if (ts[3].rank == 0 || ts[3].shape[0] == 0 || ts[2].dataType != PTO_DT_INT8)
-        return fail(PTO_ERR_DTYPE, "%s: only the int8 form (INT8 w_uq_qr with its dequant_scale, INT8 kv_cache) is built", op);
-    static const struct { const char* name; int dtype; int rank; } spec[21] = {
-        {"token_x", PTO_DT_BF16, 2}, {"w_dq", PTO_DT_BF16, 2}, {"w_uq_qr", PTO_DT_INT8, 2}, {"dequant_scale", PTO_DT_FP32, 2},
+    // int8 form: INT8 w_uq_qr with its dequant_scale, INT8 kv_cache and q_norm_out.  bf16 form: an empty dequant_scale,
+    // BF16 w_uq_qr, kv_cache and q_norm_out (k_scale_cache and q_norm_scale_out are then left untouched).
+    const bool quant = !(ts[3].rank >= 1 && ts[3].shape[0] == 0);
+    const int wdt = quant ? PTO_DT_INT8 : PTO_DT_BF16;
+    if (ts[3].rank < 1 || ts[3].rank > 2) return fail(PTO_ERR_SHAPE, "%s: dequant_scale must have rank 1 or 2", op);
+    if (ts[3].dataType != PTO_DT_FP32) return fail(PTO_ERR_DTYPE, "%s: dequant_scale must be fp32", op);
+    if (ts[2].dataType != wdt || ts[11].dataType != wdt || ts[14].dataType != wdt || ts[18].dataType != wdt)
+        return fail(PTO_ERR_DTYPE, "%s: with %s dequant_scale, w_uq_qr, kv_cache and q_norm_out must all be %s (int8 form: INT8 w_uq_qr with its dequant_scale, INT8 kv_cache; bf16 form: empty dequant_scale, BF16 throughout)",
+                    op, quant ? "a non-empty" : "an empty", dtype_name(wdt));
+    const struct { const char* name; int dtype; int rank; } spec[21] = {
+        {"token_x", PTO_DT_BF16, 2}, {"w_dq", PTO_DT_BF16, 2}, {"w_uq_qr", wdt, 2}, {"dequant_scale", PTO_DT_FP32, ts[3].rank},
         {"w_uk", PTO_DT_BF16, 3}, {"w_dkv_kr", PTO_DT_BF16, 2}, {"gamma_cq", PTO_DT_BF16, 1}, {"gamma_ckv", PTO_DT_BF16, 1},
-        {"cos", PTO_DT_BF16, 2}, {"sin", PTO_DT_BF16, 2}, {"cache_index", PTO_DT_INT64, 1}, {"kv_cache", PTO_DT_INT8, 4},
-        {"kr_cache", PTO_DT_BF16, 4}, {"k_scale_cache", PTO_DT_FP32, 4}, {"q_norm_out", PTO_DT_INT8, 2},
+        {"cos", PTO_DT_BF16, 2}, {"sin", PTO_DT_BF16, 2}, {"cache_index", PTO_DT_INT64, 1}, {"kv_cache", wdt, 4},
+        {"kr_cache", PTO_DT_BF16, 4}, {"k_scale_cache", PTO_DT_FP32, 4}, {"q_norm_out", wdt, 2},
         {"q_norm_scale_out", PTO_DT_FP32, 2}, {"query_nope_out", PTO_DT_BF16, 3}, {"query_rope_out", PTO_DT_BF16, 3},
-        {"kv_cache_out", PTO_DT_INT8, 4}, {"kr_cache_out", PTO_DT_BF16, 4}, {"k_scale_cache_out", PTO_DT_FP32, 4}};
+        {"kv_cache_out", wdt, 4}, {"kr_cache_out", PTO_DT_BF16, 4}, {"k_scale_cache_out", PTO_DT_FP32, 4}};
     int rc;
     for (int i = 0; i < 21; ++i)
         if ((rc = check_tensor(op, ts[i], spec[i].name, spec[i].dtype, spec[i].rank))) return rc;
@@ -459,9 +466,11 @@ int plan_mla_prolog(const PtoTensorDesc* ts, uint32_t n, const PtoMlaPrologParam
     if (!pto::mla_prolog_supported(h, r, nh, dn, rope, c))
         return fail(PTO_ERR_SHAPE, "%s: need w_uk [heads, 128, 512] with an even number of heads, rotary dim 64, q_lora_rank a multiple of 128 (at most 2048) and h a multiple of 256; got h %lld r %lld heads %lld nope %lld rotary %lld kv rank %lld",
                     op, (long long)h, (long long)r, (long long)nh, (long long)dn, (long long)rope, (long long)c);
+    if (!quant && r % 256 != 0)
+        return fail(PTO_ERR_SHAPE, "%s: the bf16 form needs q_lora_rank a multiple of 256, got %lld", op, (long long)r);
     const int64_t nq = nh * (dn + rope);
-    const bool ok = ts[1].shape[0] == h && ts[2].shape[0] == r && ts[2].shape[1] == nq && ts[3].shape[0] == nq &&
-                    ts[3].shape[1] == 1 && ts[5].shape[0] == h && ts[5].shape[1] == c + rope && ts[6].shape[0] == r &&
+    const bool ok = ts[1].shape[0] == h && ts[2].shape[0] == r && ts[2].shape[1] == nq &&
+                    (!quant || (ts[3].rank == 2 && ts[3].shape[0] == nq && ts[3].shape[1] == 1)) && ts[5].shape[0] == h && ts[5].shape[1] == c + rope && ts[6].shape[0] == r &&
                     ts[7].shape[0] == c && ts[8].shape[0] == t && ts[8].shape[1] == rope && ts[9].shape[0] == t &&
                     ts[10].shape[0] == t && ts[11].shape[2] == 1 && ts[11].shape[3] == c &&
                     ts[12].shape[0] == ts[11].shape[0] && ts[12].shape[1] == ts[11].shape[1] && ts[12].shape[2] == 1 &&
@@ -476,7 +485,9 @@ int plan_mla_prolog(const PtoTensorDesc* ts, uint32_t n, const PtoMlaPrologParam
     pto::MlaPrologArgs& a = plan->args;
     a.x = static_cast<const uint16_t*>(ts[0].addr);
     a.w_dq = static_cast<const uint16_t*>(ts[1].addr);
-    a.w_uq_qr = static_cast<const int8_t*>(ts[2].addr);
+    a.w_uq_qr = ts[2].addr;
+    a.quant = quant;
+    a.qb_part = nullptr;
     a.w_qb_scale = static_cast<const float*>(ts[3].addr);
     a.w_uk = static_cast<const uint16_t*>(ts[4].addr);
     a.w_dkv_kr = static_cast<const uint16_t*>(ts[5].addr);
@@ -506,7 +517,7 @@ int plan_mla_prolog(const PtoTensorDesc* ts, uint32_t n, const PtoMlaPrologParam
     a.ksplits = (int32_t)((h + 1023) / 1024);
     a.eps_cq = p->epsilon_cq;
     a.eps_ckv = p->epsilon_ckv;
-    plan->ws_bytes = pto::mla_prolog_workspace_bytes(t, h, r, nh, 0);
+    plan->ws_bytes = pto::mla_prolog_workspace_bytes(t, h, r, nh, 0, quant);
     return PTO_OK;
 }
 
@@ -550,6 +561,8 @@ int plan_fused_prolog(const PtoTensorDesc* ts, uint32_t n, const PtoMlaIndexerPr
     const PtoMlaPrologParams mp = {p->epsilon_cq, p->epsilon_ckv, p->cache_mode};
     int rc = plan_mla_prolog(m, 21, &mp, &plan->mla);
     if (rc) return rc;
+    if (!plan->mla.args.quant)
+        return fail(PTO_ERR_DTYPE, "%s: the fused operator exists in the int8 form only (INT8 mla_w_uq_qr with its dequant_scale)", op);
     q[0] = ts[0];
     q[1] = qn;
     q[2] = qs;
@@ -567,7 +580,7 @@ int plan_fused_prolog(const PtoTensorDesc* ts, uint32_t n, const PtoMlaIndexerPr
     if (rc) return rc;
     plan->fused = pto::fused_prolog_supported(plan->ip.args.n);
     if (plan->fused) { // the indexer's partial sums live inside the MLA prolog's: no workspace of its own
-        plan->mla.ws_bytes = pto::mla_prolog_workspace_bytes(t, plan->mla.args.h, r, plan->mla.args.n, plan->ip.args.n);
+        plan->mla.ws_bytes = pto::mla_prolog_workspace_bytes(t, plan->mla.args.h, r, plan->mla.args.n, plan->ip.args.n, true);
         plan->ip.ws_bytes = 0;
     }
     plan->off_ip_ws = up256(plan->mla.ws_bytes);

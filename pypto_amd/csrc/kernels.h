@@ -128,7 +128,7 @@ hipError_t prolog_launch(const PrologArgs& a, hipStream_t stream);
 struct MlaPrologArgs {
     const uint16_t* x;          // [t, h] bf16
     const uint16_t* w_dq;       // [h, r] bf16
-    const int8_t* w_uq_qr;      // [r, n*192]
+    const void* w_uq_qr;        // [r, n*192] int8 (bf16 in the bf16 form)
     const float* w_qb_scale;    // [n*192]
     const uint16_t* w_uk;       // [n, 128, 512] bf16
     const uint16_t* w_dkv_kr;   // [h, 576] bf16
@@ -137,10 +137,10 @@ struct MlaPrologArgs {
     const uint16_t* cos;        // [t, 64] bf16
     const uint16_t* sin;        // [t, 64] bf16
     const int64_t* cache_index; // [t]
-    int8_t* kv_cache;           // [cache_rows, 512], updated in place
+    int8_t* kv_cache;           // [cache_rows, 512] int8 (bf16 in the bf16 form), updated in place
     uint16_t* kr_cache;         // [cache_rows, 64] bf16, updated in place
     float* k_scale_cache;       // [cache_rows, 4], updated in place
-    int8_t* q_norm;             // [t, r]
+    int8_t* q_norm;             // [t, r] int8 (bf16 in the bf16 form)
     float* q_norm_scale;        // [t]
     uint16_t* q_nope;           // [t, n, 512] bf16
     uint16_t* q_rope;           // [t, n, 64] bf16
@@ -148,14 +148,16 @@ struct MlaPrologArgs {
     const uint16_t* w_proj;     // products with x ride along in the first kernel
     float* xa_part;             // workspace [ksplits, t, ncols]
     uint16_t* qb_nope;          // workspace [t, n, 128] bf16
+    float* qb_part;             // workspace, bf16 form only: [ceil(r / 1024), t, n*192] partial sums of q_norm @ w_uq_qr
     int64_t cache_rows;
     int32_t t, h, r, n, ksplits;
     int32_t n_idx, ncols;       // index heads (0: not fused); columns of a partial-sum row: r + 576 (+ 128 + n_idx)
     float eps_cq, eps_ckv;
+    bool quant;                 // int8 form (w_uq_qr int8 + scales, int8 cache) or bf16 form
 };
 
 bool mla_prolog_supported(int64_t h, int64_t r, int64_t n, int64_t d_nope, int64_t d_rope, int64_t c);
-uint64_t mla_prolog_workspace_bytes(int64_t t, int64_t h, int64_t r, int64_t n, int64_t n_idx);
+uint64_t mla_prolog_workspace_bytes(int64_t t, int64_t h, int64_t r, int64_t n, int64_t n_idx, bool quant);
 void mla_prolog_bind_workspace(MlaPrologArgs& a, void* workspace);
 hipError_t mla_prolog_launch(const MlaPrologArgs& a, hipStream_t stream);
 // The fused MLA + indexer prolog as four launches (needs n_idx a multiple of 64); fused_prolog_bind points the indexer's

@@ -87,36 +87,21 @@ __device__ __forceinline__ void gemm_tr_tile(f32x16& acc, const uint8_t* wtile, 
 // duration is one memory latency plus the transfer), transposed through the group's LDS buffer.  Within a group wave w
 // owns the 32 outputs of block w & 1 over rows [128 (w >> 1), + 128).  The eight partial sums of an output are added
 // through LDS in a fixed order; fp32 partial sums per 1024-row split go to the workspace.
-__global__ __launch_bounds__(1024) void mla_xa_kernel(MlaPrologArgs a)
+// x [t, ldx] (bf16) times the 64 output columns at src (row stride ld), contraction rows [split * 1024, ..) of kdim;
+// the workgroup's fp32 partial sums go to part_out[(split * t + token) * ncols + col0 + ..]
+__device__ __forceinline__ void xa_body(const uint16_t* x, int ldx, int kdim, const uint16_t* src, int ld, float* part_out,
+                                        int ncols, int col0, int split, int tok0, int t, uint8_t* xa_lds)
 {
-    extern __shared__ __align__(16) uint8_t xa_lds[]; // [4 groups][256 k][64 n] bf16, rows of XROW2 bytes
     const int tid = threadIdx.x & 255, grp = threadIdx.x >> 8, lane = tid & 63, wave = tid >> 6;
     const int l32 = lane & 31, hl = lane >> 5;
-    const int split = blockIdx.x, tile = blockIdx.y, tok0 = blockIdx.z * MTOK;
-    const int stages = min(XA_SPLIT, a.h - split * XA_SPLIT) / XA_K; // 256-row stages of this split (4 but for the last)
+    const int stages = min(XA_SPLIT, kdim - split * XA_SPLIT) / XA_K; // 256-row stages of this split (4 but for the last)
     const int sg = min(grp, stages - 1);                              // idle groups re-read the last stage and drop it
     const int64_t kbase = (int64_t)split * XA_SPLIT + sg * XA_K;
-    const int qtiles = a.r / 64;
-    const uint16_t* src;
-    int ld;
-    if (tile < qtiles) {
-        src = a.w_dq + tile * 64;
-        ld = a.r;
-    } else if (tile < qtiles + MKV / 64) {
-        src = a.w_dkv_kr + (tile - qtiles) * 64;
-        ld = MKV;
-    } else if (tile < qtiles + MKV / 64 + PD / 64) { // fused with the indexer prolog: its x @ [w_k | w_proj] rides along
-        src = a.w_k + (tile - qtiles - MKV / 64) * 64;
-        ld = PD;
-    } else {
-        src = a.w_proj + (tile - qtiles - MKV / 64 - PD / 64) * 64;
-        ld = a.n_idx;
-    }
     uint8_t* wl = xa_lds + grp * (XA_K * XROW2);
     const int nb = wave & 1, kh = wave >> 1;
     // the B operand first, then the weights (memory operations complete in order)
     u32x2 bx[16];
-    load_b_rows<8>(bx, a.x + (int64_t)min(tok0 + l32, a.t - 1) * a.h + kbase + 128 * kh, lane);
+    load_b_rows<8>(bx, x + (int64_t)min(tok0 + l32, t - 1) * ldx + kbase + 128 * kh, lane);
     // 256 rows x 128 bytes = 8 pieces of 16 bytes per lane (rows tid/8 + 32 i, piece tid%8)
     const int srow = tid >> 3, spc = tid & 7;
     const uint16_t* sp = src + (kbase + srow) * ld + 8 * spc;
@@ -144,11 +129,77 @@ __global__ __launch_bounds__(1024) void mla_xa_kernel(MlaPrologArgs a)
 #pragma unroll
         for (int e = 0; e < 16; ++e) acc[e] += red[((pp * 2 + nb) * 16 + e) * 64 + lane];
     const int gt = tok0 + l32;
-    if (gt < a.t) {
-        float* out = a.xa_part + ((int64_t)split * a.t + gt) * a.ncols + tile * 64 + 32 * nb + 4 * hl;
+    if (gt < t) {
+        float* out = part_out + ((int64_t)split * t + gt) * ncols + col0 + 32 * nb + 4 * hl;
 #pragma unroll
         for (int e4 = 0; e4 < 4; ++e4)
             *reinterpret_cast<f32x4*>(out + 8 * e4) = f32x4{acc[4 * e4], acc[4 * e4 + 1], acc[4 * e4 + 2], acc[4 * e4 + 3]};
+    }
+}
+
+__global__ __launch_bounds__(1024) void mla_xa_kernel(MlaPrologArgs a)
+{
+    extern __shared__ __align__(16) uint8_t xa_lds[]; // [4 groups][256 k][64 n] bf16, rows of XROW2 bytes
+    const int tile = blockIdx.y;
+    const int qtiles = a.r / 64;
+    const uint16_t* src;
+    int ld;
+    if (tile < qtiles) {
+        src = a.w_dq + tile * 64;
+        ld = a.r;
+    } else if (tile < qtiles + MKV / 64) {
+        src = a.w_dkv_kr + (tile - qtiles) * 64;
+        ld = MKV;
+    } else if (tile < qtiles + MKV / 64 + PD / 64) { // fused with the indexer prolog: its x @ [w_k | w_proj] rides along
+        src = a.w_k + (tile - qtiles - MKV / 64) * 64;
+        ld = PD;
+    } else {
+        src = a.w_proj + (tile - qtiles - MKV / 64 - PD / 64) * 64;
+        ld = a.n_idx;
+    }
+    xa_body(a.x, a.h, a.h, src, ld, a.xa_part, a.ncols, tile * 64, blockIdx.x, blockIdx.z * MTOK, a.t, xa_lds);
+}
+
+// bf16 form of the operator: q_b = q_norm (bf16 [t, r]) @ w_uq_qr (bf16 [r, n * 192]) with the same kernel body;
+// grid (ceil(r / 1024), n * 192 / 64, token tiles of 32); partial sums to qb_part
+__global__ __launch_bounds__(1024) void mla_qb16_kernel(MlaPrologArgs a)
+{
+    extern __shared__ __align__(16) uint8_t xa_lds[];
+    const int nq = a.n * MQH;
+    xa_body(reinterpret_cast<const uint16_t*>(a.q_norm), a.r, a.r, reinterpret_cast<const uint16_t*>(a.w_uq_qr) + blockIdx.y * 64,
+            nq, a.qb_part, nq, blockIdx.y * 64, blockIdx.x, blockIdx.z * MTOK, a.t, xa_lds);
+}
+
+// bf16 form: q_b = bf16(sum of the partial sums); its first 128 dims of a head to qb_nope, the last 64 through the rotary
+// embedding to q_rope.  grid (tokens, n * 192 / 1024 rounded up), 256 lanes: four columns (two pairs) per lane
+__global__ __launch_bounds__(256) void mla_qb16_epilogue_kernel(MlaPrologArgs a)
+{
+#pragma clang fp contract(off)
+    const int tok = blockIdx.x, col = (blockIdx.y * 256 + threadIdx.x) * 4;
+    const int nq = a.n * MQH, splits = (a.r + XA_SPLIT - 1) / XA_SPLIT;
+    if (col >= nq) return;
+    f32x4 acc = *reinterpret_cast<const f32x4*>(a.qb_part + (int64_t)tok * nq + col);
+    for (int sp = 1; sp < splits; ++sp) acc += *reinterpret_cast<const f32x4*>(a.qb_part + ((int64_t)sp * a.t + tok) * nq + col);
+    uint16_t vb[4];
+#pragma unroll
+    for (int e = 0; e < 4; ++e) vb[e] = f32_to_bf16(acc[e]);
+    const int head = col / MQH, d = col % MQH;
+    if (d < MNOPE) {
+        const u32x2 pk = {(uint32_t)vb[0] | ((uint32_t)vb[1] << 16), (uint32_t)vb[2] | ((uint32_t)vb[3] << 16)};
+        *reinterpret_cast<u32x2*>(a.qb_nope + ((int64_t)tok * a.n + head) * MNOPE + d) = pk;
+    } else {
+        const uint16_t* cp = a.cos + (int64_t)tok * MROPE;
+        const uint16_t* snp = a.sin + (int64_t)tok * MROPE;
+        uint16_t* out = a.q_rope + ((int64_t)tok * a.n + head) * MROPE;
+#pragma unroll
+        for (int pr = 0; pr < 2; ++pr) {
+            const int i = (d - MNOPE) / 2 + pr;
+            const float xe = bf16_to_f32(vb[2 * pr]), xo = bf16_to_f32(vb[2 * pr + 1]);
+            const float o1 = xe * bf16_to_f32(cp[i]) + (-xo) * bf16_to_f32(snp[i]);
+            const float o2 = xo * bf16_to_f32(cp[i + 32]) + xe * bf16_to_f32(snp[i + 32]);
+            out[i] = f32_to_bf16(o1);
+            out[i + 32] = f32_to_bf16(o2);
+        }
     }
 }
 
@@ -240,15 +291,22 @@ __device__ __forceinline__ void mla_norm_body(const MlaPrologArgs& a, int tok)
         if (lane == 0) red[4 + wave] = mx;
         __syncthreads();
         mx = fmaxf(fmaxf(red[4], red[5]), fmaxf(red[6], red[7]));
-        const float sq = quant_scale(mx);
-        // four values per lane and store
-        for (int c = 4 * tid; c < r; c += 1024) {
-            uint32_t pk = 0;
+        if (a.quant) {
+            const float sq = quant_scale(mx);
+            // four values per lane and store
+            for (int c = 4 * tid; c < r; c += 1024) {
+                uint32_t pk = 0;
 #pragma unroll
-            for (int e = 0; e < 4; ++e) pk |= ((uint32_t)(int)__builtin_rintf(buf[c + e] * sq) & 0xffu) << (8 * e);
-            *reinterpret_cast<uint32_t*>(a.q_norm + (int64_t)tok * r + c) = pk;
+                for (int e = 0; e < 4; ++e) pk |= ((uint32_t)(int)__builtin_rintf(buf[c + e] * sq) & 0xffu) << (8 * e);
+                *reinterpret_cast<uint32_t*>(a.q_norm + (int64_t)tok * r + c) = pk;
+            }
+            if (tid == 0) a.q_norm_scale[tok] = 1.0f / sq;
+        } else { // bf16 form: q_norm is the normalised row itself
+            uint16_t* qo = reinterpret_cast<uint16_t*>(a.q_norm) + (int64_t)tok * r;
+            for (int c = 4 * tid; c < r; c += 1024)
+                *reinterpret_cast<u32x2*>(qo + c) = u32x2{(uint32_t)f32_to_bf16(buf[c]) | ((uint32_t)f32_to_bf16(buf[c + 1]) << 16),
+                                                          (uint32_t)f32_to_bf16(buf[c + 2]) | ((uint32_t)f32_to_bf16(buf[c + 3]) << 16)};
         }
-        if (tid == 0) a.q_norm_scale[tok] = 1.0f / sq;
     }
     __syncthreads();
     // key: RmsNorm over 512 (lane: elements tid and tid + 256), groups of 128 quantised on their own
@@ -271,13 +329,17 @@ __device__ __forceinline__ void mla_norm_body(const MlaPrologArgs& a, int tok)
         const int pair = wave & 2;
         const float sq0 = quant_scale(fmaxf(red[pair], red[pair + 1]));
         const float sq1 = quant_scale(fmaxf(red[4 + pair], red[4 + pair + 1]));
-        if (row_ok) {
+        if (row_ok && a.quant) {
             a.kv_cache[row * MC + tid] = (int8_t)(int)__builtin_rintf(v0 * sq0);
             a.kv_cache[row * MC + 256 + tid] = (int8_t)(int)__builtin_rintf(v1 * sq1);
             if ((tid & 127) == 0) {
                 a.k_scale_cache[row * 4 + (tid >> 7)] = 1.0f / sq0;
                 a.k_scale_cache[row * 4 + 2 + (tid >> 7)] = 1.0f / sq1;
             }
+        } else if (row_ok) { // bf16 form: the cache row is the normalised key itself, no scales
+            uint16_t* kvo = reinterpret_cast<uint16_t*>(a.kv_cache) + row * MC;
+            kvo[tid] = f32_to_bf16(v0);
+            kvo[256 + tid] = f32_to_bf16(v1);
         }
     }
     // key rotary: pair i = elements (2i, 2i+1) -> positions (i, 32 + i)
@@ -322,7 +384,7 @@ __device__ __forceinline__ void mla_qb_body(const MlaPrologArgs& a, int col0, in
     // tid%8); stages past the end re-read the last one and are dropped
     const int stages = r / QB_K;
     const int srow = tid >> 3, spc = tid & 7;
-    const int8_t* sp = a.w_uq_qr + (int64_t)srow * nq + col0 + 16 * spc;
+    const int8_t* sp = static_cast<const int8_t*>(a.w_uq_qr) + (int64_t)srow * nq + col0 + 16 * spc;
     u32x4 stg[QB_MAXS][4];
 #pragma unroll
     for (int j = 0; j < QB_MAXS; ++j) {
@@ -513,9 +575,11 @@ static uint64_t xa_part_bytes(int64_t t, int64_t h, int64_t ncols)
     return up256((uint64_t)((h + XA_SPLIT - 1) / XA_SPLIT) * t * ncols * sizeof(float));
 }
 
-uint64_t mla_prolog_workspace_bytes(int64_t t, int64_t h, int64_t r, int64_t n, int64_t n_idx)
+uint64_t mla_prolog_workspace_bytes(int64_t t, int64_t h, int64_t r, int64_t n, int64_t n_idx, bool quant)
 {
-    return xa_part_bytes(t, h, r + MKV + (n_idx ? PD + n_idx : 0)) + up256((uint64_t)t * n * MNOPE * 2);
+    // bf16 form: also the partial sums of q_norm @ w_uq_qr
+    return xa_part_bytes(t, h, r + MKV + (n_idx ? PD + n_idx : 0)) + up256((uint64_t)t * n * MNOPE * 2) +
+           (quant ? 0 : xa_part_bytes(t, r, n * MQH));
 }
 
 void mla_prolog_bind_workspace(MlaPrologArgs& a, void* ws)
@@ -524,6 +588,8 @@ void mla_prolog_bind_workspace(MlaPrologArgs& a, void* ws)
     a.xa_part = reinterpret_cast<float*>(p);
     p += xa_part_bytes(a.t, a.h, a.ncols);
     a.qb_nope = reinterpret_cast<uint16_t*>(p);
+    p += up256((uint64_t)a.t * a.n * MNOPE * 2);
+    a.qb_part = reinterpret_cast<float*>(p);
 }
 
 bool fused_prolog_supported(int64_t n_idx) { return n_idx % 64 == 0; }
@@ -550,6 +616,9 @@ static hipError_t set_lds_limits()
     if (e != hipSuccess) return e;
     e = hipFuncSetAttribute(reinterpret_cast<const void*>(mla_qb_kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
                             mla_qb_lds_bytes(MAX_R));
+    if (e != hipSuccess) return e;
+    e = hipFuncSetAttribute(reinterpret_cast<const void*>(mla_qb16_kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
+                            4 * XA_K * XROW2);
     if (e != hipSuccess) return e;
     e = hipFuncSetAttribute(reinterpret_cast<const void*>(fused_qb_kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
                             mla_qb_lds_bytes(MAX_R) > prolog_q_lds_bytes(QMAX_R) ? mla_qb_lds_bytes(MAX_R) : prolog_q_lds_bytes(QMAX_R));
@@ -580,7 +649,12 @@ static hipError_t launch_prologs(const MlaPrologArgs& a, const PrologArgs* p, hi
     if ((e = hipGetLastError()) != hipSuccess) return e;
     {
         ScopedKernelTimer tm(KID_MLA_QB, stream);
-        if (p) {
+        if (!a.quant) {
+            const int nq = a.n * MQH;
+            hipLaunchKernelGGL(mla_qb16_kernel, dim3((a.r + XA_SPLIT - 1) / XA_SPLIT, nq / 64, ttiles), dim3(1024),
+                               4 * XA_K * XROW2, stream, a);
+            hipLaunchKernelGGL(mla_qb16_epilogue_kernel, dim3(a.t, (nq / 4 + 255) / 256), dim3(256), 0, stream, a);
+        } else if (p) {
             const int smem = mla_qb_lds_bytes(a.r) > prolog_q_lds_bytes(a.r) ? mla_qb_lds_bytes(a.r) : prolog_q_lds_bytes(a.r);
             hipLaunchKernelGGL(fused_qb_kernel, dim3(a.n * MQH / 128 + p->n, ttiles), dim3(1024), smem, stream, a, *p);
         } else {

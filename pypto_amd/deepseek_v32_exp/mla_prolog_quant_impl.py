@@ -1,4 +1,4 @@
-"""MLA prolog, int8 form: hidden states -> the attention query (q_nope, q_rope), the quantised normalised query that
+"""MLA prolog: hidden states -> the attention query (q_nope, q_rope), the quantised normalised query that
 the lightning-indexer prolog reads (q_norm, q_norm_scale) and the new rows of the paged int8 MLA cache
 (kv_cache, k_scale_cache, kr_cache) that sparse flash attention reads.
 
@@ -6,8 +6,9 @@ Same entry points, dataclasses, argument order and semantics as the reference mo
 models/deepseek_v32_exp/mla_prolog_quant_impl.py (``MlaTileConfig`` :57-75, ``MlaQuantInputs`` :78-86,
 ``RopeTileShapeConfig`` :89-93, ``mla_prolog_quant_p`` :745-842, ``mla_prolog_quant_d`` :845-951); the device code is
 the gfx950 HIP kernels behind ``pto_mla_prolog_quant_launch``.  The weights are taken in plain row-major layout (the
-reference casts w_dq, w_uq_qr and w_dkv_kr to the Ascend NZ tiling, a device format, before the call).  Only the int8
-form is built: w_uq_qr INT8 with its dequant_scale, kv_cache INT8 with the FP32 k_scale_cache.
+reference casts w_dq, w_uq_qr and w_dkv_kr to the Ascend NZ tiling, a device format, before the call).  Both forms of
+the reference: int8 (w_uq_qr INT8 with its dequant_scale, q_norm_out and kv_cache INT8 with FP32 scales) and bf16 (an
+empty dequant_scale; w_uq_qr, q_norm_out and kv_cache BF16, the scale tensors left alone).
 """
 from dataclasses import dataclass, field
 from typing import List

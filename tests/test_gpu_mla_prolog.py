@@ -28,7 +28,7 @@ def run(case, dev, entry="mla_prolog_quant_d", eps=EPS):
     r = case["w_dq"].shape[1]
     d = {k: v.to(dev) for k, v in case.items()}
     kv, kr, ks = d["kv_cache"].clone(), d["kr_cache"].clone(), d["k_scale_cache"].clone()
-    q_norm = torch.zeros((t, r), dtype=torch.int8, device=dev)
+    q_norm = torch.zeros((t, r), dtype=d["kv_cache"].dtype, device=dev)   # int8 form: int8; bf16 form: bf16
     q_norm_scale = torch.zeros((t, 1), dtype=torch.float32, device=dev)
     q_nope = torch.zeros((t, n, 512), dtype=torch.bfloat16, device=dev)
     q_rope = torch.zeros((t, n, 64), dtype=torch.bfloat16, device=dev)
@@ -113,6 +113,67 @@ def test_reference_prefill_case_t128(cuda):
     check(case, run(case, cuda, entry="mla_prolog_quant_p"))
 
 
+def check_bf16_form(case, got, eps=EPS):
+    """bf16 form (the reference's tolerances, :686-694: q_norm, kv, kr rtol 2^-7 / atol 1e-4; q_nope, q_rope rtol 2^-7 /
+    atol 5e-3): everything within those everywhere, and bit-equal in at least 98 % of the places - the difference is
+    the summation order of x @ w, which now and then moves a bf16 rounding."""
+    gold = op.mla_prolog(case, eps, eps)
+    rows = case["cache_index"]
+
+    def floats(a, b, name, rtol, atol, min_equal=0.98):
+        a, b = a.float(), b.float()
+        assert torch.isfinite(a).all(), name
+        ratio = (a - b).abs() / (atol + rtol * b.abs())
+        assert ratio.max() <= 1, f"{name}: worst {float(ratio.max())} x the tolerance"
+        assert (a == b).float().mean() >= min_equal, f"{name}: only {(a == b).float().mean():.3f} bit-equal"
+
+    floats(got["q_norm"], gold["q_norm"], "q_norm", 0.0078125, 1e-4)
+    floats(got["q_nope"], gold["q_nope"], "q_nope", 0.0078125, 0.005, 0.90)
+    floats(got["q_rope"], gold["q_rope"], "q_rope", 0.0078125, 0.005, 0.90)
+    tail_nope, tail_rope = op.query_tail(case, got["q_norm"], None)
+    floats(got["q_nope"], tail_nope, "q_nope from the product's q_norm", 0.0078125, 0.005, 0.99)
+    floats(got["q_rope"], tail_rope, "q_rope from the product's q_norm", 0.0078125, 0.005, 0.99)
+    floats(got["kv_cache"].view(-1, 512)[rows], gold["kv_cache"].view(-1, 512)[rows], "kv_cache", 0.0078125, 1e-4)
+    floats(got["kr_cache"].view(-1, 64)[rows], gold["kr_cache"].view(-1, 64)[rows], "kr_cache", 0.0078125, 1e-4, 0.95)
+    keep = torch.ones(case["kv_cache"].shape[0] * case["kv_cache"].shape[1], dtype=torch.bool)
+    keep[rows] = False
+    assert torch.equal(got["kv_cache"].view(-1, 512)[keep], case["kv_cache"].view(-1, 512)[keep])
+    assert torch.equal(got["kr_cache"].view(-1, 64)[keep], case["kr_cache"].view(-1, 64)[keep])
+    assert torch.equal(got["k_scale_cache"], case["k_scale_cache"])          # the scale tensors are not touched
+    assert torch.equal(got["q_norm_scale"], torch.zeros_like(got["q_norm_scale"]))
+
+
+def test_bf16_form_reference_case_b4_s2(cuda):
+    # the reference's test_b4_s64k2_pa_nd_bf16_d: no quantisation anywhere (empty dequant_scale, bf16 w_uq_qr and cache)
+    case = op.make_case(4, 2, 1024, seed=18, quant_b=False)
+    check_bf16_form(case, run(case, cuda))
+
+
+def test_bf16_form_small_sizes_and_ragged_token_tiles(cuda):
+    for b, s1, seed in ((1, 1, 19), (37, 1, 20)):
+        case = op.make_case(b, s1, 300, seed=seed, h=512, q_lora_rank=256, n=4, quant_b=False)
+        check_bf16_form(case, run(case, cuda))
+    case = op.make_case(3, 2, 300, seed=21, h=1280, q_lora_rank=1280, n=6, quant_b=False)   # ragged last splits
+    check_bf16_form(case, run(case, cuda, entry="mla_prolog_quant_p"))
+
+
+def test_bf16_form_feeds_sparse_flash_attention(cuda):
+    """The bf16 cache rows the bf16 form writes are what sparse flash attention reads in its bf16-cache flavour."""
+    from _cases import run_sfa
+    from test_gpu_sfa import full_check
+    b, s1, s2 = 2, 2, 300
+    case = op.make_case(b, s1, s2, seed=22, quant_b=False)
+    got = run(case, cuda)
+    tk = torch.zeros((b * s1, 2048), dtype=torch.int32)
+    tk[:, :s2] = torch.arange(s2, dtype=torch.int32)
+    ca = {"b": b, "s1": s1, "nq": 128, "topk": 2048, "block_size": 128, "softmax_scale": 192 ** -0.5,
+          "act_seq": [s2] * b, "q": torch.cat([got["q_nope"], got["q_rope"]], dim=-1).reshape(b, s1, 128, 576),
+          "kn": got["kv_cache"].view(-1, 512), "kr": got["kr_cache"].view(-1, 64),
+          "kn_scales": torch.ones((got["kv_cache"].view(-1, 512).shape[0], 4), dtype=torch.float32),
+          "topk_indices": tk, "block_table": case["block_table"]}
+    full_check(run_sfa(ca, cuda), ca, "bf16 prolog -> attention")
+
+
 def test_prolog_feeds_sparse_flash_attention(cuda):
     """Stage chaining: the query the prolog writes and the cache rows it adds are, as they are, what sparse flash
     attention reads (int8 kv rows with four fp32 scales, bf16 rope rows, q_nope | q_rope)."""
@@ -140,7 +201,9 @@ def test_errors(cuda):
     case = op.make_case(2, 1, 256, seed=1, h=512, q_lora_rank=256, n=4)
     with pytest.raises(FeError, match="int64|INT64"):
         run(dict(case, cache_index=case["cache_index"].int()), cuda)
-    with pytest.raises(FeError, match="int8 form"):
+    with pytest.raises(FeError, match="multiple of 256"):
+        run(op.make_case(2, 1, 256, seed=1, h=512, q_lora_rank=384, n=4, quant_b=False), cuda)
+    with pytest.raises(FeError, match="int8 form"):     # bf16 weights with a non-empty dequant_scale: neither form
         run(dict(case, w_uq_qr=case["w_uq_qr"].to(torch.bfloat16)), cuda)
     with pytest.raises(FeError, match="heads"):
         run(dict(case, w_uk=case["w_uk"][:3].contiguous(), w_uq_qr=case["w_uq_qr"][:, :576].contiguous(),

@@ -114,3 +114,24 @@ def test_epsilon_form_is_within_the_reference_tolerance_of_the_golden():
     assert (a["q_norm"].int() - b["q_norm"].int()).abs().max() <= 1
     assert torch.allclose(a["q_norm_scale"], b["q_norm_scale"], rtol=5e-3, atol=2.5e-5)
     assert (a["kv_cache"].int() - b["kv_cache"].int()).abs().max() <= 1
+
+
+def test_bf16_form_has_no_quantisation_anywhere():
+    c = op.make_case(3, 2, 300, seed=7, quant_b=False, **SMALL)
+    assert c["w_uq_qr"].dtype == torch.bfloat16 and c["w_qb_scale"].numel() == 0 and c["kv_cache"].dtype == torch.bfloat16
+    out = op.mla_prolog(c)
+    im = op.intermediates(c)
+    rows = c["cache_index"]
+    t = rows.numel()
+    assert out["q_norm_scale"] is None and torch.equal(out["q_norm"], im["q_rms"])           # q_norm is the RmsNorm output
+    qb = (im["q_rms"].double() @ c["w_uq_qr"].double()).reshape(t, 4, 192)                    # fp64 product, bf16 slack
+    assert ((im["q_b"].double() - qb).abs() <= 2.0 ** -8 * qb.abs() + 1e-6).all()
+    qn = torch.einsum("tnd,ndc->tnc", im["q_b"][..., :128].double(), c["w_uk"].double())
+    assert ((out["q_nope"].double() - qn).abs() <= 2.0 ** -8 * qn.abs() + 1e-6).all()
+    assert torch.equal(out["q_rope"], op.rope_interleaved(im["q_b"][..., 128:], c["cos"], c["sin"]))
+    kv = out["kv_cache"].view(-1, 512)
+    assert torch.equal(kv[rows], im["kv_rms"])                                                # the cache row is the normalised key
+    assert torch.equal(out["k_scale_cache"], c["k_scale_cache"])                              # scales untouched
+    keep = torch.ones(kv.shape[0], dtype=torch.bool)
+    keep[rows] = False
+    assert torch.equal(kv[keep], c["kv_cache"].view(-1, 512)[keep])
