@@ -139,6 +139,34 @@ def test_index_head_counts_without_the_side_by_side_kernels(cuda):
         assert torch.equal(v, sep[k]), f"{k}: fused and separate calls differ"
 
 
+def test_decode_layer_front_end_chain(cuda):
+    """One decode layer's attention front end as three chained calls on the GPU, each stage checked against the oracle
+    on the previous stage's actual outputs: fused prolog -> (indexer query, weights, updated index cache) -> lightning
+    indexer -> top-k rows -> sparse flash attention over the updated int8 MLA cache with the prolog's query."""
+    from _cases import run_indexer, run_sfa
+    from test_gpu_indexer import check_topk
+    from test_gpu_sfa import full_check
+    b, s1, s2 = 2, 2, 3000
+    mla_case, idx_case = op.make_fused_case(b, s1, s2, seed=25)
+    got = run_fused(mla_case, idx_case, cuda)
+    n_pages = got["k_cache"].shape[0]
+    ci = {"query": got["q_int8"], "q_scale": got["q_scale"].reshape(b * s1, 64), "weights": got["weights"],
+          "key_cache": got["k_cache"], "k_scale": got["idx_k_scale_cache"].reshape(n_pages, 128, 1),
+          "act_seq": [s2] * b, "block_table": mla_case["block_table"], "b": b, "s1": s1, "selected_count": 2048,
+          "block_size": 128}
+    topk = run_indexer(ci, cuda)
+    check_topk(ci, topk)
+    ca = {"b": b, "s1": s1, "nq": 128, "topk": 2048, "block_size": 128, "softmax_scale": 192 ** -0.5, "act_seq": [s2] * b,
+          "q": torch.cat([got["q_nope"], got["q_rope"]], dim=-1).reshape(b, s1, 128, 576),
+          "kn": got["kv_cache"].view(-1, 512), "kr": got["kr_cache"].view(-1, 64),
+          "kn_scales": got["k_scale_cache"].view(-1, 4), "topk_indices": topk.reshape(b * s1, 2048),
+          "block_table": mla_case["block_table"]}
+    # the newest token of a query's causal range is its own, just-written cache row: it must be reachable
+    new_rows = mla_case["cache_index"].reshape(b, s1)
+    assert (ca["kn_scales"][new_rows.reshape(-1)] > 0).all()
+    full_check(run_sfa(ca, cuda), ca, "prolog -> indexer -> attention")
+
+
 def test_no_tokens_is_a_no_op(cuda):
     """An empty batch (t = 0) is accepted by all three prolog entries and touches nothing."""
     mla_case, idx_case = op.make_fused_case(2, 1, 256, seed=24, n_idx=64, h=512, q_lora_rank=256, n=4)
