@@ -48,7 +48,7 @@ def parse():
     ap.add_argument("--cpu-seqs", type=int, default=8, help="sequences of the workload timed on the CPU oracle")
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--packed", action="store_true", help="use the packed 656-byte-row attention entry point")
-    ap.add_argument("--workload", choices=["v32", "gqa", "select_experts", "indexer_prolog", "mla_prolog", "mla_indexer_prolog"], default="v32",
+    ap.add_argument("--workload", choices=["v32", "gqa", "select_experts", "indexer_prolog", "mla_prolog", "mla_indexer_prolog", "decode_layer"], default="v32",
                     help="v32 (default): the headline DeepSeek-V3.2 indexer + sparse attention decode step; gqa: GLM-4.5 "
                          "paged GQA decode (batch 64, 96/8 heads, contexts U[4096, 32768]); select_experts: GLM-4.5 "
                          "router (8192 tokens x 160 experts)")
@@ -383,6 +383,67 @@ def bench_mla_indexer_prolog(args, torch, lib, dev):
     }))
 
 
+def bench_decode_layer(args, torch, lib, dev):
+    """The attention front end of one DeepSeek-V3.2 decode layer as three chained calls on shared buffers: the fused MLA +
+    indexer prolog writes the query tensors and the new cache rows (the last position of every sequence), the lightning
+    indexer selects 2048 rows per token, sparse flash attention reads them.  Shapes of the default workload (batch 32, one
+    token each, every context 65536) and of the prolog workloads."""
+    from pypto_amd.deepseek_v32_exp import mla_indexer_prolog_quant_impl as pimpl
+    from pypto_amd.deepseek_v32_exp.lightning_indexer_quant_impl import LightningIndexerConfigs, lightning_indexer_decode
+    from pypto_amd.deepseek_v32_exp.sparse_flash_attention_quant_impl import (SaTileShapeConfig,
+                                                                              sparse_flash_attention_quant_d)
+    b, ctx, s1 = args.batch, args.ctx, 1
+    t, n, ni, h, r, c, d, bs = b, 128, 64, 7168, 1536, 512, 128, 128
+    w = make_workload(torch, dev, b, ctx, s1, 1)
+    cs = w["sets"][0]
+    g = torch.Generator(device=dev).manual_seed(1)
+    bf = torch.bfloat16
+
+    def uni(lo, hi, *shape):
+        return torch.rand(shape, generator=g, device=dev) * (hi - lo) + lo
+
+    wq = uni(-0.1, 0.1, r, n * 192)
+    wq_scale = (wq.abs().amax(0, keepdim=True) / 127)
+    pos = ctx - 1
+    rows = (w["table"][:, pos // bs].to(torch.int64) * bs + pos % bs).contiguous()
+    n_pages = w["table"].numel()
+    kv, kr, ks = cs["kn"].view(n_pages, bs, 1, c), cs["kr"].view(n_pages, bs, 1, 64), cs["ks"].view(n_pages, bs, 1, 4)
+    ik, iks = cs["idx_k"], cs["idx_ks"].view(n_pages, bs, 1, 1)
+    q_nope, q_rope = w["q_nope"].view(t, n, c), w["q_rope"].view(t, n, 64)
+    idx_q, idx_qs, idx_w = w["idx_q"], w["idx_qs"].view(t, ni, 1), w["idx_w"]
+    ang = torch.rand((t, 64), generator=g, device=dev) * 6.2831853
+    prolog = [uni(-1, 1, t, h).to(bf), uni(-0.1, 0.1, h, r).to(bf), torch.round(wq / wq_scale).to(torch.int8),
+              wq_scale.reshape(-1, 1).contiguous(), uni(-0.1, 0.1, n, 128, c).to(bf), uni(-0.1, 0.1, h, c + 64).to(bf),
+              uni(-1, 1, r).to(bf), uni(-1, 1, c).to(bf), torch.cos(ang).to(bf), torch.sin(ang).to(bf), rows, kv, kr, ks,
+              torch.randint(-128, 128, (r, ni * d), generator=g, device=dev, dtype=torch.int8), uni(0.001, 0.01, ni * d, 1),
+              uni(-0.1, 0.1, h, d).to(bf), uni(-0.1, 0.1, h, ni).to(bf), torch.ones(d, dtype=bf, device=dev),
+              torch.zeros(d, dtype=bf, device=dev), uni(-1, 1, d, d).to(bf) / 11.3, uni(-1, 1, d, d).to(bf) / 11.3, ik, iks,
+              q_nope, q_rope, kv, kr, ks, idx_q, idx_qs, ik, iks, idx_w]
+    scal = (1e-5, 1e-5, "PA_BSND", pimpl.MlaTileConfig(), pimpl.IndexerPrologQuantAttr(), pimpl.IndexerPrologQuantConfigs(),
+            pimpl.RopeTileShapeConfig([32, 64], [32, 32, 128], [16, 128, 128, 128]))
+    cfg, tile, unroll = LightningIndexerConfigs(), SaTileShapeConfig(), [128, 64, 32, 16, 8, 4, 1]
+    scale = 192 ** -0.5
+
+    def step(i):
+        pimpl.mla_indexer_prolog_quant_d(*prolog, *scal)
+        lightning_indexer_decode(idx_q, w["idx_qs"], ik, cs["idx_ks"], idx_w, w["act"], w["table"], w["topk_res"], unroll,
+                                 cfg, 2048)
+        sparse_flash_attention_quant_d(w["q_nope"], w["q_rope"], cs["kn"], cs["kr"], cs["ks"], w["topk_res"].view(t, 2048),
+                                       w["table"], w["act"], w["out"], 128, 1, scale, 2048, 128, w["pages_per_seq"], tile)
+
+    ms, kernels = timed(torch, lib, step, args)
+    assert torch.isfinite(w["out"].float()).all()
+    print(json.dumps({
+        "metric": "decode tokens/sec, DeepSeek-V3.2 attention front end (fused prolog + indexer + SFA) b=32 ctx=64K",
+        "value": round(t / (ms * 1e-3), 1), "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(ms, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "int8+bf16", "data": "synthetic", "launch": "hip graph replay" if args.graph else "eager",
+        "config": {"workload": f"fused MLA + indexer prolog -> lightning indexer top-2048 -> sparse flash attention, batch {b}, "
+                               f"1 query token per sequence, context {ctx}, model sizes"},
+        "roofline": None, "kernels": [{"kernel": k, "us": round(u, 2)} for k, u in kernels.items()], "cpu_baseline": None,
+    }))
+
+
 def main():
     args = parse()
     if args.gpus != 1:
@@ -411,6 +472,8 @@ def main():
         return bench_mla_prolog(args, torch, lib, dev)
     if args.workload == "mla_indexer_prolog":
         return bench_mla_indexer_prolog(args, torch, lib, dev)
+    if args.workload == "decode_layer":
+        return bench_decode_layer(args, torch, lib, dev)
     b, ctx, s1 = args.batch, args.ctx, args.s1
     scale = 192 ** -0.5
     nbuf = 3
