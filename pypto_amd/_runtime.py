@@ -10,6 +10,7 @@ used for device memory and streams only; all compute is in the HIP library.
 import ctypes
 import functools
 import os
+import struct
 import threading
 
 import torch
@@ -110,53 +111,95 @@ def load_library():
     return _lib
 
 
+_DESC = struct.Struct("Pii8q")          # PtoTensorDesc: addr, dataType, rank, shape[8]
+assert _DESC.size == ctypes.sizeof(TensorDesc)
+_PAD = tuple((0,) * (8 - r) for r in range(9))
+
+
 def describe(tensors):
-    descs = (TensorDesc * len(tensors))()
-    for d, t in zip(descs, tensors):
+    """PtoTensorDesc array of the tensors (no checks beyond dtype and rank)."""
+    n = len(tensors)
+    buf = bytearray(_DESC.size * n)
+    off = 0
+    for t in tensors:
         code = _DTYPE_CODE.get(t.dtype)
         if code is None:
             raise ValueError(f"unsupported tensor dtype {t.dtype}")
-        if t.dim() > 8:
+        shape = t.shape
+        r = len(shape)
+        if r > 8:
             raise ValueError("tensors of more than 8 dimensions are not supported")
-        d.addr = t.data_ptr() if t.numel() else None
-        d.dataType = code
-        d.rank = t.dim()
-        for i, s in enumerate(t.shape):
-            d.shape[i] = s
-    return descs
+        _DESC.pack_into(buf, off, t.data_ptr() if t.numel() else 0, code, r, *shape, *_PAD[r])
+        off += _DESC.size
+    return (TensorDesc * n).from_buffer(buf)
 
 
-def _validate_tensors(tensors):
+def _check_and_describe(tensors):
+    """The checks of the reference's binding (every operand a dense torch.Tensor, all on one HIP device) and the
+    descriptor array, in one pass over the tensors: this is the host's cost of a call, and it shows for the operators
+    whose kernels take a few tens of microseconds."""
+    n = len(tensors)
+    buf = bytearray(_DESC.size * n)
+    off = 0
+    dev = None
     for idx, t in enumerate(tensors):
-        if not isinstance(t, torch.Tensor):
-            raise FeError(RuntimeError(f"Input {idx + 1} (index {idx}) must be a torch.Tensor, got {t.__class__}"))
-        if type(t).__name__ == "DTensor":
-            raise FeError(RuntimeError(f"Input {idx + 1} (index {idx}) must not be a DTensor, got {t.__class__}"))
+        if type(t) is not torch.Tensor:
+            if not isinstance(t, torch.Tensor):
+                raise FeError(RuntimeError(f"Input {idx + 1} (index {idx}) must be a torch.Tensor, got {t.__class__}"))
+            if type(t).__name__ == "DTensor":
+                raise FeError(RuntimeError(f"Input {idx + 1} (index {idx}) must not be a DTensor, got {t.__class__}"))
         if not t.is_contiguous():
             raise FeError(RuntimeError("not all tensors are contiguous"))
-    dev = tensors[0].device
-    for t in tensors:
-        if t.device != dev:
-            raise FeError(RuntimeError(f"all tensors must be on the same device, got {dev} and {t.device}"))
+        d = t.device
+        if dev is None:
+            dev = d
+        elif d != dev:
+            raise FeError(RuntimeError(f"all tensors must be on the same device, got {dev} and {d}"))
+        code = _DTYPE_CODE.get(t.dtype)
+        if code is None:
+            raise ValueError(f"unsupported tensor dtype {t.dtype}")
+        shape = t.shape
+        r = len(shape)
+        if r > 8:
+            raise ValueError("tensors of more than 8 dimensions are not supported")
+        _DESC.pack_into(buf, off, t.data_ptr() if t.numel() else 0, code, r, *shape, *_PAD[r])
+        off += _DESC.size
     if dev.type != "cuda":
         raise FeError(RuntimeError(f"tensors must be on a HIP device (torch device type 'cuda'), got {dev}"))
-    return dev
+    return dev, (TensorDesc * n).from_buffer(buf)
+
+
+_fns = {}
+
+
+def _entry_points(op):
+    fns = _fns.get(op)
+    if fns is None:
+        lib = load_library()
+        fns = _fns[op] = (getattr(lib, f"pto_{op}_workspace"), getattr(lib, f"pto_{op}_launch"))
+    return fns
+
+
+def _launch_on_current_device(dev, ws_fn, launch_fn, descs, n, params):
+    p = ctypes.byref(params)
+    ws_bytes = ws_fn(descs, n, p)
+    ws = torch.empty(ws_bytes, dtype=torch.uint8, device=dev) if ws_bytes else None
+    return launch_fn(descs, n, p, ws.data_ptr() if ws is not None else None, ws_bytes,
+                     torch.cuda.current_stream(dev).cuda_stream)
 
 
 def launch(op, tensors, params):
     """Validate, size the workspace, launch on the current stream of the tensors' device."""
-    lib = load_library()
-    dev = _validate_tensors(tensors)
-    descs = describe(tensors)
+    ws_fn, launch_fn = _entry_points(op)
+    dev, descs = _check_and_describe(tensors)
     n = len(tensors)
-    with torch.cuda.device(dev):
-        ws_bytes = getattr(lib, f"pto_{op}_workspace")(descs, n, ctypes.byref(params))
-        ws = torch.empty(ws_bytes, dtype=torch.uint8, device=dev) if ws_bytes else None
-        stream = torch.cuda.current_stream(dev).cuda_stream
-        rc = getattr(lib, f"pto_{op}_launch")(descs, n, ctypes.byref(params), ws.data_ptr() if ws is not None else None,
-                                              ws_bytes, stream)
+    if dev.index is None or dev.index == torch.cuda.current_device():
+        rc = _launch_on_current_device(dev, ws_fn, launch_fn, descs, n, params)
+    else:
+        with torch.cuda.device(dev):
+            rc = _launch_on_current_device(dev, ws_fn, launch_fn, descs, n, params)
     if rc != 0:
-        msg = lib.pto_last_error().decode()
+        msg = _lib.pto_last_error().decode()
         raise _STATUS_EXC.get(rc, RuntimeError)(msg)
 
 

@@ -50,33 +50,32 @@ constexpr int QB_QP = MTOK * (MAX_R / 16) / 1024; // 16-byte pieces of the q_nor
 
 
 // 32 outputs x 32 tokens += W[KSTEPS steps of 16 rows, outputs]^T . X[tokens, k]: A by transposing reads of the [k][n]
-// tile in LDS, rows of ROWB bytes (lane jj of a 16-lane group points at row 4 hl + jj / 4 (+ 8) of the step, columns
-// 16 mh + 4 (jj & 3)), which hand lane half hl the contraction rows {4 hl .. 4 hl + 3} and {8 + 4 hl .. + 3}; B takes the
-// same rows of X as two 8-byte pieces.  Register e of the result: output 8 (e / 4) + 4 hl + e % 4, token lane % 32.
+// tile in LDS, rows of ROWB bytes.  Lane jj of a 16-lane group points at row 8 hl + jj / 4 (+ 4 for the second read) of
+// the step, columns 16 mh + 4 (jj & 3); a read hands lane i the column 16 mh + i over the four rows its group's lanes
+// i / 4, i / 4 + 4, ... point at, so lane half hl ends up with the contraction rows 8 hl .. 8 hl + 7 of the step - and B
+// takes the same rows of X with ONE 16-byte load per step (x[token][16 ks + 8 hl ..]: 32 bytes contiguous per token row
+// and instruction; narrower pieces cost the texture addresser twice the cycles, and it is what bounds these loads:
+// every lane pair reads a different row).  Register e of the result: output 8 (e / 4) + 4 hl + e % 4, token lane % 32.
 // The B operand is loaded by its own call so that a caller can put these loads ahead of a prefetch in program order:
 // memory operations complete in order, and a wait for loads issued after a prefetch would wait for the prefetch too.
 template <int KSTEPS>
-__device__ __forceinline__ void load_b_rows(u32x2 (&b)[2 * KSTEPS], const uint16_t* xrow, int lane)
+__device__ __forceinline__ void load_b_rows(u32x4 (&b)[KSTEPS], const uint16_t* xrow, int lane)
 {
-    const uint16_t* xp = xrow + (lane >> 5) * 4;
+    const uint16_t* xp = xrow + (lane >> 5) * 8;
 #pragma unroll
-    for (int ks = 0; ks < KSTEPS; ++ks) {
-        b[2 * ks] = *reinterpret_cast<const u32x2*>(xp + ks * 16);
-        b[2 * ks + 1] = *reinterpret_cast<const u32x2*>(xp + ks * 16 + 8);
-    }
+    for (int ks = 0; ks < KSTEPS; ++ks) b[ks] = *reinterpret_cast<const u32x4*>(xp + ks * 16);
 }
 template <int KSTEPS, int ROWB>
-__device__ __forceinline__ void gemm_tr_tile(f32x16& acc, const uint8_t* wtile, int ncol0, const u32x2 (&b)[2 * KSTEPS], int lane)
+__device__ __forceinline__ void gemm_tr_tile(f32x16& acc, const uint8_t* wtile, int ncol0, const u32x4 (&b)[KSTEPS], int lane)
 {
     const int jj = lane & 15, mh = (lane >> 4) & 1, hl = lane >> 5;
-    const uint8_t* hp = wtile + (4 * hl + (jj >> 2)) * ROWB + (ncol0 + 16 * mh + 4 * (jj & 3)) * 2;
+    const uint8_t* hp = wtile + (8 * hl + (jj >> 2)) * ROWB + (ncol0 + 16 * mh + 4 * (jj & 3)) * 2;
 #pragma unroll
     for (int ks = 0; ks < KSTEPS; ++ks) {
-        const bf16x8 bv = __builtin_bit_cast(bf16x8, u32x4{b[2 * ks][0], b[2 * ks][1], b[2 * ks + 1][0], b[2 * ks + 1][1]});
         const s16x4 lo = lds_read_tr(hp + ks * 16 * ROWB);
-        const s16x4 hi = lds_read_tr(hp + (ks * 16 + 8) * ROWB);
+        const s16x4 hi = lds_read_tr(hp + (ks * 16 + 4) * ROWB);
         const bf16x8 av = __builtin_bit_cast(bf16x8, __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
-        acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(av, bv, acc, 0, 0, 0);
+        acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(av, __builtin_bit_cast(bf16x8, b[ks]), acc, 0, 0, 0);
     }
 }
 
@@ -100,7 +99,7 @@ __device__ __forceinline__ void xa_body(const uint16_t* x, int ldx, int kdim, co
     uint8_t* wl = xa_lds + grp * (XA_K * XROW2);
     const int nb = wave & 1, kh = wave >> 1;
     // the B operand first, then the weights (memory operations complete in order)
-    u32x2 bx[16];
+    u32x4 bx[8];
     load_b_rows<8>(bx, x + (int64_t)min(tok0 + l32, t - 1) * ldx + kbase + 128 * kh, lane);
     // 256 rows x 128 bytes = 8 pieces of 16 bytes per lane (rows tid/8 + 32 i, piece tid%8)
     const int srow = tid >> 3, spc = tid & 7;
@@ -537,7 +536,7 @@ __global__ __launch_bounds__(256) void mla_wuk_kernel(MlaPrologArgs a)
     const int head = blockIdx.x, ct = blockIdx.y, tok0 = blockIdx.z * MTOK;
     const uint16_t* src = a.w_uk + (int64_t)head * MNOPE * MC + ct * 128;
     const int gt = tok0 + l32;
-    u32x2 bx[2 * (MNOPE / 16)];
+    u32x4 bx[MNOPE / 16];
     load_b_rows<MNOPE / 16>(bx, a.qb_nope + ((int64_t)min(gt, a.t - 1) * a.n + head) * MNOPE, lane);
 #pragma unroll
     for (int i = tid; i < MNOPE * 16; i += 256) {

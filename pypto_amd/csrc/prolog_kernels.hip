@@ -62,24 +62,23 @@ __device__ __forceinline__ void prolog_xw_body(const PrologArgs& a, int split, i
     __syncthreads();
     const int nblocks = nw / 32; // 32-wide output blocks; wave w takes blocks w, w + 4
     const int jj = lane & 15, mh = (lane >> 4) & 1;
-    // B operand rows as the transposing reads order them: {4 hl .. + 3} and {8 + 4 hl .. + 3} of every 16-row step
-    const uint16_t* xp = a.x + (int64_t)min(tok0 + l32, a.t - 1) * a.h + kbase + hl * 4;
+    // B operand: the transposing reads below hand lane half hl the contraction rows 8 hl .. 8 hl + 7 of every 16-row step,
+    // so B is one 16-byte load per step (32 bytes contiguous per token row and instruction)
+    const uint16_t* xp = a.x + (int64_t)min(tok0 + l32, a.t - 1) * a.h + kbase + hl * 8;
     f32x16 acc[2];
 #pragma unroll
     for (int j = 0; j < 2; ++j)
 #pragma unroll
         for (int e = 0; e < 16; ++e) acc[j][e] = 0.f;
     for (int ks = 0; ks < XW_K / 16; ++ks) {
-        const u32x2 b0 = *reinterpret_cast<const u32x2*>(xp + ks * 16);
-        const u32x2 b1 = *reinterpret_cast<const u32x2*>(xp + ks * 16 + 8);
-        const bf16x8 bv = __builtin_bit_cast(bf16x8, u32x4{b0[0], b0[1], b1[0], b1[1]});
+        const bf16x8 bv = __builtin_bit_cast(bf16x8, *reinterpret_cast<const u32x4*>(xp + ks * 16));
 #pragma unroll
         for (int j = 0; j < 2; ++j) {
             const int nb = wave + 4 * j;
             if (nb < nblocks) {
-                const uint8_t* hp = wl + (ks * 16 + 4 * hl + (jj >> 2)) * rowb + (32 * nb + 16 * mh + 4 * (jj & 3)) * 2;
+                const uint8_t* hp = wl + (ks * 16 + 8 * hl + (jj >> 2)) * rowb + (32 * nb + 16 * mh + 4 * (jj & 3)) * 2;
                 const s16x4 lo = lds_read_tr(hp);
-                const s16x4 hi = lds_read_tr(hp + 8 * rowb);
+                const s16x4 hi = lds_read_tr(hp + 4 * rowb);
                 const bf16x8 av = __builtin_bit_cast(bf16x8, __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
                 acc[j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(av, bv, acc[j], 0, 0, 0);
             }
