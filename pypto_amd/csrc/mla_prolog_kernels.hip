@@ -358,8 +358,11 @@ __device__ __forceinline__ void mla_norm_body(const MlaPrologArgs& a, int tok)
 // transposed.  The token tile of q_norm sits in LDS (loaded ahead of the weights: memory operations complete in
 // order).  Within a group wave w owns outputs [32 w, 32 w + 32) of the tile.  The groups' int32 sums are added through LDS
 // at the end (exact, so the result does not depend on the split).
-__host__ __device__ constexpr int mla_qb_lds_bytes(int r) { return QB_GROUPS * QB_K * MQROW + MTOK * (r + 16); }
-// qb_lds: [QB_GROUPS][QB_K * MQROW] weights | [32][r + 16] q_norm
+__host__ __device__ constexpr int mla_qb_lds_bytes(int r)
+{
+    return QB_GROUPS * QB_K * MQROW + MTOK * (r + 16) + 2 * MTOK * MROPE * 2;
+}
+// qb_lds: [QB_GROUPS][QB_K * MQROW] weights | [32][r + 16] q_norm | [2][32][64] cos, sin
 __device__ __forceinline__ void mla_qb_body(const MlaPrologArgs& a, int col0, int tok0, uint8_t* qb_lds)
 {
 #pragma clang fp contract(off)
@@ -369,6 +372,7 @@ __device__ __forceinline__ void mla_qb_body(const MlaPrologArgs& a, int col0, in
     const int64_t nq = (int64_t)a.n * MQH;
     uint8_t* wl = qb_lds + grp * (QB_K * MQROW);
     uint8_t* ql = qb_lds + QB_GROUPS * (QB_K * MQROW);
+    uint16_t* csl = reinterpret_cast<uint16_t*>(ql + MTOK * qrowb); // [2][32][64]: the token tile's cos and sin rows
 
     // q_norm tile: 32 rows of r bytes, 16-byte pieces over the 1024 lanes (at most QB_QP per lane)
     const int qpieces = MTOK * (r / 16);
@@ -379,6 +383,18 @@ __device__ __forceinline__ void mla_qb_body(const MlaPrologArgs& a, int col0, in
         const int row = pc / (r / 16), c = pc % (r / 16);
         qst[i] = *reinterpret_cast<const u32x4*>(a.q_norm + (int64_t)min(tok0 + row, a.t - 1) * r + 16 * c);
     }
+    // the token tile's cos / sin rows and scales for the epilogue: loaded now, so that the epilogue waits for nothing
+    u32x4 cst = {0u, 0u, 0u, 0u};
+    if (threadIdx.x < 512) {
+        const int which = threadIdx.x >> 8, row = (threadIdx.x & 255) >> 3, c = threadIdx.x & 7;
+        cst = *reinterpret_cast<const u32x4*>((which ? a.sin : a.cos) + (int64_t)min(tok0 + row, a.t - 1) * MROPE + 8 * c);
+    }
+    float qs_pre[2];
+    f32x4 ws_pre[2];
+#pragma unroll
+    for (int tb = 0; tb < 2; ++tb) qs_pre[tb] = a.q_norm_scale[min(tok0 + 16 * tb + l16, a.t - 1)];
+#pragma unroll
+    for (int nb = 0; nb < 2; ++nb) ws_pre[nb] = *reinterpret_cast<const f32x4*>(a.w_qb_scale + col0 + 32 * wave + 16 * nb + 4 * g);
     // weights: every stage of this group, 128 rows x 128 bytes = 4 pieces of 16 bytes per lane (rows tid/8 + 32 i, piece
     // tid%8); stages past the end re-read the last one and are dropped
     const int stages = r / QB_K;
@@ -396,6 +412,7 @@ __device__ __forceinline__ void mla_qb_body(const MlaPrologArgs& a, int col0, in
         const int pc = (int)threadIdx.x + 1024 * i;
         if (pc < qpieces) *reinterpret_cast<u32x4*>(ql + (pc / (r / 16)) * qrowb + 16 * (pc % (r / 16))) = qst[i];
     }
+    if (threadIdx.x < 512) reinterpret_cast<u32x4*>(csl)[threadIdx.x] = cst;
     i32x4 acc[2][2];
 #pragma unroll
     for (int nb = 0; nb < 2; ++nb)
@@ -460,12 +477,12 @@ __device__ __forceinline__ void mla_qb_body(const MlaPrologArgs& a, int col0, in
     for (int tb = 0; tb < 2; ++tb) {
         const int gt = tok0 + 16 * tb + l16;
         if (gt >= a.t) continue;
-        const float qs = a.q_norm_scale[gt];
+        const float qs = qs_pre[tb];
 #pragma unroll
         for (int nb = 0; nb < 2; ++nb) {
             const int col = col0 + 32 * wave + 16 * nb + 4 * g;
             const int head = col / MQH, d = col % MQH;
-            const f32x4 ws = *reinterpret_cast<const f32x4*>(a.w_qb_scale + col);
+            const f32x4 ws = ws_pre[nb];
             uint16_t vb[4];
 #pragma unroll
             for (int e = 0; e < 4; ++e) vb[e] = f32_to_bf16(((float)acc[nb][tb][e] * qs) * ws[e]);
@@ -473,8 +490,8 @@ __device__ __forceinline__ void mla_qb_body(const MlaPrologArgs& a, int col0, in
                 const u32x2 pk = {(uint32_t)vb[0] | ((uint32_t)vb[1] << 16), (uint32_t)vb[2] | ((uint32_t)vb[3] << 16)};
                 *reinterpret_cast<u32x2*>(a.qb_nope + ((int64_t)gt * a.n + head) * MNOPE + d) = pk;
             } else {
-                const uint16_t* cp = a.cos + (int64_t)gt * MROPE;
-                const uint16_t* snp = a.sin + (int64_t)gt * MROPE;
+                const uint16_t* cp = csl + (16 * tb + l16) * MROPE;
+                const uint16_t* snp = csl + (MTOK + 16 * tb + l16) * MROPE;
                 uint16_t* out = a.q_rope + ((int64_t)gt * a.n + head) * MROPE;
 #pragma unroll
                 for (int pr = 0; pr < 2; ++pr) {
