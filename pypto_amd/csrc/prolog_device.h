@@ -20,23 +20,27 @@ constexpr int QMAX_R = 2048; // largest q_lora_rank
 constexpr int QMAXS = QMAX_R / QK / QGROUPS;   // stages per group at the largest q_lora_rank
 constexpr int QQP = PTOK * (QMAX_R / 16) / 1024; // 16-byte pieces of the q_norm tile per lane at the largest q_lora_rank
 
-__host__ __device__ constexpr int prolog_q_lds_bytes(int r) { return QGROUPS * QK * QROW + PTOK * (r + 16); }
+constexpr int QAUX = 2 * PTOK * PROPE * 2 + PD * 4 + PTOK * 4; // cos and sin rows of the token tile, w_qb_scale, q_norm_scale
+
+__host__ __device__ constexpr int prolog_q_lds_bytes(int r) { return QGROUPS * QK * QROW + PTOK * (r + 16) + QAUX; }
 static_assert(QGROUPS * QK * QROW >= PD * PD * 2 + PTOK * XROW + 4 * PTOK * 4, "the epilogue fits in the stage buffers");
 
 // Rotary embedding of the first 64 dims of the 32 x 128 bf16 tile in LDS, fp32 arithmetic with every product and sum
-// rounded (the golden's x * cos + rotate_half(x) * sin), back to bf16.  256 lanes: 4 (token, pair) items each.
-__device__ __forceinline__ void rope_tile(uint8_t* xt, const uint16_t* cosp, const uint16_t* sinp, int tok0, int t, int tid)
+// rounded (the golden's x * cos + rotate_half(x) * sin), back to bf16.  256 lanes: 4 (token, pair) items each.  csl is the
+// tile's [2][32][64] cos and sin rows in LDS.
+__device__ __forceinline__ void rope_tile(uint8_t* xt, const uint16_t* csl, int tid)
 {
 #pragma clang fp contract(off)
 #pragma unroll
     for (int it = 0; it < 4; ++it) {
         const int item = tid + 256 * it;
         const int tok = item >> 5, i = item & 31;
-        const int gt = min(tok0 + tok, t - 1);
         uint16_t* row = reinterpret_cast<uint16_t*>(xt + tok * XROW);
+        const uint16_t* cosp = csl + tok * PROPE;
+        const uint16_t* sinp = csl + (PTOK + tok) * PROPE;
         const float x1 = bf16_to_f32(row[i]), x2 = bf16_to_f32(row[i + 32]);
-        const float c1 = bf16_to_f32(cosp[(int64_t)gt * PROPE + i]), c2 = bf16_to_f32(cosp[(int64_t)gt * PROPE + i + 32]);
-        const float s1 = bf16_to_f32(sinp[(int64_t)gt * PROPE + i]), s2 = bf16_to_f32(sinp[(int64_t)gt * PROPE + i + 32]);
+        const float c1 = bf16_to_f32(cosp[i]), c2 = bf16_to_f32(cosp[i + 32]);
+        const float s1 = bf16_to_f32(sinp[i]), s2 = bf16_to_f32(sinp[i + 32]);
         const float o1 = x1 * c1 + (-x2) * s1;
         const float o2 = x2 * c2 + x1 * s2;
         row[i] = f32_to_bf16(o1);
@@ -49,7 +53,8 @@ __device__ __forceinline__ void rope_tile(uint8_t* xt, const uint16_t* cosp, con
 // (prolog_q_lds_bytes).
 __device__ __forceinline__ void prolog_q_body(const PrologArgs& a, int head, int tok0, uint8_t* plds)
 {
-    // LDS: [4 groups][QK x QROW] weight stages | [32][r + 16] q_norm tile.  Once the GEMM is done the first region is
+    // LDS: [4 groups][QK x QROW] weight stages | [32][r + 16] q_norm tile | cos, sin rows and scales for the epilogue.
+    // Once the GEMM is done the first region is
     // reused for hadamard_q [128][128] bf16, the head's bf16 tile [32][XROW] and the per-wave maxima.
     uint8_t* had = plds;
     uint8_t* xt = plds + PD * PD * 2;
@@ -61,6 +66,10 @@ __device__ __forceinline__ void prolog_q_body(const PrologArgs& a, int head, int
     const int64_t nd = (int64_t)a.n * PD;
     uint8_t* wl = plds + grp * (QK * QROW);
     uint8_t* ql = plds + QGROUPS * (QK * QROW);
+    uint8_t* aux = ql + PTOK * qrowb; // [2][32][64] bf16 cos, sin | [128] w_qb_scale | [32] q_norm_scale
+    const uint16_t* csl = reinterpret_cast<const uint16_t*>(aux);
+    const float* wsl = reinterpret_cast<const float*>(aux + 2 * PTOK * PROPE * 2);
+    const float* qsl = wsl + PD;
 
     // loads in the order they are needed: hadamard_q (parked in registers until the GEMM is over), the q_norm tile,
     // then every weight stage of this group - all in flight together
@@ -75,6 +84,14 @@ __device__ __forceinline__ void prolog_q_body(const PrologArgs& a, int head, int
         const int row = pc / (r / 16), c = pc % (r / 16);
         qst[i] = *reinterpret_cast<const u32x4*>(a.q_norm + (int64_t)min(tok0 + row, a.t - 1) * r + 16 * c);
     }
+    // what the epilogue reads (rotary rows, scales): fetched now, so that it waits for nothing later
+    // (every lane loads - a load under a condition would be waited for on the spot; lanes past 544 fetch piece 0 again)
+    const int ai = threadIdx.x < 544 ? (int)threadIdx.x : 0;
+    const uint8_t* ap = ai < 512 ? reinterpret_cast<const uint8_t*>((ai >> 8 ? a.sin : a.cos) +
+                                                                     (int64_t)min(tok0 + ((ai & 255) >> 3), a.t - 1) * PROPE + 8 * (ai & 7))
+                                 : reinterpret_cast<const uint8_t*>(a.w_qb_scale + (int64_t)head * PD + 4 * (ai - 512));
+    const u32x4 ast = *reinterpret_cast<const u32x4*>(ap);
+    const float qst1 = a.q_norm_scale[min(tok0 + (int)(threadIdx.x & 31), a.t - 1)];
     const int stages = r / QK;
     const int srow = tid >> 3, spc = tid & 7;
     const int8_t* sp = a.w_qb + (int64_t)srow * nd + head * PD + 16 * spc;
@@ -90,6 +107,8 @@ __device__ __forceinline__ void prolog_q_body(const PrologArgs& a, int head, int
         const int pc = (int)threadIdx.x + 1024 * i;
         if (pc < qpieces) *reinterpret_cast<u32x4*>(ql + (pc / (r / 16)) * qrowb + 16 * (pc % (r / 16))) = qst[i];
     }
+    if (threadIdx.x < 544) reinterpret_cast<u32x4*>(aux)[threadIdx.x] = ast;
+    if (threadIdx.x < 32) reinterpret_cast<float*>(aux)[4 * 544 + threadIdx.x] = qst1;
     // C^T[dim, token] = W^T[dim, :] . q_norm[token, :]: wave w owns dims [32 w, 32 w + 32) x 32 tokens
     i32x4 acc[2][2];
 #pragma unroll
@@ -163,11 +182,11 @@ __device__ __forceinline__ void prolog_q_body(const PrologArgs& a, int head, int
 #pragma unroll
         for (int tb = 0; tb < 2; ++tb) {
             const int tok = 16 * tb + l16;
-            const float qs = a.q_norm_scale[min(tok0 + tok, a.t - 1)];
+            const float qs = qsl[tok];
 #pragma unroll
             for (int db = 0; db < 2; ++db) {
                 const int dim = 32 * wave + 16 * db + 4 * g;
-                const f32x4 ws = *reinterpret_cast<const f32x4*>(a.w_qb_scale + (int64_t)head * PD + dim);
+                const f32x4 ws = *reinterpret_cast<const f32x4*>(wsl + dim);
                 uint16_t* dst = reinterpret_cast<uint16_t*>(xt + tok * XROW) + dim;
 #pragma unroll
                 for (int e = 0; e < 4; ++e) dst[e] = f32_to_bf16(((float)acc[db][tb][e] * qs) * ws[e]);
@@ -175,7 +194,7 @@ __device__ __forceinline__ void prolog_q_body(const PrologArgs& a, int head, int
         }
     }
     __syncthreads();
-    rope_tile(xt, a.cos, a.sin, tok0, a.t, tid);
+    rope_tile(xt, csl, tid);
     __syncthreads();
 
     // Y^T[n, token] = H^T[n, k] . X^T[k, token]: wave w owns n in [32 w, 32 w + 32).  A (H^T) by transposing reads of
