@@ -157,14 +157,19 @@ __global__ __launch_bounds__(256) void indexer_score_kernel(IndexerArgs a)
     }
 }
 
-// relu(a) * 2^-11 and relu(b) * 2^-11, each rounded once to fp16, packed (a in the low half).  The product is exact in
-// fp32 (|a| < 2^21) and relu commutes with the rounding, so it is taken on the packed pair.  (Written in plain C on
-// purpose: the compiler's hazard recognizer does not look inside inline assembly, and a hand-placed VALU write into a
-// register that an MFMA is still writing goes wrong.)
+// relu(a) * 2^-11 and relu(b) * 2^-11, each rounded once to fp16, packed (a in the low half).  The int32 sums arrive
+// biased: the MFMA accumulators start at SCORE_BIAS = the bit pattern of the float 1.5 * 2^23, and since |a| < 2^21 the
+// accumulator's bits, read as a float, are exactly 12582912 + a - the integer-to-float conversion costs nothing.  One
+// fused multiply-add takes the bias off and scales (exact in fp32: a * 2^-11 has at most 21 significant bits); relu
+// commutes with the rounding to fp16, so it is taken on the packed pair.  (Written in plain C on purpose: the
+// compiler's hazard recognizer does not look inside inline assembly, and a hand-placed VALU write into a register that
+// an MFMA is still writing goes wrong.)
+constexpr int SCORE_BIAS = 0x4B400000;
 typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
 __device__ __forceinline__ uint32_t relu_scale_pack(int a, int b)
 {
-    f16x2 v = {(_Float16)((float)a * 0x1p-11f), (_Float16)((float)b * 0x1p-11f)};
+    f16x2 v = {(_Float16)__builtin_fmaf(__int_as_float(a), 0x1p-11f, -6144.0f),
+               (_Float16)__builtin_fmaf(__int_as_float(b), 0x1p-11f, -6144.0f)};
     const f16x2 z = {(_Float16)0.f, (_Float16)0.f};
     return __builtin_bit_cast(uint32_t, __builtin_elementwise_max(v, z));
 }
@@ -182,24 +187,29 @@ __global__ __launch_bounds__(256, S1 == 1 ? 3 : 2) void indexer_score_paged_kern
     constexpr int NBUF = 2; // half-pass buffers: NBUF-1 halves ahead (deeper prefetch measured no faster)
     constexpr int NHALF = 2 * PPASSES;
     __shared__ uint32_t hist[S1][NBINS];
-    __shared__ __align__(16) _Float16 s_ws[S1][64];
+    __shared__ __align__(16) float s_sc[S1][CHUNK * PPASSES]; // the workgroup's scores, written out in one burst at the end
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int l16 = lane & 15, g = lane >> 4;
     const int bi = blockIdx.y;
     const int sgrp = blockIdx.z;
-    const int L = a.act_seq[bi];
-    if (blockIdx.x * (CHUNK * PPASSES) >= L) return;
     const int row0 = bi * a.s1 + sgrp * S1;
     const int bs = a.block_size;
     const int wtok = blockIdx.x * (CHUNK * PPASSES) + wave * 128; // first key of this wave's pass 0
 
-    // lane p: first cache row of pass p (-1: unmapped page); a pass past the end re-reads the sequence's first page
-    // and is discarded
+    // The sequence length and the page-table entries are fetched together (one round trip before the first key load,
+    // not two): lane p takes the entry of pass p and the sequence's first entry, and picks once the length is known.
+    // lane p then holds the first cache row of pass p (-1: unmapped page); a pass past the end re-reads the sequence's
+    // first page and is discarded.
+    const int mytok = wtok + (lane < PPASSES ? lane : 0) * CHUNK;
+    const int32_t* bt = a.block_table + (int64_t)bi * a.bt_stride;
+    const int pg_mine = bt[min(mytok / bs, a.bt_stride - 1)];
+    const int pg_first = bt[0];
+    const int L = a.act_seq[bi];
+    if (blockIdx.x * (CHUNK * PPASSES) >= L) return;
     int64_t myrow;
     {
-        const int mytok = wtok + (lane < PPASSES ? lane : 0) * CHUNK;
         const int tc = mytok < L ? mytok : 0;
-        const int pg = a.block_table[(int64_t)bi * a.bt_stride + tc / bs];
+        const int pg = mytok < L ? pg_mine : pg_first;
         myrow = (pg >= 0 && pg < a.n_blocks) ? (int64_t)pg * bs + tc % bs : -1;
     }
     auto pass_row = [&](int pass) {
@@ -221,13 +231,11 @@ __global__ __launch_bounds__(256, S1 == 1 ? 3 : 2) void indexer_score_paged_kern
         }
         ksc[buf][0] = a.k_scale[rb + 64 * (hh & 1) + lane];
     };
-    for (int i = tid; i < S1 * NBINS; i += 256) (&hist[0][0])[i] = 0;
-    if (tid < 64 * S1) {
-        const int64_t h = (int64_t)row0 * a.nh + tid;
-        const _Float16 qs = __builtin_bit_cast(_Float16, a.q_scale[h]);
-        const _Float16 w = __builtin_bit_cast(_Float16, a.weights[h]);
-        (&s_ws[0][0])[tid] = (_Float16)(qs * w); // one fp16 rounding
-    }
+    // The key loads go out first; the query and its scales follow them (memory operations complete in order, and the
+    // first MFMA needs all of them).  Every memory operation from here on is unconditional, so that the number in
+    // flight is the same on every path into the loop and the waits can count them.
+#pragma unroll
+    for (int u = 0; u < NBUF - 1; ++u) load_half(u, u);
     // int8 A fragments: head hb*16 + l16, bytes 64*ks + 16*g .. +15
     i32x4 qf[S1][4][2];
 #pragma unroll
@@ -238,23 +246,22 @@ __global__ __launch_bounds__(256, S1 == 1 ? 3 : 2) void indexer_score_paged_kern
             qf[s][hb][0] = *reinterpret_cast<const i32x4*>(qp);
             qf[s][hb][1] = *reinterpret_cast<const i32x4*>(qp + 64);
         }
-    __syncthreads();
     // fp16 A fragments of the head sum, the same in every row: k-slot (g, e) of MFMA mm is head
-    // 32*mm + 16*(e/4) + 4*g + e%4 - the head whose int32 result this lane group holds in that slot
+    // 32*mm + 16*(e/4) + 4*g + e%4 - the head whose int32 result this lane group holds in that slot; the value is
+    // q_scale * weights in one fp16 rounding
     f16x8 wa[S1][2];
 #pragma unroll
     for (int s = 0; s < S1; ++s)
 #pragma unroll
         for (int mm = 0; mm < 2; ++mm) {
             typedef _Float16 f16x4 __attribute__((ext_vector_type(4)));
-            const f16x4 lo = *reinterpret_cast<const f16x4*>(&s_ws[s][32 * mm + 4 * g]);
-            const f16x4 hi = *reinterpret_cast<const f16x4*>(&s_ws[s][32 * mm + 16 + 4 * g]);
-            wa[s][mm] = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+            const int64_t h = (int64_t)(row0 + s) * a.nh + 32 * mm + 4 * g;
+            const f16x4 qlo = *reinterpret_cast<const f16x4*>(a.q_scale + h), qhi = *reinterpret_cast<const f16x4*>(a.q_scale + h + 16);
+            const f16x4 wlo = *reinterpret_cast<const f16x4*>(a.weights + h), whi = *reinterpret_cast<const f16x4*>(a.weights + h + 16);
+            wa[s][mm] = __builtin_shufflevector(qlo * wlo, qhi * whi, 0, 1, 2, 3, 4, 5, 6, 7);
         }
-    // The prefetch starts only here, and every memory operation of the loop below is unconditional, so that the
-    // number of memory operations in flight is the same on every path into the loop and the waits can count them
-#pragma unroll
-    for (int u = 0; u < NBUF - 1; ++u) load_half(u, u);
+    for (int i = tid; i < S1 * NBINS; i += 256) (&hist[0][0])[i] = 0;
+    __syncthreads();
 
     auto compute_half = [&](int hh, int buf) {
         float res[S1];
@@ -267,7 +274,7 @@ __global__ __launch_bounds__(256, S1 == 1 ? 3 : 2) void indexer_score_paged_kern
                 u32x4 y[2];
 #pragma unroll
                 for (int hb = 0; hb < 4; ++hb) {
-                    i32x4 acc = {0, 0, 0, 0};
+                    i32x4 acc = {SCORE_BIAS, SCORE_BIAS, SCORE_BIAS, SCORE_BIAS};
                     acc = __builtin_amdgcn_mfma_i32_16x16x64_i8(qf[s][hb][0], kf[buf][jj][0], acc, 0, 0, 0);
                     acc = __builtin_amdgcn_mfma_i32_16x16x64_i8(qf[s][hb][1], kf[buf][jj][1], acc, 0, 0, 0);
                     y[hb >> 1][2 * (hb & 1)] = relu_scale_pack(acc[0], acc[1]);
@@ -279,13 +286,12 @@ __global__ __launch_bounds__(256, S1 == 1 ? 3 : 2) void indexer_score_paged_kern
                 res[s] = jj == g ? sum[0] : res[s];
             }
         }
-        // score rows are padded to whole workgroup spans, so the store needs no bounds check
         const int tok = wtok + (hh >> 1) * CHUNK + 64 * (hh & 1) + lane;
         const float ks = pass_row(hh >> 1) >= 0 ? f16_bits_to_f32(ksc[buf][0]) : 0.f;
 #pragma unroll
         for (int s = 0; s < S1; ++s) {
             const float sc = res[s] * ks;
-            a.scores[(int64_t)(row0 + s) * a.score_stride + tok] = sc;
+            s_sc[s][tok - (int)blockIdx.x * (CHUNK * PPASSES)] = sc;
             const int eff = L - (a.s1 - 1 - (sgrp * S1 + s));
             if (tok < eff) atomicAdd(&hist[s][score_key(sc) >> 21], 1u);
         }
@@ -306,6 +312,15 @@ __global__ __launch_bounds__(256, S1 == 1 ? 3 : 2) void indexer_score_paged_kern
         }
     }
     __syncthreads();
+    // one contiguous 8 KB write per query token (256-byte stores from inside the loop, between the key loads, cost
+    // 2 us more); score rows are padded to whole workgroup spans, so no bounds check
+#pragma unroll
+    for (int s = 0; s < S1; ++s) {
+        float* dst = a.scores + (int64_t)(row0 + s) * a.score_stride + (int64_t)blockIdx.x * (CHUNK * PPASSES);
+#pragma unroll
+        for (int i = 0; i < CHUNK * PPASSES / 1024; ++i)
+            *reinterpret_cast<f32x4*>(dst + 4 * (tid + 256 * i)) = *reinterpret_cast<const f32x4*>(&s_sc[s][4 * (tid + 256 * i)]);
+    }
     for (int i = tid; i < S1 * NBINS; i += 256) {
         const uint32_t c = (&hist[0][0])[i];
         if (c) atomicAdd(a.hist + (int64_t)(row0 + i / NBINS) * NBINS + (i % NBINS), c);
