@@ -87,9 +87,13 @@ template <bool QUANT>
 __device__ __forceinline__ void load_raw(RawTile<QUANT>& r, const SfaArgs& a, const int* rows, const uint32_t* tmask,
                                          int tile, int wave, int lane, int tid)
 {
+    // the 8 rows are the same for every lane of the wavefront: two 16-byte LDS reads, then scalar address arithmetic
+    // (the loads take a scalar base and the lane's column offset)
+    const u32x4 ra = *reinterpret_cast<const u32x4*>(rows + tile * T + 8 * wave);
+    const u32x4 rb = *reinterpret_cast<const u32x4*>(rows + tile * T + 8 * wave + 4);
 #pragma unroll
     for (int e = 0; e < 8; ++e) {
-        const uint32_t row = (uint32_t)rows[tile * T + 8 * wave + e];
+        const uint32_t row = __builtin_amdgcn_readfirstlane(e < 4 ? ra[e & 3] : rb[e & 3]);
         if constexpr (QUANT)
             r.nope[e] = *reinterpret_cast<const u32x2*>(a.kn + (uint64_t)row * a.kn_stride + lane * 8);
         else
@@ -147,6 +151,54 @@ __device__ __forceinline__ void dequant_store(const RawTile<QUANT>& r, uint8_t* 
     }
 }
 
+// Resolves a workgroup's share of a token's top-k list: logical indices -> physical cache rows (absent entries: row 0
+// and a cleared bit in the tile's validity word) and their 4 dequant scales (0 when absent), all in LDS.  NT lanes.
+template <int NT, bool QUANT>
+__device__ __forceinline__ void resolve_split(const SfaArgs& a, int bi, int tq, int tok0, int cur, int ntiles_real,
+                                              int ntiles, uint32_t* tmask, int* rows, float* scales, int* bt_lds, int tid,
+                                              int lane)
+{
+    // this sequence's page table -> LDS (saves one dependent global load per selected token)
+    const bool bt_cached = a.bt_cached != 0;
+    if (bt_cached)
+        for (int i = tid; i < a.bt_stride; i += NT) bt_lds[i] = a.block_table[(int64_t)bi * a.bt_stride + i];
+    // logical top-k entries of this split
+    const int64_t max_logical = (int64_t)a.bt_stride * a.block_size;
+    int my_idx[MAX_SPLIT_TOKENS / NT];
+#pragma unroll
+    for (int j = 0; j < MAX_SPLIT_TOKENS / NT; ++j) {
+        const int i = tid + NT * j, g = tok0 + i;
+        my_idx[j] = -1;
+        if (i < ntiles_real * T && g < cur) my_idx[j] = a.topk_idx[(int64_t)tq * a.topk_stride + g];
+    }
+    __syncthreads();
+#pragma unroll
+    for (int j = 0; j < MAX_SPLIT_TOKENS / NT; ++j) {
+        const int i = tid + NT * j;
+        if (i >= ntiles * T) break; // wave-uniform: tiles are 32 wide, waves 64
+        const int idx = my_idx[j];
+        int row = -1;
+        if (idx >= 0 && idx < max_logical) {
+            const int page = bt_cached ? bt_lds[idx / a.block_size]
+                                       : a.block_table[(int64_t)bi * a.bt_stride + idx / a.block_size];
+            const int64_t r = (int64_t)page * a.block_size + idx % a.block_size;
+            if (page >= 0 && r < a.n_rows) row = (int)r;
+        }
+        rows[i] = max(row, 0);
+        const uint64_t present = __ballot(row >= 0);
+        if (lane == 0) {
+            tmask[i >> 5] = (uint32_t)present;
+            tmask[(i >> 5) + 1] = (uint32_t)(present >> 32);
+        }
+        if constexpr (QUANT) {
+            f32x4 sc = {0.f, 0.f, 0.f, 0.f};
+            if (row >= 0) sc = *reinterpret_cast<const f32x4*>(a.ks + (uint64_t)row * a.ks_stride);
+            *reinterpret_cast<f32x4*>(scales + i * 4) = sc;
+        }
+    }
+    __syncthreads(); // rows[] / scales[] / tmask[] ready
+}
+
 template <bool QUANT>
 __global__ __attribute__((amdgpu_flat_work_group_size(512, 512), amdgpu_waves_per_eu(2, 2))) void sfa_decode_kernel(
     SfaArgs a)
@@ -171,47 +223,7 @@ __global__ __attribute__((amdgpu_flat_work_group_size(512, 512), amdgpu_waves_pe
     const int ntiles = (ntiles_real + 1) & ~1;
     const int tok0 = tile0 * T;
 
-    // this sequence's page table -> LDS (saves one dependent global load per selected token)
-    const bool bt_cached = a.bt_cached != 0;
-    if (bt_cached)
-        for (int i = tid; i < a.bt_stride; i += 512) bt_lds[i] = a.block_table[(int64_t)bi * a.bt_stride + i];
-    // logical top-k entries of this split
-    const int64_t max_logical = (int64_t)a.bt_stride * a.block_size;
-    int my_idx[MAX_SPLIT_TOKENS / 512];
-#pragma unroll
-    for (int j = 0; j < MAX_SPLIT_TOKENS / 512; ++j) {
-        const int i = tid + 512 * j, g = tok0 + i;
-        my_idx[j] = -1;
-        if (i < ntiles_real * T && g < cur) my_idx[j] = a.topk_idx[(int64_t)tq * a.topk_stride + g];
-    }
-    __syncthreads();
-    // -> physical cache rows (absent entries: row 0 and a cleared bit in the tile's validity word) and their
-    // 4 dequant scales (0 when absent)
-#pragma unroll
-    for (int j = 0; j < MAX_SPLIT_TOKENS / 512; ++j) {
-        const int i = tid + 512 * j;
-        if (i >= ntiles * T) break; // wave-uniform: tiles are 32 wide, waves 64
-        const int idx = my_idx[j];
-        int row = -1;
-        if (idx >= 0 && idx < max_logical) {
-            const int page = bt_cached ? bt_lds[idx / a.block_size]
-                                       : a.block_table[(int64_t)bi * a.bt_stride + idx / a.block_size];
-            const int64_t r = (int64_t)page * a.block_size + idx % a.block_size;
-            if (page >= 0 && r < a.n_rows) row = (int)r;
-        }
-        rows[i] = max(row, 0);
-        const uint64_t present = __ballot(row >= 0);
-        if (lane == 0) {
-            tmask[i >> 5] = (uint32_t)present;
-            tmask[(i >> 5) + 1] = (uint32_t)(present >> 32);
-        }
-        if constexpr (QUANT) {
-            f32x4 sc = {0.f, 0.f, 0.f, 0.f};
-            if (row >= 0) sc = *reinterpret_cast<const f32x4*>(a.ks + (uint64_t)row * a.ks_stride);
-            *reinterpret_cast<f32x4*>(scales + i * 4) = sc;
-        }
-    }
-    __syncthreads(); // rows[] / scales[] / tmask[] ready
+    resolve_split<512, QUANT>(a, bi, tq, tok0, cur, ntiles_real, ntiles, tmask, rows, scales, bt_lds, tid, lane);
 
     // Both roles run the same barrier sequence: one before the first tile, then two per tile
     // (partial S exchanged; tile consumed and next tile stored).
