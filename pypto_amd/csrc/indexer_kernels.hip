@@ -333,6 +333,12 @@ __global__ void indexer_zero_kernel(uint32_t* p, int n)
     if (i < n) p[i] = 0u;
 }
 
+__global__ void indexer_fill_kernel(int32_t* p, int n, int32_t v)
+{
+    const int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) p[i] = v;
+}
+
 // block-wide inclusive suffix sum (lane t gets sum of v[t .. nthreads-1]); tmp holds one word per wavefront
 template <int NWAVES>
 __device__ __forceinline__ uint32_t block_suffix_sum(uint32_t v, uint32_t* tmp)
@@ -670,6 +676,11 @@ hipError_t indexer_launch(const IndexerArgs& a, hipStream_t stream)
     const int t = a.b * a.s1;
     if (t == 0) return hipSuccess;
     const int max_ctx = a.bt_stride * a.block_size;
+    if (max_ctx == 0) { // a page table without columns: no key can be addressed, every slot is -1
+        const int n = t * a.k;
+        hipLaunchKernelGGL(indexer_fill_kernel, dim3((n + 255) / 256), dim3(256), 0, stream, a.topk_res, n, -1);
+        return hipGetLastError();
+    }
     const int chunks = (max_ctx + CHUNK * PASSES - 1) / (CHUNK * PASSES);
     const int pchunks = (max_ctx + CHUNK * PPASSES - 1) / (CHUNK * PPASSES);
     const int nzero = t * (NBINS + 4);
