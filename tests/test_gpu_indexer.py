@@ -27,8 +27,8 @@ def check_topk(case, got, exact=None, strict_ties=False):
     gold = oi.select(indexer_scores(case), case["act_seq"], s1, k)
     swaps = 0
     for r in range(got.shape[0]):
-        n = oi.eff_seq_of(case["act_seq"][r // s1], s1, r % s1)
-        kk = max(min(n, k), 0)
+        n = max(oi.eff_seq_of(case["act_seq"][r // s1], s1, r % s1), 0)
+        kk = min(n, k)
         row = got[r, 0]
         assert (row[kk:] == -1).all(), f"row {r}: padding"
         sel = row[:kk].long()
@@ -49,7 +49,9 @@ def check_topk(case, got, exact=None, strict_ties=False):
             a, e = int(row[j]), int(gold[r, 0, j])
             assert a >= 0 and e >= 0 and abs(float(sc[a]) - float(sc[e])) <= tol, f"row {r} slot {j}: {a} vs {e}"
             swaps += 1
-    topk_idx_compare(got, gold, "topk_res", 5e-4, k)  # the reference's own comparator
+    # the reference's own comparator: it allows int(k * 5e-4) ids per row to differ, one at the reference's k = 2048
+    # (a near-tie at the selection boundary); smaller selections get the same allowance of one
+    topk_idx_compare(got, gold, "topk_res", max(5e-4, 1.5 / k), k)
     return swaps
 
 
@@ -129,6 +131,7 @@ def test_empty_sequences_and_empty_page_table(cuda):
         assert case["block_table"].shape[1] == 0 and case["key_cache"].shape[0] == 0
         got = run_indexer(case, cuda)
         assert (got == -1).all()
+        check_topk(case, got)
     # an empty sequence beside a live one
     case = oi.make_case(3, 2, [0, 700, 1], seed=16)
     check_topk(case, run_indexer(case, cuda))
