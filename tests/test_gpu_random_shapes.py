@@ -1,0 +1,65 @@
+"""GPU parity over randomly drawn shapes: lightning indexer and sparse flash attention against the CPU oracle.
+
+The named tests pin the reference's cases and the edge cases one by one; this one walks a seeded sample of the space
+between them (batch, query tokens per sequence, lengths around the tile / page / selection boundaries, page sizes,
+selection sizes, head counts, entry points, cache forms), with the same checkers and the same bars.
+"""
+import random
+
+import pytest
+import torch
+
+from oracle import indexer as oi
+from oracle import sfa as osfa
+
+from _cases import run_indexer, run_sfa, sfa_golden
+from test_gpu_indexer import check_topk
+from test_gpu_sfa import check
+
+pytestmark = pytest.mark.gpu
+
+EDGES = [0, 1, 2, 15, 127, 128, 129, 2047, 2048, 2049, 4095, 4096, 4097]
+
+
+def draw_len(rng, hi):
+    c = rng.random()
+    if c < 0.15:
+        return rng.choice(EDGES)
+    if c < 0.5:
+        return rng.randint(1, 5000)
+    return rng.randint(1, hi)
+
+
+@pytest.mark.parametrize("seed", [101, 202, 303])
+def test_indexer_random_shapes(cuda, seed):
+    rng = random.Random(seed)
+    for i in range(25):
+        b, s1 = rng.randint(1, 4), rng.choice([1, 1, 2, 3, 4])
+        act = [draw_len(rng, 40000) for _ in range(b)]
+        bs = rng.choice([128, 128, 128, 256, 64, 48, 16])
+        k = rng.choice([2048, 2048, 512, 64, 1024])
+        dist = rng.choice(["bench", "driver"])
+        case = oi.make_case(b, s1, act, seed=1000 * seed + i, block_size=bs, selected_count=k, dist=dist)
+        try:
+            check_topk(case, run_indexer(case, cuda))
+        except AssertionError as e:
+            raise AssertionError(f"b={b} s1={s1} act={act} block_size={bs} k={k} dist={dist}: {e}") from e
+
+
+@pytest.mark.parametrize("seed", [404, 505])
+def test_attention_random_shapes(cuda, seed):
+    rng = random.Random(seed)
+    for i in range(20):
+        b, s1 = rng.randint(1, 3), rng.choice([1, 1, 2, 3])
+        nq = rng.choice([128, 64, 16, 32, 8, 96])
+        topk = rng.choice([2048, 2048, 256, 512, 96])
+        act = [draw_len(rng, 20000) for _ in range(b)]
+        bs = rng.choice([128, 128, 64, 256])
+        quant = rng.random() < 0.8
+        packed = quant and rng.random() < 0.4
+        entry = rng.choice(["d", "p", "d_950"])
+        dist = rng.choice(["uniform", "bench"]) if quant else "uniform"
+        name = (f"b={b} s1={s1} nq={nq} topk={topk} act={act} block_size={bs} quant={quant} packed={packed} "
+                f"entry={entry} dist={dist}")
+        case = osfa.make_case(b, nq, s1, act, topk=topk, block_size=bs, seed=1000 * seed + i, quant=quant, dist=dist)
+        check(run_sfa(case, cuda, entry=entry, packed=packed), sfa_golden(case), name)
