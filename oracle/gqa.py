@@ -93,7 +93,7 @@ def rope_neox(x, positions, theta=1e6, rotary_dim=64):
 
 
 def make_case(b, s1, nq, nkv, act_seqs, block_size=128, seed=0, dist="normal", d=128, extra_blocks=2):
-    """dist "normal": BASELINE's GQA configuration (q, k, v ~ N(0,1), rotary embedding theta 1e6 on the first 64 dims of
+    """dist "normal": the benchmark's GQA configuration (q, k, v ~ N(0,1), rotary embedding theta 1e6 on the first 64 dims of
     q and k); dist "uniform": the reference driver's inputs (U[-1,1), glm_attention.py:1313-1315)."""
     g = torch.Generator().manual_seed(seed)
     max_blocks = max((max(act_seqs) + block_size - 1) // block_size, 1)

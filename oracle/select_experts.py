@@ -38,7 +38,7 @@ def biased_scores(router_logits, e_score_correction_bias):
 
 
 def make_case(t, ne=160, seed=0, logits_dtype=torch.float32, bias_dtype=torch.bfloat16, dist="normal"):
-    """dist "normal": BASELINE's expert-selector configuration (logits N(0,1), bias N(0,0.1));
+    """dist "normal": the benchmark's expert-selector configuration (logits N(0,1), bias N(0,0.1));
     dist "uniform": the reference test's inputs (both U[0,1), glm_select_experts.py:262-263)."""
     g = torch.Generator().manual_seed(seed)
     if dist == "uniform":

@@ -95,7 +95,7 @@ def test_forced_chunks_agree(cuda):
 
 
 def test_full_size_config4_sample(cuda):
-    # BASELINE's GQA configuration (b=64, 96/8 heads, contexts U[4096, 32768]); the oracle checks 6 of the sequences
+    # the benchmark's GQA configuration (b=64, 96/8 heads, contexts U[4096, 32768]); the oracle checks 6 of the sequences
     g = torch.Generator().manual_seed(44)
     act = torch.randint(4096, 32769, (6,), generator=g).tolist()
     case = gqa.make_case(6, 1, 96, 8, act, seed=44)

@@ -116,7 +116,7 @@ def test_contexts_beyond_131072_tokens(cuda):
 
 
 def test_full_size_config3(cuda):
-    # BASELINE config 3: b=32, 64x128 index heads, context lengths U[8192, 65536], top-2048
+    # benchmark configuration 3: b=32, 64x128 index heads, context lengths U[8192, 65536], top-2048
     g = torch.Generator().manual_seed(33)
     act = torch.randint(8192, 65537, (32,), generator=g).tolist()
     case = oi.make_case(32, 1, act, seed=33)

@@ -45,7 +45,7 @@ def test_reference_test_shapes(cuda):
 
 
 def test_config2_grouped(cuda):
-    # BASELINE's expert-selector configuration: 8192 tokens x 160 experts, bf16 logits, fp32 bias, 8 groups, top-4
+    # the benchmark's expert-selector configuration: 8192 tokens x 160 experts, bf16 logits, fp32 bias, 8 groups, top-4
     # groups, top-8 experts, renormalised, x 2.5
     logits, bias = ose.make_case(8192, 160, 2, logits_dtype=torch.bfloat16, bias_dtype=torch.float32)
     check(logits, bias, 8, True, 4, 8, cuda, scale=2.5, neg=True)

@@ -1,6 +1,6 @@
 """GPU parity: sparse flash attention (HIP, through the C ABI) against the CPU oracle.
 
-Bars.  BASELINE: every element within 1e-2 absolute + 2e-2 relative of the reference's golden (checked against
+Bars.  The benchmark's own: every element within 1e-2 absolute + 2e-2 relative of the reference's golden (checked against
 both of its goldens, no-flash and flash).  The reference's own comparator (at most 0.5 % of elements outside
 1e-4 + 5e-3 relative) presumes the golden's rounding points for P; the kernel rounds P~ = exp(s - m) to bf16
 relative to its running maximum, as the reference's online-softmax golden does per tile, and the two goldens
@@ -50,7 +50,7 @@ def full_check(out, case, name):
 
 
 def test_tiny_config1(cuda):
-    # BASELINE config 1: b=1, 16 heads, 4096-token cache, top-256, scale 1/sqrt(192)
+    # benchmark configuration 1: b=1, 16 heads, 4096-token cache, top-256, scale 1/sqrt(192)
     case = osfa.make_case(1, 16, 1, [4096], topk=256, seed=7, dist="bench", softmax_scale=192 ** -0.5)
     full_check(run_sfa(case, cuda), case, "config1")
 
@@ -155,7 +155,7 @@ def test_forced_kv_splits_agree(cuda):
 
 
 def test_full_size_config5(cuda):
-    # BASELINE config 5: b=32, 128 heads, context lengths U[16384, 65536], top-2048, bench distribution
+    # benchmark configuration 5: b=32, 128 heads, context lengths U[16384, 65536], top-2048, bench distribution
     g = torch.Generator().manual_seed(55)
     act = torch.randint(16384, 65537, (32,), generator=g).tolist()
     case = osfa.make_case(32, 128, 1, act, topk=2048, seed=55, dist="bench", softmax_scale=192 ** -0.5)
