@@ -45,6 +45,8 @@ def parse():
     ap.add_argument("--batch", type=int, default=32)
     ap.add_argument("--ctx", type=int, default=65536)
     ap.add_argument("--s1", type=int, default=1)
+    ap.add_argument("--ctx-min", type=int, default=0,
+                    help="v32 workload: draw every context length from U{ctx-min..ctx} (seeded) instead of ctx for all")
     ap.add_argument("--cpu-seqs", type=int, default=8, help="sequences of the workload timed on the CPU oracle")
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--packed", action="store_true", help="use the packed 656-byte-row attention entry point")
@@ -61,7 +63,7 @@ def parse():
     return ap.parse_args()
 
 
-def make_workload(torch, dev, b, ctx, s1, nbuf, seed=0):
+def make_workload(torch, dev, b, ctx, s1, nbuf, seed=0, ctx_min=0):
     g = torch.Generator(device=dev).manual_seed(seed)
     bs = 128
     pages_per_seq = (ctx + bs - 1) // bs
@@ -85,7 +87,8 @@ def make_workload(torch, dev, b, ctx, s1, nbuf, seed=0):
         "idx_w": (torch.randn((t, 64), generator=g, device=dev) / 8).to(torch.float16),
         "q_nope": torch.randn((t * 128, 512), generator=g, device=dev).to(torch.bfloat16),
         "q_rope": torch.randn((t * 128, 64), generator=g, device=dev).to(torch.bfloat16),
-        "act": torch.full((b,), ctx, dtype=torch.int32, device=dev),
+        "act": (torch.randint(ctx_min, ctx + 1, (b,), generator=g, device=dev).to(torch.int32) if ctx_min
+                else torch.full((b,), ctx, dtype=torch.int32, device=dev)),
         "topk_res": torch.zeros((t, 1, 2048), dtype=torch.int32, device=dev),
         "out": torch.zeros((b, s1, 128, 512), dtype=torch.bfloat16, device=dev),
     }
@@ -477,7 +480,8 @@ def main():
     b, ctx, s1 = args.batch, args.ctx, args.s1
     scale = 192 ** -0.5
     nbuf = 3
-    w = make_workload(torch, dev, b, ctx, s1, nbuf)
+    w = make_workload(torch, dev, b, ctx, s1, nbuf, ctx_min=args.ctx_min)
+    lengths = w["act"].tolist()
     if args.packed:
         for s in w["sets"]:
             rows = torch.empty((s["kn"].shape[0], 656), dtype=torch.int8, device=dev)
@@ -546,19 +550,19 @@ def main():
     kernels = read_kernel_times(lib)
 
     t = b * s1
-    L = ctx
-    # algorithmic traffic / work per launch
-    score_bytes = b * (L * 128 + L * 2 + (L + 127) // 128 * 4) + t * (64 * 128 + 64 * 2 + 64 * 2)
+    # algorithmic traffic / work per launch, summed over the sequences' lengths
+    score_bytes = sum(L * 128 + L * 2 + (L + 127) // 128 * 4 for L in lengths) + t * (64 * 128 + 64 * 2 + 64 * 2)
     topk_bytes = t * 2048 * 4
-    cur = min(L, 2048)
-    sfa_bytes = t * (cur * 656 + 128 * 576 * 2 + 128 * 512 * 2 + 2048 * 4)
-    sfa_flops = t * 278528 * cur
+    curs = [min(max(L - s1 + 1 + i, 0), 2048) for L in lengths for i in range(s1)]
+    sfa_bytes = sum(cur * 656 for cur in curs) + t * (128 * 576 * 2 + 128 * 512 * 2 + 2048 * 4)
+    sfa_flops = sum(278528 * cur for cur in curs)
+    select_bytes = s1 * sum(lengths) * 4
     info = {
         "indexer_score_kernel": {"bound": "hbm", "work": score_bytes, "peak": HBM_PEAK_GBS, "unit": "GB/s"},
         "indexer_topk_kernel": {"bound": "hbm", "work": topk_bytes, "peak": HBM_PEAK_GBS, "unit": "GB/s"},
         "sfa_decode_kernel": {"bound": "mfma", "work": sfa_flops, "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s"},
         "sfa_combine_kernel": {"bound": "hbm", "work": t * 128 * 512 * 2, "peak": HBM_PEAK_GBS, "unit": "GB/s"},
-        "indexer_select_kernel": {"bound": "hbm", "work": t * L * 4, "peak": HBM_PEAK_GBS, "unit": "GB/s"},
+        "indexer_select_kernel": {"bound": "hbm", "work": select_bytes, "peak": HBM_PEAK_GBS, "unit": "GB/s"},
     }
     per_kernel = []
     for name, us in kernels.items():
@@ -569,7 +573,7 @@ def main():
                            "peak": k["peak"], "unit": k["unit"], "frac": round(achieved / k["peak"], 4)})
     per_kernel.sort(key=lambda r: -r["us"])
     dom = per_kernel[0]
-    default_workload = (b, ctx, s1, args.packed) == (32, 65536, 1, False)
+    default_workload = (b, ctx, s1, args.packed, args.ctx_min) == (32, 65536, 1, False, 0)
     roofline = {"kernel": dom["kernel"], "bound": dom["bound"], "achieved": dom["achieved"], "peak": dom["peak"],
                 "unit": dom["unit"], "frac": dom["frac"],
                 "traffic": MEASURED_TRAFFIC_BYTES.get(dom["kernel"]) if default_workload else None,
@@ -590,7 +594,7 @@ def main():
         "vs_baseline": None, "dtype": "int8+bf16",
         "data": "synthetic", "launch": "hip graph replay" if args.graph else "eager",
         "config": {"workload": f"lightning indexer top-2048 + sparse flash attention decode, batch {b}, "
-                               f"s1 {s1}, ctx {ctx}, 64x128 int8 index heads, 128 heads x (512 nope + 64 rope), "
+                               f"s1 {s1}, ctx {f'U[{args.ctx_min}, {ctx}]' if args.ctx_min else ctx}, 64x128 int8 index heads, 128 heads x (512 nope + 64 rope), "
                                f"int8 paged MLA cache, block 128, {'packed 656 B rows' if args.packed else 'three cache tensors'}"},
         "roofline": roofline, "kernels": per_kernel, "event_pair_offset_us": round(read_kernel_times.offset_us, 2),
         "cpu_baseline": cpu_baseline,
@@ -606,7 +610,7 @@ def time_cpu_oracle(torch, w, n_seq, scale):
     s = w["sets"][0]
     host = {k: v.cpu() for k, v in s.items() if k != "rows"}
     table = w["table"][:n_seq].cpu()
-    act = [ctx] * n_seq
+    act = w["act"][:n_seq].tolist()
     t = n_seq * s1
     idx_q, idx_qs, idx_w = w["idx_q"][:t].cpu(), w["idx_qs"][:t].cpu(), w["idx_w"][:t].cpu()
     q = torch.cat([w["q_nope"][:t * 128].cpu().reshape(n_seq, s1, 128, 512),
