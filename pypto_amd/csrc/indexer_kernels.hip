@@ -190,22 +190,40 @@ __global__ __launch_bounds__(256, S1 == 1 ? 3 : 2) void indexer_score_paged_kern
     __shared__ __align__(16) float s_sc[S1][CHUNK * PPASSES]; // the workgroup's scores, written out in one burst at the end
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int l16 = lane & 15, g = lane >> 4;
-    const int bi = blockIdx.y;
     const int sgrp = blockIdx.z;
-    const int row0 = bi * a.s1 + sgrp * S1;
     const int bs = a.block_size;
-    const int wtok = blockIdx.x * (CHUNK * PPASSES) + wave * 128; // first key of this wave's pass 0
-
-    // The sequence length and the page-table entries are fetched together (one round trip before the first key load,
-    // not two): lane p takes the entry of pass p and the sequence's first entry, and picks once the length is known.
-    // lane p then holds the first cache row of pass p (-1: unmapped page); a pass past the end re-reads the sequence's
+    // The (sequence, 2048-key span) of this workgroup: by its place in the grid, or - when the span list exists - entry
+    // w of the list, w its place in launch order.  The list entry is fetched together with the sequence length and the
+    // page-table entries of the grid place; only if it names another span (ragged lengths) are those fetched again.
+    // Lane p takes the page-table entry of pass p and the sequence's first entry, and picks once the length is known:
+    // it then holds the first cache row of pass p (-1: unmapped page); a pass past the end re-reads the sequence's
     // first page and is discarded.
-    const int mytok = wtok + (lane < PPASSES ? lane : 0) * CHUNK;
-    const int32_t* bt = a.block_table + (int64_t)bi * a.bt_stride;
-    const int pg_mine = bt[min(mytok / bs, a.bt_stride - 1)];
-    const int pg_first = bt[0];
-    const int L = a.act_seq[bi];
-    if (blockIdx.x * (CHUNK * PPASSES) >= L) return;
+    int bi = blockIdx.y, span = blockIdx.x;
+    const uint32_t w = blockIdx.x + gridDim.x * blockIdx.y;
+    const bool listed = a.span_list != nullptr;
+    // (unconditional loads - from the lengths when there is no list - so that they travel with the ones below)
+    const uint32_t* lp = listed ? a.span_list : reinterpret_cast<const uint32_t*>(a.act_seq);
+    const uint32_t lp_count = lp[0], lp_item = lp[listed ? 1 + min(w, (uint32_t)SPAN_LIST_CAP - 1) : 0];
+    int pg_mine, pg_first, L, mytok;
+    auto fetch = [&]() {
+        mytok = span * (CHUNK * PPASSES) + wave * 128 + (lane < PPASSES ? lane : 0) * CHUNK;
+        const int32_t* bt = a.block_table + (int64_t)bi * a.bt_stride;
+        pg_mine = bt[min(mytok / bs, a.bt_stride - 1)];
+        pg_first = bt[0];
+        L = a.act_seq[bi];
+    };
+    fetch();
+    if (listed) {
+        if (w >= lp_count) return;
+        if (lp_item != (((uint32_t)bi << 10) | (uint32_t)span)) {
+            bi = (int)(lp_item >> 10);
+            span = (int)(lp_item & 1023u);
+            fetch();
+        }
+    }
+    if (span * (CHUNK * PPASSES) >= L) return;
+    const int row0 = bi * a.s1 + sgrp * S1;
+    const int wtok = span * (CHUNK * PPASSES) + wave * 128; // first key of this wave's pass 0
     int64_t myrow;
     {
         const int tc = mytok < L ? mytok : 0;
@@ -291,7 +309,7 @@ __global__ __launch_bounds__(256, S1 == 1 ? 3 : 2) void indexer_score_paged_kern
 #pragma unroll
         for (int s = 0; s < S1; ++s) {
             const float sc = res[s] * ks;
-            s_sc[s][tok - (int)blockIdx.x * (CHUNK * PPASSES)] = sc;
+            s_sc[s][tok - span * (CHUNK * PPASSES)] = sc;
             const int eff = L - (a.s1 - 1 - (sgrp * S1 + s));
             if (tok < eff) atomicAdd(&hist[s][score_key(sc) >> 21], 1u);
         }
@@ -316,7 +334,7 @@ __global__ __launch_bounds__(256, S1 == 1 ? 3 : 2) void indexer_score_paged_kern
     // 2 us more); score rows are padded to whole workgroup spans, so no bounds check
 #pragma unroll
     for (int s = 0; s < S1; ++s) {
-        float* dst = a.scores + (int64_t)(row0 + s) * a.score_stride + (int64_t)blockIdx.x * (CHUNK * PPASSES);
+        float* dst = a.scores + (int64_t)(row0 + s) * a.score_stride + (int64_t)span * (CHUNK * PPASSES);
 #pragma unroll
         for (int i = 0; i < CHUNK * PPASSES / 1024; ++i)
             *reinterpret_cast<f32x4*>(dst + 4 * (tid + 256 * i)) = *reinterpret_cast<const f32x4*>(&s_sc[s][4 * (tid + 256 * i)]);
@@ -325,12 +343,6 @@ __global__ __launch_bounds__(256, S1 == 1 ? 3 : 2) void indexer_score_paged_kern
         const uint32_t c = (&hist[0][0])[i];
         if (c) atomicAdd(a.hist + (int64_t)(row0 + i / NBINS) * NBINS + (i % NBINS), c);
     }
-}
-
-__global__ void indexer_zero_kernel(uint32_t* p, int n)
-{
-    const int i = blockIdx.x * blockDim.x + threadIdx.x;
-    if (i < n) p[i] = 0u;
 }
 
 __global__ void indexer_fill_kernel(int32_t* p, int n, int32_t v)
@@ -355,6 +367,39 @@ __device__ __forceinline__ uint32_t block_suffix_sum(uint32_t v, uint32_t* tmp)
     uint32_t add = 0;
     for (int w = wave + 1; w < NWAVES; ++w) add += tmp[w];
     return v + add;
+}
+
+// Clears the histograms and counters; its first workgroup also lists the 2048-key spans that hold keys, in launch
+// order of the score kernel's grid (sequence-major): span_list[0] = their number, span_list[1 + i] = sequence << 10 | span.
+// The score kernel's workgroup i takes entry i, so that with ragged lengths the workgroups that have work are the
+// first ones of the launch order and spread evenly over the CUs (when every sequence fills its spans the list is the
+// identity and changes nothing).  256 lanes per workgroup.
+__global__ __launch_bounds__(256) void indexer_zero_kernel(uint32_t* p, int n, const int32_t* act_seq, int b, int pchunks,
+                                                           uint32_t* span_list)
+{
+    const int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) p[i] = 0u;
+    if (blockIdx.x != 0 || span_list == nullptr) return;
+    __shared__ uint32_t tmp[4];
+    __shared__ uint32_t s_total;
+    const int tid = threadIdx.x;
+    uint32_t base_off = 0;
+    for (int base = 0; base < b; base += 256) {
+        const int seq = base + tid;
+        uint32_t cnt = 0;
+        if (seq < b) {
+            const int L = act_seq[seq];
+            cnt = L > 0 ? (uint32_t)min((L + CHUNK * PPASSES - 1) / (CHUNK * PPASSES), pchunks) : 0u;
+        }
+        const uint32_t suffix = block_suffix_sum<4>(cnt, tmp); // sum over lanes tid .. 255
+        if (tid == 0) s_total = suffix;
+        __syncthreads();
+        const uint32_t off = base_off + (s_total - suffix); // spans of the sequences before this one
+        for (uint32_t j = 0; j < cnt; ++j) span_list[1 + off + j] = ((uint32_t)seq << 10) | j;
+        base_off += s_total;
+        __syncthreads();
+    }
+    if (tid == 0) span_list[0] = base_off;
 }
 
 // Valid length of query token `row`'s score row.
@@ -655,7 +700,7 @@ static uint64_t align256(uint64_t x) { return (x + 255) & ~(uint64_t)255; }
 uint64_t indexer_workspace_bytes(int t, int stride)
 {
     return align256((uint64_t)t * stride * 4) + align256((uint64_t)t * (NBINS + 4) * 4) +
-           (uint64_t)t * (MAX_K + TIE_CAP) * 8;
+           align256((uint64_t)t * (MAX_K + TIE_CAP) * 8) + (1 + SPAN_LIST_CAP) * 4;
 }
 
 void indexer_bind_workspace(IndexerArgs& a, void* ws)
@@ -669,6 +714,8 @@ void indexer_bind_workspace(IndexerArgs& a, void* ws)
     p += align256((uint64_t)t * (NBINS + 4) * 4);
     a.winners = reinterpret_cast<uint64_t*>(p);
     a.ties = a.winners + (uint64_t)t * MAX_K;
+    p += align256((uint64_t)t * (MAX_K + TIE_CAP) * 8);
+    a.span_list = reinterpret_cast<uint32_t*>(p); // the launch drops it when the grid does not fit
 }
 
 hipError_t indexer_launch(const IndexerArgs& a, hipStream_t stream)
@@ -684,15 +731,19 @@ hipError_t indexer_launch(const IndexerArgs& a, hipStream_t stream)
     const int chunks = (max_ctx + CHUNK * PASSES - 1) / (CHUNK * PASSES);
     const int pchunks = (max_ctx + CHUNK * PPASSES - 1) / (CHUNK * PPASSES);
     const int nzero = t * (NBINS + 4);
-    hipLaunchKernelGGL(indexer_zero_kernel, dim3((nzero + 255) / 256), dim3(256), 0, stream, a.hist, nzero);
+    IndexerArgs args = a;
+    const bool paged = a.block_size % 128 == 0;
+    if (!paged || (int64_t)a.b * pchunks > SPAN_LIST_CAP || pchunks > 1024) args.span_list = nullptr;
+    hipLaunchKernelGGL(indexer_zero_kernel, dim3((nzero + 255) / 256), dim3(256), 0, stream, a.hist, nzero, a.act_seq, a.b,
+                       pchunks, args.span_list);
     {
         ScopedKernelTimer tm(KID_INDEXER_SCORE, stream);
         const bool pow2 = (a.block_size & (a.block_size - 1)) == 0;
         if (a.block_size % 128 == 0) {
             if (a.s1 % 2 == 0)
-                hipLaunchKernelGGL(indexer_score_paged_kernel<2>, dim3(pchunks, a.b, a.s1 / 2), dim3(256), 0, stream, a);
+                hipLaunchKernelGGL(indexer_score_paged_kernel<2>, dim3(pchunks, a.b, a.s1 / 2), dim3(256), 0, stream, args);
             else
-                hipLaunchKernelGGL(indexer_score_paged_kernel<1>, dim3(pchunks, a.b, a.s1), dim3(256), 0, stream, a);
+                hipLaunchKernelGGL(indexer_score_paged_kernel<1>, dim3(pchunks, a.b, a.s1), dim3(256), 0, stream, args);
         } else if (a.s1 % 2 == 0) {
             auto kern = pow2 ? indexer_score_kernel<2, true> : indexer_score_kernel<2, false>;
             hipLaunchKernelGGL(kern, dim3(chunks, a.b, a.s1 / 2), dim3(256), 0, stream, a);

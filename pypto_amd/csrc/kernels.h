@@ -48,10 +48,13 @@ struct IndexerArgs {
     uint32_t* counters;          // workspace [t, 4]: winners, ties
     uint64_t* winners;           // workspace [t, 2048]
     uint64_t* ties;              // workspace [t, 8192]
+    uint32_t* span_list;         // workspace [1 + SPAN_LIST_CAP]: count, then (sequence << 10 | span) of every 2048-key span
+                                 // that holds keys; nullptr when the grid is too large for the list
     int64_t n_blocks;
     int32_t b, s1, nh, block_size, bt_stride, k, score_stride;
 };
 
+constexpr int SPAN_LIST_CAP = 16384;
 uint64_t indexer_workspace_bytes(int t, int score_stride);
 void indexer_bind_workspace(IndexerArgs& a, void* workspace);
 hipError_t indexer_launch(const IndexerArgs& a, hipStream_t stream);
