@@ -41,14 +41,14 @@ constexpr int MAX_SPLIT_TOKENS = 2048; // largest share of a top-k list one work
 constexpr int NREG_KSTEPS = 12;        // of a wave's 18 k-steps of Q, these stay in registers ...
 constexpr int NPARK = KSTEPS / 2 - NREG_KSTEPS; // ... and these are parked in LDS (16 bytes per lane each)
 // LDS layout: two tile stages | S exchange | parked Q | per-split arrays sized by SfaArgs::split_cap
-// (validity words, rows, scales) | this sequence's page table (when it fits)
+// (validity words, rows) | this sequence's page table (when it fits)
 constexpr int XBUF_OFF = 2 * STAGE;
 constexpr int QPARK_OFF = XBUF_OFF + 4 * 4096;
 constexpr int SPLIT_OFF = QPARK_OFF + 4 * NPARK * 1024; // 114688
 constexpr int LDS_LIMIT = 160 * 1024;
 constexpr int OUT_ROW = DN * 4;  // epilogue staging: 64 heads x 512 fp32, reusing the front of LDS
 __host__ __device__ constexpr int tmask_bytes(int cap) { return (cap / T + 2) * 4; }
-__host__ __device__ constexpr int split_bytes(int cap) { return tmask_bytes(cap) + cap * 4 + cap * 16; }
+__host__ __device__ constexpr int split_bytes(int cap) { return tmask_bytes(cap) + cap * 4; }
 static_assert(64 * OUT_ROW <= LDS_LIMIT, "epilogue staging must fit");
 constexpr int HEADS_PER_WG = 64;
 
@@ -69,6 +69,7 @@ struct RawTile;
 template <>
 struct RawTile<true> {
     u32x2 nope[8]; // 8 rows x 8 int8 (this lane's 8 columns)
+    float sc[8];   // the rows' dequant scales for this lane's column group
     u32x4 rope;
     uint32_t absent;
 };
@@ -94,9 +95,10 @@ __device__ __forceinline__ void load_raw(RawTile<QUANT>& r, const SfaArgs& a, co
 #pragma unroll
     for (int e = 0; e < 8; ++e) {
         const uint32_t row = __builtin_amdgcn_readfirstlane(e < 4 ? ra[e & 3] : rb[e & 3]);
-        if constexpr (QUANT)
+        if constexpr (QUANT) {
             r.nope[e] = *reinterpret_cast<const u32x2*>(a.kn + (uint64_t)row * a.kn_stride + lane * 8);
-        else
+            r.sc[e] = *reinterpret_cast<const float*>(a.ks + (uint64_t)row * a.ks_stride + (lane >> 4) * 4);
+        } else
             r.nope[e] = *reinterpret_cast<const u32x4*>(a.kn + (uint64_t)row * a.kn_stride + lane * 16);
     }
     const uint32_t row = (uint32_t)rows[tile * T + (tid >> 3)];
@@ -116,18 +118,18 @@ __device__ __forceinline__ float dq(uint32_t w, int k, float s, float neg128s)
 // Dequantise rows [E0, E1) of this lane's 8 rows x 8 columns and store them into an LDS stage; with ROPE also
 // the lane's rope piece.
 template <bool QUANT, int E0, int E1, bool ROPE>
-__device__ __forceinline__ void dequant_store(const RawTile<QUANT>& r, uint8_t* stage, const float* scales, int tile,
-                                              int wave, int lane, int tid)
+__device__ __forceinline__ void dequant_store(const RawTile<QUANT>& r, uint8_t* stage, int wave, int lane, int tid)
 {
 #pragma unroll
     for (int e = E0; e < E1; ++e) {
         const int t = 8 * wave + e;
         u32x4 v;
         if constexpr (QUANT) {
-            const float s = scales[(tile * T + t) * 4 + (lane >> 4)]; // 0 for an absent row
             uint32_t w0 = r.nope[e][0], w1 = r.nope[e][1];
+            float s = r.sc[e];
             // keep the unpacking here: hoisted to the load, it would wait for the load right after issuing it
-            asm volatile("" : "+v"(w0), "+v"(w1));
+            asm volatile("" : "+v"(w0), "+v"(w1), "+v"(s));
+            s = ((r.absent >> e) & 1u) ? 0.f : s; // an absent row is stored as zeros
             w0 ^= 0x80808080u;
             w1 ^= 0x80808080u;
             const float c = -128.f * s;
@@ -152,10 +154,10 @@ __device__ __forceinline__ void dequant_store(const RawTile<QUANT>& r, uint8_t* 
 }
 
 // Resolves a workgroup's share of a token's top-k list: logical indices -> physical cache rows (absent entries: row 0
-// and a cleared bit in the tile's validity word) and their 4 dequant scales (0 when absent), all in LDS.  NT lanes.
-template <int NT, bool QUANT>
+// and a cleared bit in the tile's validity word), in LDS.  NT lanes.
+template <int NT>
 __device__ __forceinline__ void resolve_split(const SfaArgs& a, int bi, int tq, int tok0, int cur, int ntiles_real,
-                                              int ntiles, uint32_t* tmask, int* rows, float* scales, int* bt_lds, int tid,
+                                              int ntiles, uint32_t* tmask, int* rows, int* bt_lds, int tid,
                                               int lane)
 {
     // this sequence's page table -> LDS (saves one dependent global load per selected token)
@@ -190,13 +192,8 @@ __device__ __forceinline__ void resolve_split(const SfaArgs& a, int bi, int tq, 
             tmask[i >> 5] = (uint32_t)present;
             tmask[(i >> 5) + 1] = (uint32_t)(present >> 32);
         }
-        if constexpr (QUANT) {
-            f32x4 sc = {0.f, 0.f, 0.f, 0.f};
-            if (row >= 0) sc = *reinterpret_cast<const f32x4*>(a.ks + (uint64_t)row * a.ks_stride);
-            *reinterpret_cast<f32x4*>(scales + i * 4) = sc;
-        }
     }
-    __syncthreads(); // rows[] / scales[] / tmask[] ready
+    __syncthreads(); // rows[] / tmask[] ready
 }
 
 template <bool QUANT>
@@ -206,7 +203,6 @@ __global__ __attribute__((amdgpu_flat_work_group_size(512, 512), amdgpu_waves_pe
     extern __shared__ __align__(16) uint8_t smem[];
     uint32_t* tmask = reinterpret_cast<uint32_t*>(smem + SPLIT_OFF);
     int* rows = reinterpret_cast<int*>(smem + SPLIT_OFF + tmask_bytes(a.split_cap));
-    float* scales = reinterpret_cast<float*>(smem + SPLIT_OFF + tmask_bytes(a.split_cap) + a.split_cap * 4);
     int* bt_lds = reinterpret_cast<int*>(smem + SPLIT_OFF + split_bytes(a.split_cap));
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -223,7 +219,7 @@ __global__ __attribute__((amdgpu_flat_work_group_size(512, 512), amdgpu_waves_pe
     const int ntiles = (ntiles_real + 1) & ~1;
     const int tok0 = tile0 * T;
 
-    resolve_split<512, QUANT>(a, bi, tq, tok0, cur, ntiles_real, ntiles, tmask, rows, scales, bt_lds, tid, lane);
+    resolve_split<512>(a, bi, tq, tok0, cur, ntiles_real, ntiles, tmask, rows, bt_lds, tid, lane);
 
     // Both roles run the same barrier sequence: one before the first tile, then two per tile
     // (partial S exchanged; tile consumed and next tile stored).
@@ -237,7 +233,7 @@ __global__ __attribute__((amdgpu_flat_work_group_size(512, 512), amdgpu_waves_pe
         if (ntiles > 0) {
             load_raw<QUANT>(raw0, a, rows, tmask, 0, pw, lane, ptid);
             load_raw<QUANT>(raw1, a, rows, tmask, 1, pw, lane, ptid);
-            dequant_store<QUANT, 0, 8, true>(raw0, smem, scales, 0, pw, lane, ptid);
+            dequant_store<QUANT, 0, 8, true>(raw0, smem, pw, lane, ptid);
             load_raw<QUANT>(raw0, a, rows, tmask, min(2, last), pw, lane, ptid);
         }
         __syncthreads();
@@ -248,9 +244,9 @@ __global__ __attribute__((amdgpu_flat_work_group_size(512, 512), amdgpu_waves_pe
         // S MFMAs, the rest (and the loads of a later tile) beside softmax and PV.
         auto produce = [&](int it, RawTile<QUANT>& next) {
             uint8_t* dst = smem + ((it + 1) & 1) * STAGE;
-            dequant_store<QUANT, 0, 5, false>(next, dst, scales, min(it + 1, last), pw, lane, ptid);
+            dequant_store<QUANT, 0, 5, false>(next, dst, pw, lane, ptid);
             __syncthreads();
-            dequant_store<QUANT, 5, 8, true>(next, dst, scales, min(it + 1, last), pw, lane, ptid);
+            dequant_store<QUANT, 5, 8, true>(next, dst, pw, lane, ptid);
             load_raw<QUANT>(next, a, rows, tmask, min(it + 3, last), pw, lane, ptid);
             __syncthreads();
         };
