@@ -230,10 +230,10 @@ __global__ __attribute__((amdgpu_flat_work_group_size(512, 512), amdgpu_waves_pe
         const int pw = wave - 4, ptid = tid - 256;
         const int last = ntiles - 1;
         RawTile<QUANT> raw0, raw1;
+        // (tile 0 is gathered and stored by the consumer wavefronts, which would otherwise idle here: the cold first
+        // gathers are slow to issue, and two sets of waves issue them side by side)
         if (ntiles > 0) {
-            load_raw<QUANT>(raw0, a, rows, tmask, 0, pw, lane, ptid);
             load_raw<QUANT>(raw1, a, rows, tmask, 1, pw, lane, ptid);
-            dequant_store<QUANT, 0, 8, true>(raw0, smem, pw, lane, ptid);
             load_raw<QUANT>(raw0, a, rows, tmask, min(2, last), pw, lane, ptid);
         }
         __syncthreads();
@@ -269,6 +269,8 @@ __global__ __attribute__((amdgpu_flat_work_group_size(512, 512), amdgpu_waves_pe
     // every tile, which keeps the consumer inside its 256 registers.
     bf16x8 q[NREG_KSTEPS];
     uint8_t* qpark = smem + QPARK_OFF + wave * (NPARK * 1024) + lane * 16;
+    RawTile<QUANT> first; // tile 0: wave w takes rows 8w .. 8w + 7, as producer wave w does for the later tiles
+    if (ntiles > 0) load_raw<QUANT>(first, a, rows, tmask, 0, wave, lane, tid);
     {
         const int64_t qrow = (int64_t)tq * a.nq + (head_ok ? head : 0);
         const __bf16* qn = reinterpret_cast<const __bf16*>(a.q_nope) + qrow * DN + kh * 16 + hl * 8;
@@ -311,6 +313,7 @@ __global__ __attribute__((amdgpu_flat_work_group_size(512, 512), amdgpu_waves_pe
     }
     uint8_t* xmine = smem + XBUF_OFF + wave * 4096 + lane * 16;
 
+    if (ntiles > 0) dequant_store<QUANT, 0, 8, true>(first, smem, wave, lane, tid);
     __syncthreads(); // tile 0 stored
 
     for (int it = 0; it < ntiles; ++it) {
