@@ -415,15 +415,21 @@ __global__ __launch_bounds__(256) void indexer_select_kernel(IndexerArgs a)
     __shared__ uint32_t tmp[4];
     __shared__ uint32_t s_bin, s_base_gt, s_base_tie;
     const int tid = threadIdx.x, row = blockIdx.y;
-    const int n = row_length(a.act_seq, row, a.s1, a.score_stride);
     const int i_begin = blockIdx.x * SEL_CHUNK;
-    if (i_begin >= n) return;
-    if (tid == 0) s_bin = 0xffffffffu; // n <= k: no threshold bin, everything is a winner
-
-    // bin of the k-th largest key: lane t owns bins 8t .. 8t+7
+    // everything this workgroup reads is requested at once - the row's length, its histogram (lane t owns bins
+    // 8t .. 8t+7) and the workgroup's 16 scores per lane (addresses clamped to the padded row) - one round trip, not three
     const uint32_t* hist = a.hist + (int64_t)row * NBINS;
     const u32x4 ha = *reinterpret_cast<const u32x4*>(hist + 8 * tid);
     const u32x4 hb = *reinterpret_cast<const u32x4*>(hist + 8 * tid + 4);
+    const float* x = a.scores + (int64_t)row * a.score_stride;
+    f32x4 v[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) v[j] = *reinterpret_cast<const f32x4*>(x + min(i_begin + 4 * (j * 256 + tid), a.score_stride - 4));
+    const int n = row_length(a.act_seq, row, a.s1, a.score_stride);
+    if (i_begin >= n) return;
+    if (tid == 0) s_bin = 0xffffffffu; // n <= k: no threshold bin, everything is a winner
+
+    // bin of the k-th largest key
     const uint32_t h[8] = {ha[0], ha[1], ha[2], ha[3], hb[0], hb[1], hb[2], hb[3]};
     uint32_t own = 0;
 #pragma unroll
@@ -439,10 +445,6 @@ __global__ __launch_bounds__(256) void indexer_select_kernel(IndexerArgs a)
     const uint32_t bin = s_bin;
 
     // file this workgroup's scores: 16 per lane
-    const float* x = a.scores + (int64_t)row * a.score_stride;
-    f32x4 v[4];
-#pragma unroll
-    for (int j = 0; j < 4; ++j) v[j] = *reinterpret_cast<const f32x4*>(x + min(i_begin + 4 * (j * 256 + tid), a.score_stride - 4));
     uint32_t key[16];
     uint32_t c_gt = 0, c_tie = 0;
 #pragma unroll
@@ -649,13 +651,23 @@ __global__ __launch_bounds__(1024) void indexer_topk_kernel(IndexerArgs a)
     __shared__ uint32_t s_bin, s_krem, s_cnt, s_out;
 
     const int tid = threadIdx.x, row = blockIdx.x;
+    // the winners and the first 2048 ties are requested together with the counts that say how many of them are real
+    // (the lists are workspace memory: reading past their fill is harmless), one round trip instead of three
+    const uint64_t* wsrc = a.winners + (int64_t)row * MAX_K;
+    const uint64_t* tsrc = a.ties + (int64_t)row * TIE_CAP;
+    static_assert(MAX_K == 2048 && TIE_CAP >= 2048, "two winners and two early ties per lane");
+    const uint64_t w0 = wsrc[tid], w1 = wsrc[tid + 1024];
+    const uint64_t t0 = tsrc[tid], t1 = tsrc[tid + 1024];
     const int n = row_length(a.act_seq, row, a.s1, a.score_stride);
     const int k = a.k;
     const uint32_t n_gt = min(a.counters[(int64_t)row * 4], (uint32_t)MAX_K);
     const uint32_t n_tie = a.counters[(int64_t)row * 4 + 1];
     const uint32_t need = (uint32_t)min(n, k) - min(n_gt, (uint32_t)min(n, k));
 
-    for (int i = tid; i < MAX_K; i += 1024) cand[i] = i < (int)n_gt ? a.winners[(int64_t)row * MAX_K + i] : 0ull;
+    cand[tid] = tid < (int)n_gt ? w0 : 0ull;
+    cand[tid + 1024] = tid + 1024 < (int)n_gt ? w1 : 0ull;
+    tie[tid] = t0;
+    tie[tid + 1024] = t1;
     if (tid == 0) s_out = n_gt;
     __syncthreads();
     auto emit = [&](uint64_t w) {
@@ -665,8 +677,10 @@ __global__ __launch_bounds__(1024) void indexer_topk_kernel(IndexerArgs a)
 
     if (need > 0 && n_tie <= TIE_CAP) {
         // the usual case: the tie list (one histogram bin) fits in LDS; its words share the top 11 bits
-        for (int i = tid; i < (int)n_tie; i += 1024) tie[i] = a.ties[(int64_t)row * TIE_CAP + i];
-        __syncthreads();
+        if (n_tie > 2048) { // block-uniform
+            for (int i = tid + 2048; i < (int)n_tie; i += 1024) tie[i] = tsrc[i];
+            __syncthreads();
+        }
         auto each = [&](auto&& f) {
             for (int i = tid; i < (int)n_tie; i += 1024) f(tie[i]);
         };
