@@ -119,8 +119,8 @@ int bind_workspace(const char* op, SfaPlan* plan, void* ws, uint64_t ws_bytes)
                     (unsigned long long)plan->ws_bytes, (unsigned long long)(ws ? ws_bytes : 0));
     pto::SfaArgs& a = plan->args;
     const uint64_t rows = (uint64_t)a.b * a.s1 * a.nsplit * a.nq;
-    a.part_o = static_cast<float*>(ws);
-    a.part_ml = a.part_o + rows * 512;
+    a.part_o = static_cast<_Float16*>(ws);
+    a.part_ml = reinterpret_cast<float*>(a.part_o + rows * 512);
     return PTO_OK;
 }
 

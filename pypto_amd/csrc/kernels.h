@@ -20,7 +20,7 @@ struct SfaArgs {
     const int32_t* block_table; // [b, bt_stride]
     const int32_t* act_seq;     // [b]
     void* out;                  // [t*nq, 512] bf16
-    float* part_o;              // [t, nsplit, nq, 512] fp32 (nsplit > 1)
+    _Float16* part_o;           // [t, nsplit, nq, 512] fp16: each split's output normalised by its own sum (nsplit > 1)
     float* part_ml;             // [t, nsplit, nq, 2]  fp32 (running max in log2 units, sum)
     int32_t b, s1, nq, topk, topk_stride, block_size, bt_stride, nsplit;
     int32_t split_cap; // set by sfa_launch: capacity (tokens) of the per-split LDS arrays

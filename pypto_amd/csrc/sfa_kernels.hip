@@ -53,6 +53,7 @@ static_assert(64 * OUT_ROW <= LDS_LIMIT, "epilogue staging must fit");
 constexpr int HEADS_PER_WG = 64;
 
 typedef short s16x4 __attribute__((ext_vector_type(4)));
+typedef _Float16 f16x4 __attribute__((ext_vector_type(4)));
 typedef short s16x8 __attribute__((ext_vector_type(8)));
 typedef __attribute__((address_space(3))) s16x4 lds_s16x4;
 
@@ -448,7 +449,7 @@ __global__ __attribute__((amdgpu_flat_work_group_size(512, 512), amdgpu_waves_pe
     // chunks XOR-swizzled with the head so that the 8 lanes of a b128 write hit distinct banks.  Register r of
     // o[i] holds dim 32*(2*i + kh) + 8*(r/4) + 4*hl + r%4 of head l32.
     const float l_tot = l_run + __shfl_xor(l_run, 32);
-    const float mul = a.nsplit == 1 ? (l_tot > 0.f ? 1.f / l_tot : 0.f) : 1.f;
+    const float mul = l_tot > 0.f ? 1.f / l_tot : 0.f; // splits hand over their normalised output as well
     const int hrow = hg * 32 + l32;
     uint8_t* orow = smem + hrow * OUT_ROW;
 #pragma unroll
@@ -479,8 +480,11 @@ __global__ __attribute__((amdgpu_flat_work_group_size(512, 512), amdgpu_waves_pe
             const u32x2 w = {pack_bf16x2(v[0], v[1]), pack_bf16x2(v[2], v[3])};
             *reinterpret_cast<u32x2*>(reinterpret_cast<uint8_t*>(a.out) + (((int64_t)tq * a.nq + head) * DN + c * 4) * 2) = w;
         } else {
+            // a split's share, normalised by its own sum, in fp16: |value| <= max |V| and 2^-12 relative rounding, a
+            // quarter of the final bf16 rounding; half the bytes of fp32 for this kernel to write and the merge to read
             const int64_t prow = ((int64_t)tq * a.nsplit + sp) * a.nq + head;
-            *reinterpret_cast<f32x4*>(a.part_o + prow * DN + c * 4) = v;
+            const f16x4 hv = {(_Float16)v[0], (_Float16)v[1], (_Float16)v[2], (_Float16)v[3]};
+            *reinterpret_cast<f16x4*>(a.part_o + prow * DN + c * 4) = hv;
         }
     }
 }
@@ -492,8 +496,10 @@ __global__ void sfa_zero_kernel(uint32_t* out, int64_t n_words)
     if (i < n_words) out[i] = 0u;
 }
 
-// out[row, :] = sum_s 2^(m_s - M) O_s[row, :] / sum_s 2^(m_s - M) l_s ; one block of 128 lanes per output row
-__global__ __launch_bounds__(128) void sfa_combine_kernel(const float* __restrict__ part_o,
+// out[row, :] = sum_s (2^(m_s - M) l_s / L) o_s[row, :] with L = sum_s 2^(m_s - M) l_s and o_s the split's normalised
+// output; one block of 128 lanes per output row.  Splits are taken four at a time, every load of a group requested
+// before any is used (splits past the last are the last again with weight 0).
+__global__ __launch_bounds__(128) void sfa_combine_kernel(const _Float16* __restrict__ part_o,
                                                           const float* __restrict__ part_ml, void* out, int nq,
                                                           int nsplit)
 {
@@ -504,14 +510,20 @@ __global__ __launch_bounds__(128) void sfa_combine_kernel(const float* __restric
     float L = 0.f;
     f32x4 acc = {0.f, 0.f, 0.f, 0.f};
     if (M > -INFINITY) {
-        for (int s = 0; s < nsplit; ++s) {
-            const int64_t prow = ((int64_t)tq * nsplit + s) * nq + head;
-            const float l = part_ml[prow * 2 + 1];
-            if (l > 0.f) {
-                const float w = exp2f(part_ml[prow * 2] - M);
-                L += w * l;
-                const f32x4 v = *reinterpret_cast<const f32x4*>(part_o + prow * DN + threadIdx.x * 4);
-                acc += v * w;
+        for (int s0 = 0; s0 < nsplit; s0 += 4) {
+            f16x4 v[4];
+            float w[4];
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const int64_t prow = ((int64_t)tq * nsplit + min(s0 + j, nsplit - 1)) * nq + head;
+                v[j] = *reinterpret_cast<const f16x4*>(part_o + prow * DN + threadIdx.x * 4);
+                const float m = part_ml[prow * 2], l = part_ml[prow * 2 + 1];
+                w[j] = (s0 + j < nsplit && l > 0.f) ? exp2f(m - M) * l : 0.f;
+            }
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                L += w[j];
+                acc += f32x4{(float)v[j][0], (float)v[j][1], (float)v[j][2], (float)v[j][3]} * w[j];
             }
         }
     }
@@ -549,7 +561,7 @@ int sfa_pick_splits(int t, int nq, int topk)
 uint64_t sfa_workspace_bytes(int t, int nq, int nsplit)
 {
     if (nsplit <= 1) return 0;
-    return (uint64_t)t * nsplit * nq * (DN + 2) * sizeof(float);
+    return (uint64_t)t * nsplit * nq * (DN * sizeof(_Float16) + 2 * sizeof(float));
 }
 
 hipError_t sfa_launch(const SfaArgs& a, hipStream_t stream)
