@@ -499,10 +499,11 @@ __global__ void sfa_zero_kernel(uint32_t* out, int64_t n_words)
 // out[row, :] = sum_s (2^(m_s - M) l_s / L) o_s[row, :] with L = sum_s 2^(m_s - M) l_s and o_s the split's normalised
 // output; one block of 128 lanes per output row.  Splits are taken four at a time, every load of a group requested
 // before any is used (splits past the last are the last again with weight 0).
-__global__ __launch_bounds__(128) void sfa_combine_kernel(const _Float16* __restrict__ part_o,
+__global__ __launch_bounds__(128) void sfa_combine_kernel(const void* __restrict__ part_o_fp16,
                                                           const float* __restrict__ part_ml, void* out, int nq,
                                                           int nsplit)
 {
+    const _Float16* part_o = static_cast<const _Float16*>(part_o_fp16); // (a plain pointer type keeps the symbol readable)
     const int row = blockIdx.x; // tq * nq + head
     const int tq = row / nq, head = row - tq * nq;
     float M = -INFINITY;
@@ -599,7 +600,7 @@ hipError_t sfa_launch(const SfaArgs& a, hipStream_t stream)
     if (e != hipSuccess) return e;
     if (a.nsplit > 1) {
         ScopedKernelTimer tm(KID_SFA_COMBINE, stream);
-        hipLaunchKernelGGL(sfa_combine_kernel, dim3(t * a.nq), dim3(128), 0, stream, a.part_o, a.part_ml, a.out, a.nq,
+        hipLaunchKernelGGL(sfa_combine_kernel, dim3(t * a.nq), dim3(128), 0, stream, static_cast<const void*>(a.part_o), a.part_ml, a.out, a.nq,
                            a.nsplit);
         e = hipGetLastError();
     }
