@@ -144,6 +144,22 @@ def test_coincident_scores_of_different_keys(cuda):
     check_topk(case, run_indexer(case, cuda))
 
 
+def test_wide_page_table_many_sequences(cuda):
+    # 300 short sequences under a page table wide enough for 112 K tokens: 300 x 55 spans of 2048 keys, more than the
+    # score kernel's span list holds, so its workgroups take their spans by grid place; and the same sequences under a
+    # narrower table, where the list is used and most of its grid has no work
+    g = torch.Generator().manual_seed(41)
+    act = torch.randint(1, 700, (300,), generator=g).tolist()
+    case = oi.make_case(300, 1, act, seed=41, selected_count=64)
+    gold_scores = indexer_scores(case, exact=True)
+    narrow = run_indexer(case, cuda)
+    check_topk(case, narrow, exact=gold_scores)
+    bt = case["block_table"]
+    wide = dict(case)
+    wide["block_table"] = torch.cat([bt, torch.full((bt.shape[0], 880 - bt.shape[1]), -1, dtype=bt.dtype)], dim=1).contiguous()
+    assert torch.equal(run_indexer(wide, cuda), narrow)
+
+
 def test_other_selection_sizes_and_block_sizes(cuda):
     case = oi.make_case(2, 1, [1000, 70], seed=8, selected_count=64)
     check_topk(case, run_indexer(case, cuda))
