@@ -65,12 +65,12 @@ def test_tensor_desc_layout_matches_the_reference_abi():
 def test_sfa_workspace_query(lib):
     p = SfaParams(128, 1, 0.1, 2048, 128, 8, 4)
     ws = lib.pto_sfa_quant_workspace(descs(sfa_specs()), 9, ctypes.byref(p))
-    assert ws == 2 * 4 * 128 * (512 + 2) * 4  # t * splits * nq * (512 + m, l) fp32
+    assert ws == 2 * 4 * 128 * (512 * 2 + 2 * 4)  # t * splits * nq * (512 fp16 + (m, l) fp32)
     p.kv_splits = 1
     assert lib.pto_sfa_quant_workspace(descs(sfa_specs()), 9, ctypes.byref(p)) == 0  # single pass: no scratch
     p.kv_splits = 0  # automatic: some positive split count on a 256-CU part, never more than 16
     auto = lib.pto_sfa_quant_workspace(descs(sfa_specs()), 9, ctypes.byref(p))
-    assert auto % (2 * 128 * 514 * 4) == 0 and 1 <= auto // (2 * 128 * 514 * 4) <= 16
+    assert auto % (2 * 128 * 1032) == 0 and 1 <= auto // (2 * 128 * 1032) <= 16
 
 
 def launch_rc(lib, op, specs, params, ws=None, ws_bytes=0):
