@@ -480,7 +480,7 @@ __global__ __attribute__((amdgpu_flat_work_group_size(512, 512), amdgpu_waves_pe
             const u32x2 w = {pack_bf16x2(v[0], v[1]), pack_bf16x2(v[2], v[3])};
             *reinterpret_cast<u32x2*>(reinterpret_cast<uint8_t*>(a.out) + (((int64_t)tq * a.nq + head) * DN + c * 4) * 2) = w;
         } else {
-            // a split's share, normalised by its own sum, in fp16: |value| <= max |V| and 2^-12 relative rounding, a
+            // a split's share, normalised by its own sum, in fp16: |value| <= max |V| and 2^-11 relative rounding, a
             // quarter of the final bf16 rounding; half the bytes of fp32 for this kernel to write and the merge to read
             const int64_t prow = ((int64_t)tq * a.nsplit + sp) * a.nq + head;
             const f16x4 hv = {(_Float16)v[0], (_Float16)v[1], (_Float16)v[2], (_Float16)v[3]};
