@@ -54,6 +54,9 @@ def parse():
                     help="v32 (default): the headline DeepSeek-V3.2 indexer + sparse attention decode step; gqa: GLM-4.5 "
                          "paged GQA decode (batch 64, 96/8 heads, contexts U[4096, 32768]); select_experts: GLM-4.5 "
                          "router (8192 tokens x 160 experts)")
+    ap.add_argument("--warm-weights", action="store_true",
+                    help="prolog workloads: one copy of the weights, re-read every step (they then partly come out of "
+                         "the 256 MB last-level cache); default: rotate enough copies to exceed it")
     ap.add_argument("--graph", action="store_true",
                     help="replay the step from HIP graphs (one per cache copy) instead of launching it eagerly")
     ap.add_argument("--calibrate-copy", action="store_true",
@@ -114,10 +117,25 @@ def read_kernel_times(lib):
     return kernels
 
 
-def timed(torch, lib, step, args):
+def rotated(torch, tensors, weight_idx, args):
+    """Copies of an operator's tensor list that differ in their weight tensors (the entries at weight_idx): enough of
+    them to exceed the 256 MB last-level cache, so that a step finds none of its weights there - the case a layer stack
+    is in.  One list when --warm-weights."""
+    nbytes = sum(tensors[i].numel() * tensors[i].element_size() for i in weight_idx)
+    copies = 1 if args.warm_weights else max(2, min(32, -(-320 * 2 ** 20 // max(nbytes, 1))))
+    sets = [tensors]
+    for _ in range(copies - 1):
+        t = list(tensors)
+        for i in weight_idx:
+            t[i] = tensors[i].clone()
+        sets.append(t)
+    return sets
+
+
+def timed(torch, lib, step, args, nsets=1):
     """ms per step over args.steps steps after args.warmup (eager launches, or - with --graph - replays of the step
-    captured into one HIP graph, which leaves the host's per-call work out), then a second eager pass with an event pair
-    around every kernel."""
+    captured into HIP graphs, one per input set, which leaves the host's per-call work out), then a second eager pass
+    with an event pair around every kernel."""
     eager = step
     if args.graph:
         side = torch.cuda.Stream()
@@ -125,12 +143,15 @@ def timed(torch, lib, step, args):
         with torch.cuda.stream(side):
             eager(0)
         torch.cuda.current_stream().wait_stream(side)
-        graph = torch.cuda.CUDAGraph()
-        with torch.cuda.graph(graph):
-            eager(0)
+        graphs = []
+        for i in range(nsets):
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph):
+                eager(i)
+            graphs.append(graph)
 
         def step(i):  # noqa: F811
-            graph.replay()
+            graphs[i % nsets].replay()
     for i in range(args.warmup):
         step(i)
     torch.cuda.synchronize()
@@ -260,10 +281,12 @@ def bench_indexer_prolog(args, torch, lib, dev):
                k_cache, k_scale_cache, torch.zeros((t, n), dtype=torch.float16, device=dev)]
     cfg, attrs = impl.IndexerPrologQuantConfigs(), impl.IndexerPrologQuantAttr()
 
-    def step(i):
-        impl.lightning_indexer_prolog_quant(*tensors, cfg, attrs)
+    sets = rotated(torch, tensors, (3, 5, 6), args)
 
-    ms, kernels = timed(torch, lib, step, args)
+    def step(i):
+        impl.lightning_indexer_prolog_quant(*sets[i % len(sets)], cfg, attrs)
+
+    ms, kernels = timed(torch, lib, step, args, len(sets))
     work = r * n * d + h * (d + n) * 2 + t * (h * 2 + r + n * 130 + n * 2 + 130)
     total_us = sum(kernels.values())
     print(json.dumps({
@@ -274,7 +297,8 @@ def bench_indexer_prolog(args, torch, lib, dev):
         "vs_baseline": round((t / (ms * 1e-3)) / (8 / 49e-6), 3) if published else None,
         "dtype": "int8+bf16", "data": "synthetic", "launch": "hip graph replay" if args.graph else "eager",
         "config": {"workload": f"lightning indexer prolog, {t} tokens, h 7168, q_lora_rank 1536, 64 x 128 index heads"
-                               + (", batch 4 x 2 tokens over a 64K-token paged cache (the reference's quoted case)" if published else "")},
+                               + (", batch 4 x 2 tokens over a 64K-token paged cache (the reference's quoted case)" if published else "")
+                               + f", weights rotated over {len(sets)} copies"},
         "roofline": {"kernel": "prolog (4 kernels)", "bound": "hbm", "achieved": round(work / total_us / 1e3, 1),
                      "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(work / total_us / 1e3 / HBM_PEAK_GBS, 4),
                      "traffic": None, "work_per_launch": work, "us_per_launch": round(total_us, 2),
@@ -310,10 +334,12 @@ def bench_mla_prolog(args, torch, lib, dev):
                torch.zeros((t, n, c), dtype=bf, device=dev), torch.zeros((t, n, 64), dtype=bf, device=dev), kv, kr, ks]
     cfg, rope = impl.MlaTileConfig(), impl.RopeTileShapeConfig([32, 64], [32, 32, 128], [16, 128, 128, 128])
 
-    def step(i):
-        impl.mla_prolog_quant_d(*tensors, 1e-5, 1e-5, "PA_BSND", cfg, rope)
+    sets = rotated(torch, tensors, (1, 2, 4, 5), args)
 
-    ms, kernels = timed(torch, lib, step, args)
+    def step(i):
+        impl.mla_prolog_quant_d(*sets[i % len(sets)], 1e-5, 1e-5, "PA_BSND", cfg, rope)
+
+    ms, kernels = timed(torch, lib, step, args, len(sets))
     # weights once, plus per token: x, q_norm + scale, q_nope, q_rope, the cache row
     work = h * r * 2 + r * n * 192 + n * 192 * 4 + n * 128 * c * 2 + h * (c + 64) * 2 + \
         t * (h * 2 + r + 4 + n * c * 2 + n * 64 * 2 + c + 16 + 128)
@@ -323,7 +349,7 @@ def bench_mla_prolog(args, torch, lib, dev):
         "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms, 4),
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "int8+bf16", "data": "synthetic", "launch": "hip graph replay" if args.graph else "eager",
         "config": {"workload": f"MLA prolog (int8 form), {t} tokens, h 7168, q_lora_rank 1536, 128 heads x 192, "
-                               f"kv_lora_rank 512"},
+                               f"kv_lora_rank 512, weights rotated over {len(sets)} copies"},
         "roofline": {"kernel": "mla prolog (4 kernels)", "bound": "hbm", "achieved": round(work / total_us / 1e3, 1),
                      "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(work / total_us / 1e3 / HBM_PEAK_GBS, 4),
                      "traffic": None, "work_per_launch": work, "us_per_launch": round(total_us, 2),
@@ -365,10 +391,12 @@ def bench_mla_indexer_prolog(args, torch, lib, dev):
     scal = (1e-5, 1e-5, "PA_BSND", impl.MlaTileConfig(), impl.IndexerPrologQuantAttr(), impl.IndexerPrologQuantConfigs(),
             impl.RopeTileShapeConfig([32, 64], [32, 32, 128], [16, 128, 128, 128]))
 
-    def step(i):
-        impl.mla_indexer_prolog_quant_d(*tensors, *scal)
+    sets = rotated(torch, tensors, (1, 2, 4, 5, 14, 16, 17), args)
 
-    ms, kernels = timed(torch, lib, step, args)
+    def step(i):
+        impl.mla_indexer_prolog_quant_d(*sets[i % len(sets)], *scal)
+
+    ms, kernels = timed(torch, lib, step, args, len(sets))
     work = h * r * 2 + r * n * 192 + n * 192 * 4 + n * 128 * c * 2 + h * (c + 64) * 2 + r * ni * d + h * (d + ni) * 2 + \
         t * (h * 2 + n * c * 2 + n * 64 * 2 + c + 16 + 128 + ni * 130 + ni * 2 + 130)
     total_us = sum(kernels.values())
@@ -377,7 +405,7 @@ def bench_mla_indexer_prolog(args, torch, lib, dev):
         "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms, 4),
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "int8+bf16", "data": "synthetic", "launch": "hip graph replay" if args.graph else "eager",
         "config": {"workload": f"fused MLA + lightning-indexer prolog, {t} tokens, h 7168, q_lora_rank 1536, 128 heads x 192, "
-                               f"kv_lora_rank 512, 64 x 128 index heads"},
+                               f"kv_lora_rank 512, 64 x 128 index heads, weights rotated over {len(sets)} copies"},
         "roofline": {"kernel": "fused prolog (4 kernels)", "bound": "hbm", "achieved": round(work / total_us / 1e3, 1),
                      "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(work / total_us / 1e3 / HBM_PEAK_GBS, 4),
                      "traffic": None, "work_per_launch": work, "us_per_launch": round(total_us, 2),
