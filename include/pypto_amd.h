@@ -207,6 +207,44 @@ uint64_t pto_indexer_prolog_workspace(const PtoTensorDesc* tensors, uint32_t n_t
 int pto_indexer_prolog_launch(const PtoTensorDesc* tensors, uint32_t n_tensors, const PtoIndexerPrologParams* params,
                               void* workspace, uint64_t workspace_bytes, void* hip_stream);
 
+/* Scalar argument of attention_pre_quant: the epsilon of its three RmsNorms, a constant 1e-5 inside the reference kernel
+ * (models/glm_v4_5/glm_attention_pre_quant.py:301). */
+typedef struct {
+    float eps;
+} PtoAttentionPreQuantParams;
+
+/*
+ * attention_pre_quant (models/glm_v4_5/glm_attention_pre_quant.py:633-747; kernel :235-505, argument checks :50-129):
+ * residual add + RmsNorm with bias, per-channel int8 quantisation, int8 QKV projection with int32 bias and per-output
+ * dequantisation, per-head RmsNorm with bias on the query and key heads, rotary embedding on each head's first
+ * 2 * half_rotary_dim dims.  tensors[19], in the order of the reference signature:
+ *    0 hidden_states                     [t, h]        BF16   (h a multiple of 256, at most 16384)
+ *    1 residual                          [t, h]        BF16
+ *    2 input_layernorm_weight            [h]           BF16
+ *    3 input_layernorm_bias              [h]           BF16
+ *    4 atten_qkv_input_scale_reciprocal  [h]           BF16   (multiplied onto the normalised row)
+ *    5 atten_qkv_input_offset            [h]           BF16   (added after the scale)
+ *    6 atten_qkv_weight                  [h, n_out]    INT8   (plain row-major; the reference's Ascend NZ tiling is a
+ *                                                              device format; n_out = q_size + 2 kv_size)
+ *    7 atten_qkv_quant_bias              [n_out]       INT32
+ *    8 atten_qkv_deq_scale               [n_out]       FP32
+ *    9 atten_q_norm_weight               [128]         BF16
+ *   10 atten_q_norm_bias                 [128]         BF16
+ *   11 atten_k_norm_weight               [128]         BF16
+ *   12 atten_k_norm_bias                 [128]         BF16
+ *   13 cos                               [t, 1, half]  BF16   (1 <= half <= 64)
+ *   14 sin                               [t, 1, half]  BF16
+ *   15 query                             [t, q_size]   BF16   (output; q_size a multiple of 128)
+ *   16 key                               [t, kv_size]  BF16   (output; kv_size a multiple of 128)
+ *   17 value                             [t, kv_size]  BF16   (output)
+ *   18 residual_res                      [t, h]        BF16   (output: hidden_states + residual)
+ */
+uint64_t pto_attention_pre_quant_workspace(const PtoTensorDesc* tensors, uint32_t n_tensors,
+                                           const PtoAttentionPreQuantParams* params);
+int pto_attention_pre_quant_launch(const PtoTensorDesc* tensors, uint32_t n_tensors,
+                                   const PtoAttentionPreQuantParams* params, void* workspace, uint64_t workspace_bytes,
+                                   void* hip_stream);
+
 /* Scalar arguments of mla_prolog_quant_d / mla_prolog_quant_p: the two RmsNorm epsilons and the cache mode
  * (models/deepseek_v32_exp/mla_prolog_quant_impl.py:866-871; tile_config and rope_cfg hold Ascend tiling knobs). */
 #define PTO_CACHE_PA_BSND 0 /* "PA_BSND": paged caches [block_num, block_size, 1, dim] */
@@ -287,9 +325,9 @@ const char* pto_last_error(void);
  * is bracketed by a HIP event pair recorded on the launch stream; pto_kernel_timing_read waits for the
  * events recorded so far for one kernel, returns their summed duration and count, and forgets them.
  * Kernel ids: 0 indexer_score_kernel, 1 indexer_topk_kernel, 2 sfa_decode_kernel, 3 sfa_combine_kernel,
- * 4 indexer_select_kernel, 5 select_experts_kernel, 6 gqa_decode_kernel, 7 gqa_combine_kernel, 8 unused,
- * 9 prolog_qx_kernel, 10 unused, 11 prolog_k_kernel, 12 mla_xa_kernel, 13 mla_norm_kernel (fused_norm_kernel in the fused
- * prolog), 14 mla_qb_kernel (fused_qb_kernel in the fused prolog), 15 mla_wuk_kernel
+ * 4 indexer_select_kernel, 5 select_experts_kernel, 6 gqa_decode_kernel, 7 gqa_combine_kernel, 8 apq_norm_kernel,
+ * 9 prolog_qx_kernel, 10 apq_gemm_kernel, 11 prolog_k_kernel, 12 mla_xa_kernel, 13 mla_norm_kernel (fused_norm_kernel in the fused
+ * prolog), 14 mla_qb_kernel (fused_qb_kernel in the fused prolog), 15 mla_wuk_kernel, 16 apq_head_kernel
  * (pto_kernel_name returns "" past the last id).
  * Off by default; not for use under graph capture.
  */

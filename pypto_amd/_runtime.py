@@ -63,6 +63,10 @@ class MlaIndexerPrologParams(ctypes.Structure):
                 ("indexer_eps", ctypes.c_float)]
 
 
+class AttentionPreQuantParams(ctypes.Structure):
+    _fields_ = [("eps", ctypes.c_float)]
+
+
 _OPS = {
     "sfa_quant": SfaParams,
     "sfa_antiquant": SfaParams,
@@ -72,6 +76,7 @@ _OPS = {
     "indexer_prolog": IndexerPrologParams,
     "mla_prolog_quant": MlaPrologParams,
     "mla_indexer_prolog_quant": MlaIndexerPrologParams,
+    "attention_pre_quant": AttentionPreQuantParams,
 }
 
 # C status -> Python exception type wrapped by FeError

@@ -257,6 +257,87 @@ int plan_indexer(const PtoTensorDesc* ts, uint32_t n, const PtoIndexerParams* p,
     return PTO_OK;
 }
 
+struct AttnPrePlan {
+    pto::AttnPreArgs args;
+    uint64_t ws_bytes;
+};
+
+int plan_attention_pre(const PtoTensorDesc* ts, uint32_t n, const PtoAttentionPreQuantParams* p, AttnPrePlan* plan)
+{
+    const char* op = "attention_pre_quant";
+    if (ts == nullptr || n != 19) return fail(PTO_ERR_ARG_COUNT, "%s: expected 19 tensors, got %u", op, n);
+    if (p == nullptr) return fail(PTO_ERR_PARAM, "%s: params is null", op);
+    if (!(p->eps >= 0.f)) return fail(PTO_ERR_PARAM, "%s: eps must be a non-negative number", op);
+    static const struct { const char* name; int dtype, rank; } spec[19] = {
+        {"hidden_states", PTO_DT_BF16, 2}, {"residual", PTO_DT_BF16, 2}, {"input_layernorm_weight", PTO_DT_BF16, 1},
+        {"input_layernorm_bias", PTO_DT_BF16, 1}, {"atten_qkv_input_scale_reciprocal", PTO_DT_BF16, 1},
+        {"atten_qkv_input_offset", PTO_DT_BF16, 1}, {"atten_qkv_weight", PTO_DT_INT8, 2},
+        {"atten_qkv_quant_bias", PTO_DT_INT32, 1}, {"atten_qkv_deq_scale", PTO_DT_FP32, 1},
+        {"atten_q_norm_weight", PTO_DT_BF16, 1}, {"atten_q_norm_bias", PTO_DT_BF16, 1},
+        {"atten_k_norm_weight", PTO_DT_BF16, 1}, {"atten_k_norm_bias", PTO_DT_BF16, 1}, {"cos", PTO_DT_BF16, 3},
+        {"sin", PTO_DT_BF16, 3}, {"query", PTO_DT_BF16, 2}, {"key", PTO_DT_BF16, 2}, {"value", PTO_DT_BF16, 2},
+        {"residual_res", PTO_DT_BF16, 2}};
+    int rc;
+    for (int i = 0; i < 19; ++i)
+        if ((rc = check_tensor(op, ts[i], spec[i].name, spec[i].dtype, spec[i].rank))) return rc;
+    const int64_t t = ts[0].shape[0], h = ts[0].shape[1], n_out = ts[6].shape[1], d = ts[9].shape[0];
+    const int64_t half = ts[13].shape[2], q_size = ts[15].shape[1], kv_size = ts[16].shape[1];
+    if (ts[1].shape[0] != t || ts[1].shape[1] != h || ts[18].shape[0] != t || ts[18].shape[1] != h)
+        return fail(PTO_ERR_SHAPE, "%s: residual and residual_res must be [%lld, %lld] like hidden_states", op, (long long)t, (long long)h);
+    for (int i = 2; i <= 5; ++i)
+        if (ts[i].shape[0] != h) return fail(PTO_ERR_SHAPE, "%s: %s must have %lld entries, got %lld", op, spec[i].name, (long long)h, (long long)ts[i].shape[0]);
+    if (ts[6].shape[0] != h) return fail(PTO_ERR_SHAPE, "%s: atten_qkv_weight must be [%lld, total_head_size], got %lld rows", op, (long long)h, (long long)ts[6].shape[0]);
+    if (ts[7].shape[0] != n_out || ts[8].shape[0] != n_out)
+        return fail(PTO_ERR_SHAPE, "%s: atten_qkv_quant_bias and atten_qkv_deq_scale must have %lld entries", op, (long long)n_out);
+    for (int i = 10; i <= 12; ++i)
+        if (ts[i].shape[0] != d) return fail(PTO_ERR_SHAPE, "%s: %s must have %lld entries like atten_q_norm_weight", op, spec[i].name, (long long)d);
+    if (!pto::attention_pre_supported(h, d, half))
+        return fail(PTO_ERR_SHAPE, "%s: need head size 128, hidden size a multiple of 256 up to 16384 and 1 <= half_rotary_dim <= 64; got head size %lld, hidden size %lld, half_rotary_dim %lld",
+                    op, (long long)d, (long long)h, (long long)half);
+    for (int i = 13; i <= 14; ++i)
+        if (ts[i].shape[0] != t || ts[i].shape[1] != 1 || ts[i].shape[2] != half)
+            return fail(PTO_ERR_SHAPE, "%s: %s must be [%lld, 1, %lld]", op, spec[i].name, (long long)t, (long long)half);
+    if (ts[15].shape[0] != t || ts[16].shape[0] != t || ts[17].shape[0] != t || ts[17].shape[1] != kv_size)
+        return fail(PTO_ERR_SHAPE, "%s: query, key and value must have %lld rows, key and value the same width", op, (long long)t);
+    if (q_size <= 0 || kv_size <= 0 || q_size % d != 0 || kv_size % d != 0 || q_size + 2 * kv_size != n_out)
+        return fail(PTO_ERR_SHAPE, "%s: query width %lld and key / value width %lld must be multiples of the head size adding up to total_head_size %lld",
+                    op, (long long)q_size, (long long)kv_size, (long long)n_out);
+    if (t > 65535 || n_out > (1 << 20)) return fail(PTO_ERR_SHAPE, "%s: problem too large", op);
+    pto::AttnPreArgs& a = plan->args;
+    a.x = static_cast<const uint16_t*>(ts[0].addr);
+    a.residual = static_cast<const uint16_t*>(ts[1].addr);
+    a.gamma = static_cast<const uint16_t*>(ts[2].addr);
+    a.bias = static_cast<const uint16_t*>(ts[3].addr);
+    a.in_scale = static_cast<const uint16_t*>(ts[4].addr);
+    a.in_offset = static_cast<const uint16_t*>(ts[5].addr);
+    a.w = static_cast<const int8_t*>(ts[6].addr);
+    a.qbias = static_cast<const int32_t*>(ts[7].addr);
+    a.deq = static_cast<const float*>(ts[8].addr);
+    a.q_gamma = static_cast<const uint16_t*>(ts[9].addr);
+    a.q_bias = static_cast<const uint16_t*>(ts[10].addr);
+    a.k_gamma = static_cast<const uint16_t*>(ts[11].addr);
+    a.k_bias = static_cast<const uint16_t*>(ts[12].addr);
+    a.cos = static_cast<const uint16_t*>(ts[13].addr);
+    a.sin = static_cast<const uint16_t*>(ts[14].addr);
+    a.q = static_cast<uint16_t*>(ts[15].addr);
+    a.k = static_cast<uint16_t*>(ts[16].addr);
+    a.v = static_cast<uint16_t*>(ts[17].addr);
+    a.residual_out = static_cast<uint16_t*>(ts[18].addr);
+    a.x_q = nullptr;
+    a.part = nullptr;
+    a.t = (int32_t)t;
+    a.h = (int32_t)h;
+    a.n_out = (int32_t)n_out;
+    a.q_heads = (int32_t)(q_size / d);
+    a.kv_heads = (int32_t)(kv_size / d);
+    a.half = (int32_t)half;
+    a.ksplits = (int32_t)(h / 256);
+    a.eps = p->eps;
+    a.mean_coff = (float)(1.0 / (double)h);
+    plan->ws_bytes = pto::attention_pre_workspace_bytes(t, h, n_out);
+    return PTO_OK;
+}
+
 int plan_select_experts(const PtoTensorDesc* ts, uint32_t n, const PtoSelectExpertsParams* p, pto::SelectExpertsArgs* a)
 {
     const char* op = "select_experts";
@@ -683,6 +764,31 @@ int pto_indexer_prolog_launch(const PtoTensorDesc* tensors, uint32_t n_tensors, 
     return PTO_OK;
 }
 
+uint64_t pto_attention_pre_quant_workspace(const PtoTensorDesc* tensors, uint32_t n_tensors,
+                                           const PtoAttentionPreQuantParams* params)
+{
+    AttnPrePlan plan;
+    return plan_attention_pre(tensors, n_tensors, params, &plan) == PTO_OK ? plan.ws_bytes : 0;
+}
+
+int pto_attention_pre_quant_launch(const PtoTensorDesc* tensors, uint32_t n_tensors,
+                                   const PtoAttentionPreQuantParams* params, void* workspace, uint64_t workspace_bytes,
+                                   void* hip_stream)
+{
+    const char* op = "attention_pre_quant";
+    AttnPrePlan plan;
+    int rc = plan_attention_pre(tensors, n_tensors, params, &plan);
+    if (rc) return rc;
+    if (plan.args.t == 0) return PTO_OK;
+    if (workspace == nullptr || workspace_bytes < plan.ws_bytes)
+        return fail(PTO_ERR_WORKSPACE, "%s: workspace of %llu bytes required, got %llu", op,
+                    (unsigned long long)plan.ws_bytes, (unsigned long long)(workspace ? workspace_bytes : 0));
+    pto::attention_pre_bind_workspace(plan.args, workspace);
+    hipError_t e = pto::attention_pre_launch(plan.args, static_cast<hipStream_t>(hip_stream));
+    if (e != hipSuccess) return fail(PTO_ERR_HIP, "%s: HIP launch failed: %s", op, hipGetErrorString(e));
+    return PTO_OK;
+}
+
 uint64_t pto_gqa_decode_workspace(const PtoTensorDesc* tensors, uint32_t n_tensors, const PtoGqaParams* params)
 {
     GqaPlan plan;
@@ -803,9 +909,9 @@ const char* pto_kernel_name(int kernel_id)
 {
     static const char* names[] = {"indexer_score_kernel", "indexer_topk_kernel", "sfa_decode_kernel",
                                   "sfa_combine_kernel", "indexer_select_kernel", "select_experts_kernel",
-                                  "gqa_decode_kernel", "gqa_combine_kernel", "unused", "prolog_qx_kernel", "unused",
+                                  "gqa_decode_kernel", "gqa_combine_kernel", "apq_norm_kernel", "prolog_qx_kernel", "apq_gemm_kernel",
                                   "prolog_k_kernel", "mla_xa_kernel", "mla_norm_kernel", "mla_qb_kernel",
-                                  "mla_wuk_kernel"};
+                                  "mla_wuk_kernel", "apq_head_kernel"};
     return kernel_id >= 0 && kernel_id < pto::KID_COUNT ? names[kernel_id] : "";
 }
 

@@ -169,4 +169,36 @@ bool fused_prolog_supported(int64_t n_idx);
 void fused_prolog_bind(MlaPrologArgs& m, PrologArgs& p, void* workspace);
 hipError_t fused_prolog_launch(const MlaPrologArgs& m, const PrologArgs& p, hipStream_t stream);
 
+// ---------------------------------------------------------------- GLM-4.5 attention_pre_quant
+struct AttnPreArgs {
+    const uint16_t* x;          // [t, h] bf16 hidden states
+    const uint16_t* residual;   // [t, h] bf16
+    const uint16_t* gamma;      // [h] bf16 input norm weight
+    const uint16_t* bias;       // [h] bf16 input norm bias
+    const uint16_t* in_scale;   // [h] bf16 quantisation scale (multiplied)
+    const uint16_t* in_offset;  // [h] bf16 quantisation offset (added)
+    const int8_t* w;            // [h, n_out] int8
+    const int32_t* qbias;       // [n_out]
+    const float* deq;           // [n_out]
+    const uint16_t* q_gamma;    // [128] bf16
+    const uint16_t* q_bias;
+    const uint16_t* k_gamma;
+    const uint16_t* k_bias;
+    const uint16_t* cos;        // [t, 1, half] bf16
+    const uint16_t* sin;
+    uint16_t* q;                // [t, q_heads * 128] bf16
+    uint16_t* k;                // [t, kv_heads * 128]
+    uint16_t* v;                // [t, kv_heads * 128]
+    uint16_t* residual_out;     // [t, h]
+    int8_t* x_q;                // workspace [t, h]: the quantised normalised rows
+    int32_t* part;              // workspace [ksplits, t, n_out]: int32 partial sums of the projection
+    int32_t t, h, n_out, q_heads, kv_heads, half, ksplits;
+    float eps, mean_coff;       // mean_coff = fp32(1 / h)
+};
+
+bool attention_pre_supported(int64_t h, int64_t d, int64_t half);
+uint64_t attention_pre_workspace_bytes(int64_t t, int64_t h, int64_t n_out);
+void attention_pre_bind_workspace(AttnPreArgs& a, void* workspace);
+hipError_t attention_pre_launch(const AttnPreArgs& a, hipStream_t stream);
+
 } // namespace pto

@@ -177,3 +177,42 @@ def test_missing_library_fails_loudly(monkeypatch, tmp_path):
     with pytest.raises(PyptoError) as e:
         _runtime.load_library()
     assert "python -m pypto_amd.build" in str(e.value)
+
+
+def apq_specs(t=8, h=5120, q=1536, kv=128, d=128, half=32):
+    n_out = q + 2 * kv
+    return [(BF16, (t, h)), (BF16, (t, h)), (BF16, (h,)), (BF16, (h,)), (BF16, (h,)), (BF16, (h,)), (INT8, (h, n_out)),
+            (INT32, (n_out,)), (FP32, (n_out,)), (BF16, (d,)), (BF16, (d,)), (BF16, (d,)), (BF16, (d,)),
+            (BF16, (t, 1, half)), (BF16, (t, 1, half)), (BF16, (t, q)), (BF16, (t, kv)), (BF16, (t, kv)), (BF16, (t, h))]
+
+
+def test_attention_pre_quant_validation_and_workspace(lib):
+    from pypto_amd._runtime import AttentionPreQuantParams
+    p = AttentionPreQuantParams(1e-5)
+    # the quantised rows (256-byte aligned) + one int32 partial sum per 256 rows of the contraction
+    assert lib.pto_attention_pre_quant_workspace(descs(apq_specs()), 19, ctypes.byref(p)) == 8 * 5120 + 20 * 8 * 1792 * 4
+    assert lib.pto_attention_pre_quant_workspace(descs(apq_specs(t=3, h=256, q=128)), 19, ctypes.byref(p)) == 768 + 3 * 384 * 4
+    rc, msg = launch_rc(lib, "attention_pre_quant", apq_specs(), p)
+    assert rc == -5 and "workspace" in msg
+    rc, msg = launch_rc(lib, "attention_pre_quant", apq_specs()[:18], p)
+    assert rc == -1 and "19 tensors" in msg
+    specs = apq_specs()
+    specs[6] = (BF16, specs[6][1])
+    rc, msg = launch_rc(lib, "attention_pre_quant", specs, p)
+    assert rc == -2 and "atten_qkv_weight must be int8" in msg
+    rc, msg = launch_rc(lib, "attention_pre_quant", apq_specs(h=5000), p)
+    assert rc == -3 and "multiple of 256" in msg
+    rc, msg = launch_rc(lib, "attention_pre_quant", apq_specs(d=64), p)
+    assert rc == -3
+    rc, msg = launch_rc(lib, "attention_pre_quant", apq_specs(half=65), p)
+    assert rc == -3 and "half_rotary_dim" in msg
+    specs = apq_specs()
+    specs[16] = (BF16, (8, 256))          # key wider than value; widths no longer add up
+    rc, msg = launch_rc(lib, "attention_pre_quant", specs, p)
+    assert rc == -3
+    specs = apq_specs()
+    specs[13] = (BF16, (8, 32))
+    rc, msg = launch_rc(lib, "attention_pre_quant", specs, p)
+    assert rc == -3 and "cos must have rank 3" in msg
+    assert launch_rc(lib, "attention_pre_quant", apq_specs(t=0), p)[0] == 0     # nothing to do, nothing launched
+    assert launch_rc(lib, "attention_pre_quant", apq_specs(), AttentionPreQuantParams(float("nan")))[0] == -4
