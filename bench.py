@@ -50,10 +50,13 @@ def parse():
     ap.add_argument("--cpu-seqs", type=int, default=8, help="sequences of the workload timed on the CPU oracle")
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--packed", action="store_true", help="use the packed 656-byte-row attention entry point")
-    ap.add_argument("--workload", choices=["v32", "gqa", "select_experts", "indexer_prolog", "mla_prolog", "mla_indexer_prolog", "decode_layer"], default="v32",
+    ap.add_argument("--workload", choices=["v32", "gqa", "select_experts", "indexer_prolog", "mla_prolog", "mla_indexer_prolog", "decode_layer", "attention_pre_quant"], default="v32",
                     help="v32 (default): the headline DeepSeek-V3.2 indexer + sparse attention decode step; gqa: GLM-4.5 "
                          "paged GQA decode (batch 64, 96/8 heads, contexts U[4096, 32768]); select_experts: GLM-4.5 "
-                         "router (8192 tokens x 160 experts)")
+                         "router (8192 tokens x 160 experts); attention_pre_quant: GLM-4.5 fused attention prolog")
+    ap.add_argument("--q-heads", type=int, default=12,
+                    help="attention_pre_quant: query heads on this device (12 = the reference test's share of GLM-4.5's "
+                         "96, with 1 key / value head; 96 = the whole model, 8 key / value heads)")
     ap.add_argument("--warm-weights", action="store_true",
                     help="prolog workloads: one copy of the weights, re-read every step (they then partly come out of "
                          "the 256 MB last-level cache); default: rotate enough copies to exceed it")
@@ -414,6 +417,58 @@ def bench_mla_indexer_prolog(args, torch, lib, dev):
     }))
 
 
+def bench_attention_pre_quant(args, torch, lib, dev):
+    """GLM-4.5 attention_pre_quant at decode size: `batch` tokens, hidden 5120, `q-heads` query heads and q-heads / 12
+    key / value heads of 128, rotary on 64 dims (the reference test's shape at 8 tokens and 12 heads:
+    models/glm_v4_5/glm_attention_pre_quant.py:510-519); zero-mean activations, a quantisation scale that spreads the
+    normalised row over the int8 range, weights uniform over int8."""
+    from pypto_amd.glm_v4_5 import glm_attention_pre_quant as impl
+    t, h, d, half = args.batch, 5120, 128, 32
+    qh = args.q_heads
+    kvh = max(qh // 12, 1)
+    n_out = (qh + 2 * kvh) * d
+    g = torch.Generator(device=dev).manual_seed(0)
+    bf = torch.bfloat16
+
+    def randn(*shape):
+        return torch.randn(shape, generator=g, device=dev)
+
+    def rand(*shape):
+        return torch.rand(shape, generator=g, device=dev)
+
+    ang = rand(t, 1, half) * 6.2831853
+    tensors = [randn(t, h).to(bf), randn(t, h).to(bf), (1 + 0.1 * randn(h)).to(bf), (0.05 * randn(h)).to(bf),
+               (30 + 10 * rand(h)).to(bf), torch.round(4 * randn(h)).to(bf),
+               torch.randint(-128, 128, (h, n_out), generator=g, device=dev, dtype=torch.int8),
+               torch.randint(-128, 128, (n_out,), generator=g, device=dev, dtype=torch.int32),
+               1e-4 * (0.5 + rand(n_out)), (1 + 0.1 * randn(d)).to(bf), (0.05 * randn(d)).to(bf),
+               (1 + 0.1 * randn(d)).to(bf), (0.05 * randn(d)).to(bf), torch.cos(ang).to(bf), torch.sin(ang).to(bf),
+               torch.zeros((t, qh * d), dtype=bf, device=dev), torch.zeros((t, kvh * d), dtype=bf, device=dev),
+               torch.zeros((t, kvh * d), dtype=bf, device=dev), torch.zeros((t, h), dtype=bf, device=dev)]
+    sets = rotated(torch, tensors, (6,), args)
+
+    def step(i):
+        impl.attention_pre_quant(*sets[i % len(sets)])
+
+    ms, kernels = timed(torch, lib, step, args, len(sets))
+    # read once: the weight, the two activation rows, the per-channel vectors; written: the four outputs
+    work = h * n_out + n_out * 8 + h * 8 + t * (h * 2 * 3 + n_out * 2 + half * 4)
+    total_us = sum(kernels.values())
+    print(json.dumps({
+        "metric": "prolog tokens/sec, GLM-4.5 attention_pre_quant decode", "value": round(t / (ms * 1e-3), 1),
+        "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms, 4),
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "int8+bf16", "data": "synthetic", "launch": "hip graph replay" if args.graph else "eager",
+        "config": {"workload": f"GLM-4.5 attention_pre_quant, {t} tokens, hidden 5120, {qh} + {kvh} + {kvh} heads of 128, "
+                               f"rotary 64, weights rotated over {len(sets)} copies"},
+        "roofline": {"kernel": "attention_pre_quant (3 kernels)", "bound": "hbm", "achieved": round(work / total_us / 1e3, 1),
+                     "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(work / total_us / 1e3 / HBM_PEAK_GBS, 4),
+                     "traffic": None, "work_per_launch": work, "us_per_launch": round(total_us, 2),
+                     "note": f"{h * n_out / 1e6:.1f} MB of weights read once: bound by launch and memory latency at decode sizes"},
+        "kernels": [{"kernel": k, "us": round(u, 2)} for k, u in kernels.items()], "cpu_baseline": None,
+    }))
+
+
 def bench_decode_layer(args, torch, lib, dev):
     """The attention front end of one DeepSeek-V3.2 decode layer as three chained calls on shared buffers: the fused MLA +
     indexer prolog writes the query tensors and the new cache rows (the last position of every sequence), the lightning
@@ -505,6 +560,8 @@ def main():
         return bench_mla_indexer_prolog(args, torch, lib, dev)
     if args.workload == "decode_layer":
         return bench_decode_layer(args, torch, lib, dev)
+    if args.workload == "attention_pre_quant":
+        return bench_attention_pre_quant(args, torch, lib, dev)
     b, ctx, s1 = args.batch, args.ctx, args.s1
     scale = 192 ** -0.5
     nbuf = 3

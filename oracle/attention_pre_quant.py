@@ -53,8 +53,9 @@ def quantize(x_norm, scale, offset):
 def quant_matmul(x_int8, weight, quant_bias, deq_scale):
     """:398-403 - exact int32 product, + int32 bias, -> fp32 (round to nearest even beyond 2^24), times the per-output
     scale, -> bf16."""
-    acc = torch.matmul(x_int8.to(torch.int32), weight.to(torch.int32)) + quant_bias.to(torch.int32)
-    return (acc.float() * deq_scale.float()).to(torch.bfloat16)
+    # the integer product through float64 BLAS: every partial sum is an integer below 2^53, so it is exact
+    acc = torch.matmul(x_int8.double(), weight.double()).to(torch.int64) + quant_bias.to(torch.int64)
+    return (acc.to(torch.int32).float() * deq_scale.float()).to(torch.bfloat16)
 
 
 def rope_half(x_rot, cos, sin):
@@ -73,21 +74,12 @@ def attention_pre_quant(inp, eps=EPS):
     """inp: the operator's input tensors by the names of the reference signature (:634-654) plus ``q_size`` and
     ``kv_size``.  Returns query [t, q_size], key [t, kv_size], value [t, kv_size], residual_res [t, h] (bf16) and the
     intermediate int8 row ``x_int8`` [t, h]."""
-    d = inp["atten_q_norm_weight"].shape[0]
-    half = inp["cos"].shape[-1]
-    q_size, kv_size = inp["q_size"], inp["kv_size"]
-    t = inp["hidden_states"].shape[0]
     x_norm, residual_res = add_rms_norm(inp["hidden_states"], inp["residual"], inp["input_layernorm_weight"],
                                         inp["input_layernorm_bias"], eps)
     x_int8 = quantize(x_norm, inp["atten_qkv_input_scale_reciprocal"], inp["atten_qkv_input_offset"])
-    mm = quant_matmul(x_int8, inp["atten_qkv_weight"], inp["atten_qkv_quant_bias"], inp["atten_qkv_deq_scale"])
-    q, k, v = mm.split([q_size, kv_size, kv_size], dim=-1)                                        # :410-425
-    q = rms_norm_bias(q.reshape(t, q_size // d, d), inp["atten_q_norm_weight"], inp["atten_q_norm_bias"], eps)
-    k = rms_norm_bias(k.reshape(t, kv_size // d, d), inp["atten_k_norm_weight"], inp["atten_k_norm_bias"], eps)
-    q = torch.cat((rope_half(q[..., :2 * half], inp["cos"], inp["sin"]), q[..., 2 * half:]), dim=-1)
-    k = torch.cat((rope_half(k[..., :2 * half], inp["cos"], inp["sin"]), k[..., 2 * half:]), dim=-1)
-    return {"query": q.reshape(t, q_size), "key": k.reshape(t, kv_size), "value": v.contiguous(),
-            "residual_res": residual_res, "x_int8": x_int8}
+    out = heads_from_x_int8(inp, x_int8, eps)
+    out.update(residual_res=residual_res, x_int8=x_int8)
+    return out
 
 
 def heads_from_x_int8(inp, x_int8, eps=EPS):
@@ -98,7 +90,7 @@ def heads_from_x_int8(inp, x_int8, eps=EPS):
     q_size, kv_size = inp["q_size"], inp["kv_size"]
     t = x_int8.shape[0]
     mm = quant_matmul(x_int8, inp["atten_qkv_weight"], inp["atten_qkv_quant_bias"], inp["atten_qkv_deq_scale"])
-    q, k, v = mm.split([q_size, kv_size, kv_size], dim=-1)
+    q, k, v = mm.split([q_size, kv_size, kv_size], dim=-1)                                        # :410-425
     q = rms_norm_bias(q.reshape(t, q_size // d, d), inp["atten_q_norm_weight"], inp["atten_q_norm_bias"], eps)
     k = rms_norm_bias(k.reshape(t, kv_size // d, d), inp["atten_k_norm_weight"], inp["atten_k_norm_bias"], eps)
     q = torch.cat((rope_half(q[..., :2 * half], inp["cos"], inp["sin"]), q[..., 2 * half:]), dim=-1)

@@ -331,7 +331,7 @@ int plan_attention_pre(const PtoTensorDesc* ts, uint32_t n, const PtoAttentionPr
     a.q_heads = (int32_t)(q_size / d);
     a.kv_heads = (int32_t)(kv_size / d);
     a.half = (int32_t)half;
-    a.ksplits = (int32_t)(h / 256);
+    a.ksplits = pto::attention_pre_ksplits(t, h, n_out);
     a.eps = p->eps;
     a.mean_coff = (float)(1.0 / (double)h);
     plan->ws_bytes = pto::attention_pre_workspace_bytes(t, h, n_out);

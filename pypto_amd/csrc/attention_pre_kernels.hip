@@ -14,7 +14,7 @@
 // At decode sizes (8 - 64 tokens) the operator reads 9 MB of int8 weights once (hidden 5120 x 1792 outputs) and is bound by
 // launch latency and that read; three launches:
 //   apq_norm_kernel   one workgroup per token: the row is read once and stays in registers across the sum
-//   apq_gemm_kernel   one workgroup per (128 outputs, 256 contraction rows, 32 tokens): the weight tile (output
+//   apq_gemm_kernel   one workgroup per (128 outputs, 256 to 1024 contraction rows, 32 tokens): the weight tile (output
 //                     dimension contiguous in memory) is loaded in one go, parked in LDS and read back with 8-bit
 //                     transposing reads as the A operand of the int8 MFMA; int32 partial sums to the workspace (exact,
 //                     so the split over the contraction changes nothing)
@@ -112,57 +112,74 @@ __global__ __launch_bounds__(256) void apq_norm_kernel(AttnPreArgs a)
 }
 
 // ------------------------------------------------------------------------------------------------ int8 projection
-// grid (n_out / 128, h / 256, token tiles of 32), 256 lanes: wave w owns outputs [32 w, 32 w + 32) of the tile
+// grid (n_out / 128, splits of the contraction, token tiles of 32), 256 lanes: wave w owns outputs [32 w, 32 w + 32) of
+// the tile.  A workgroup takes PER consecutive stages of 256 contraction rows (one where the grid would otherwise not
+// fill the chip, more where there are workgroups to spare: fewer partial sums to write and to add up); every load of all
+// its stages goes out before the first is used.
+template <int PER>
 __global__ __launch_bounds__(256) void apq_gemm_kernel(AttnPreArgs a)
 {
     __shared__ __align__(16) uint8_t wl[AK * AROW];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int l16 = lane & 15, g = lane >> 4;
     const int col0 = blockIdx.x * AD, split = blockIdx.y, tok0 = blockIdx.z * ATOK;
-    const int64_t kbase = (int64_t)split * AK;
+    const int stages = a.h / AK;
     // B operand (tokens): 16 contraction bytes per lane and MFMA, straight from the quantised rows
-    i32x4 qf[AK / 64][2];
+    i32x4 qf[PER][AK / 64][2];
 #pragma unroll
-    for (int ks = 0; ks < AK / 64; ++ks)
+    for (int j = 0; j < PER; ++j) {
+        const int64_t kbase = (int64_t)min(split * PER + j, stages - 1) * AK; // past the end: the last stage again, dropped below
 #pragma unroll
-        for (int tb = 0; tb < 2; ++tb)
-            qf[ks][tb] = *reinterpret_cast<const i32x4*>(a.x_q + (int64_t)min(tok0 + 16 * tb + l16, a.t - 1) * a.h + kbase +
-                                                         ks * 64 + 16 * g);
-    // the weight tile: 256 rows of 128 bytes, 16 bytes per lane and load
-    const int srow = tid >> 3, spc = tid & 7;
-    u32x4 stg[AK / 32];
+        for (int ks = 0; ks < AK / 64; ++ks)
 #pragma unroll
-    for (int i = 0; i < AK / 32; ++i)
-        stg[i] = *reinterpret_cast<const u32x4*>(a.w + (kbase + srow + 32 * i) * a.n_out + col0 + 16 * spc);
-#pragma unroll
-    for (int i = 0; i < AK / 32; ++i) {
-        u32x2* d = reinterpret_cast<u32x2*>(wl + (srow + 32 * i) * AROW + 16 * spc);
-        d[0] = u32x2{stg[i][0], stg[i][1]};
-        d[1] = u32x2{stg[i][2], stg[i][3]};
+            for (int tb = 0; tb < 2; ++tb)
+                qf[j][ks][tb] = *reinterpret_cast<const i32x4*>(a.x_q + (int64_t)min(tok0 + 16 * tb + l16, a.t - 1) * a.h +
+                                                                kbase + ks * 64 + 16 * g);
     }
-    __syncthreads();
+    // the weight tiles: 256 rows of 128 bytes per stage, 16 bytes per lane and load
+    const int srow = tid >> 3, spc = tid & 7;
+    u32x4 stg[PER][AK / 32];
+#pragma unroll
+    for (int j = 0; j < PER; ++j) {
+        const int64_t kbase = (int64_t)min(split * PER + j, stages - 1) * AK;
+#pragma unroll
+        for (int i = 0; i < AK / 32; ++i)
+            stg[j][i] = *reinterpret_cast<const u32x4*>(a.w + (kbase + srow + 32 * i) * a.n_out + col0 + 16 * spc);
+    }
     i32x4 acc[2][2];
 #pragma unroll
     for (int db = 0; db < 2; ++db)
 #pragma unroll
         for (int tb = 0; tb < 2; ++tb) acc[db][tb] = i32x4{0, 0, 0, 0};
 #pragma unroll
-    for (int ks = 0; ks < AK / 64; ++ks) {
-        // A operand: output 32 w + 16 db + l16, contraction bytes 16 g .. 16 g + 15 of the step.  An 8-bit transposing
-        // read hands lane i of a 16-lane group byte i % 8 of the chunks addressed by lanes i / 8, i / 8 + 2, ...: with
-        // lane i pointing at row i / 2, column half i % 2, lane i gets column i over rows 0 .. 7
-        i32x4 wf[2];
+    for (int j = 0; j < PER; ++j) {
+        if (j > 0) __syncthreads();
 #pragma unroll
-        for (int db = 0; db < 2; ++db) {
-            const uint8_t* p = wl + (ks * 64 + 16 * g + (l16 >> 1)) * AROW + 32 * wave + 16 * db + 8 * (l16 & 1);
-            const v2i lo = lds_read_tr8(p), hi = lds_read_tr8(p + 8 * AROW);
-            wf[db] = i32x4{lo[0], lo[1], hi[0], hi[1]};
+        for (int i = 0; i < AK / 32; ++i) {
+            u32x2* d = reinterpret_cast<u32x2*>(wl + (srow + 32 * i) * AROW + 16 * spc);
+            d[0] = u32x2{stg[j][i][0], stg[j][i][1]};
+            d[1] = u32x2{stg[j][i][2], stg[j][i][3]};
         }
+        __syncthreads();
+        if (split * PER + j >= stages) continue; // uniform over the workgroup
 #pragma unroll
-        for (int db = 0; db < 2; ++db)
+        for (int ks = 0; ks < AK / 64; ++ks) {
+            // A operand: output 32 w + 16 db + l16, contraction bytes 16 g .. 16 g + 15 of the step.  An 8-bit transposing
+            // read hands lane i of a 16-lane group byte i % 8 of the chunks addressed by lanes i / 8, i / 8 + 2, ...: with
+            // lane i pointing at row i / 2, column half i % 2, lane i gets column i over rows 0 .. 7
+            i32x4 wf[2];
 #pragma unroll
-            for (int tb = 0; tb < 2; ++tb)
-                acc[db][tb] = __builtin_amdgcn_mfma_i32_16x16x64_i8(wf[db], qf[ks][tb], acc[db][tb], 0, 0, 0);
+            for (int db = 0; db < 2; ++db) {
+                const uint8_t* p = wl + (ks * 64 + 16 * g + (l16 >> 1)) * AROW + 32 * wave + 16 * db + 8 * (l16 & 1);
+                const v2i lo = lds_read_tr8(p), hi = lds_read_tr8(p + 8 * AROW);
+                wf[db] = i32x4{lo[0], lo[1], hi[0], hi[1]};
+            }
+#pragma unroll
+            for (int db = 0; db < 2; ++db)
+#pragma unroll
+                for (int tb = 0; tb < 2; ++tb)
+                    acc[db][tb] = __builtin_amdgcn_mfma_i32_16x16x64_i8(wf[db], qf[j][ks][tb], acc[db][tb], 0, 0, 0);
+        }
     }
     // register e of acc[db][tb]: output 32 w + 16 db + 4 g + e, token 16 tb + l16
 #pragma unroll
@@ -232,9 +249,22 @@ bool attention_pre_supported(int64_t h, int64_t d, int64_t half)
 
 static uint64_t align256(uint64_t v) { return (v + 255) & ~(uint64_t)255; }
 
+// stages of 256 contraction rows per workgroup of the projection: as many (1, 2 or 4) as still leave 448 workgroups
+static int stages_per_split(int64_t t, int64_t h, int64_t n_out)
+{
+    const int64_t wgs = (n_out / AD) * (h / AK) * ((t + ATOK - 1) / ATOK);
+    return wgs >= 8 * 448 ? 4 : wgs >= 2 * 448 ? 2 : 1;
+}
+
+int attention_pre_ksplits(int64_t t, int64_t h, int64_t n_out)
+{
+    const int per = stages_per_split(t, h, n_out);
+    return (int)((h / AK + per - 1) / per);
+}
+
 uint64_t attention_pre_workspace_bytes(int64_t t, int64_t h, int64_t n_out)
 {
-    return align256((uint64_t)t * h) + (uint64_t)(h / AK) * t * n_out * sizeof(int32_t);
+    return align256((uint64_t)t * h) + (uint64_t)attention_pre_ksplits(t, h, n_out) * t * n_out * sizeof(int32_t);
 }
 
 void attention_pre_bind_workspace(AttnPreArgs& a, void* ws)
@@ -257,7 +287,15 @@ hipError_t attention_pre_launch(const AttnPreArgs& a, hipStream_t stream)
     if ((e = hipGetLastError()) != hipSuccess) return e;
     {
         ScopedKernelTimer tm(KID_APQ_GEMM, stream);
-        hipLaunchKernelGGL(apq_gemm_kernel, dim3(a.n_out / AD, a.ksplits, (a.t + ATOK - 1) / ATOK), dim3(256), 0, stream, a);
+        const dim3 grid(a.n_out / AD, a.ksplits, (a.t + ATOK - 1) / ATOK);
+        const int per = stages_per_split(a.t, a.h, a.n_out);
+        if (a.ksplits != attention_pre_ksplits(a.t, a.h, a.n_out)) return hipErrorInvalidValue;
+        if (per == 4)
+            hipLaunchKernelGGL(apq_gemm_kernel<4>, grid, dim3(256), 0, stream, a);
+        else if (per == 2)
+            hipLaunchKernelGGL(apq_gemm_kernel<2>, grid, dim3(256), 0, stream, a);
+        else
+            hipLaunchKernelGGL(apq_gemm_kernel<1>, grid, dim3(256), 0, stream, a);
     }
     if ((e = hipGetLastError()) != hipSuccess) return e;
     {

@@ -197,6 +197,7 @@ struct AttnPreArgs {
 };
 
 bool attention_pre_supported(int64_t h, int64_t d, int64_t half);
+int attention_pre_ksplits(int64_t t, int64_t h, int64_t n_out); // partial sums per output of the projection
 uint64_t attention_pre_workspace_bytes(int64_t t, int64_t h, int64_t n_out);
 void attention_pre_bind_workspace(AttnPreArgs& a, void* workspace);
 hipError_t attention_pre_launch(const AttnPreArgs& a, hipStream_t stream);

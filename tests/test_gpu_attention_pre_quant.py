@@ -88,6 +88,14 @@ def test_hidden_sizes_and_rotary_widths(cuda, h, half):
     check(case, run(case, cuda))
 
 
+@pytest.mark.parametrize("t,q_heads,kv_heads", [(8, 30, 3), (40, 60, 6)])
+def test_several_stages_per_workgroup_with_a_short_last_split(cuda, t, q_heads, kv_heads):
+    """Shapes with enough workgroups for the projection kernel to take two (first case) or four (second) stages of 256
+    contraction rows per workgroup; hidden 6400 = 25 stages leaves the last split with a single one."""
+    case = op.make_case(t, h=6400, q_heads=q_heads, kv_heads=kv_heads, seed=t + q_heads)
+    check(case, run(case, cuda))
+
+
 def test_saturation_at_both_ends(cuda):
     """A quantisation scale of 1000: nine in ten values of the quantised row are clamped at -128 or 127."""
     case = op.make_case(4, h=4096, q_heads=2, kv_heads=1, seed=14)
