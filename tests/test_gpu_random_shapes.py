@@ -63,3 +63,23 @@ def test_attention_random_shapes(cuda, seed):
                 f"entry={entry} dist={dist}")
         case = osfa.make_case(b, nq, s1, act, topk=topk, block_size=bs, seed=1000 * seed + i, quant=quant, dist=dist)
         check(run_sfa(case, cuda, entry=entry, packed=packed), sfa_golden(case), name)
+
+
+@pytest.mark.parametrize("seed", [404, 505])
+def test_attention_pre_quant_random_shapes(cuda, seed):
+    """GLM-4.5 attention_pre_quant: token counts around the 32-token tile, hidden sizes on both sides of the two norm
+    kernels and with short last splits of the contraction, head counts that put the projection kernel at one, two and
+    four stages per workgroup, every rotary width, both input distributions."""
+    from oracle import attention_pre_quant as oapq
+    from test_gpu_attention_pre_quant import check as check_apq
+    from test_gpu_attention_pre_quant import run as run_apq
+    rng = random.Random(seed)
+    for i in range(12):
+        t = rng.choice([1, 2, 7, 8, 31, 32, 33, 63, 64, 65, rng.randint(1, 130)])
+        h = 256 * rng.choice([1, 2, 3, 7, 20, 24, 25, 28, 33, 64])
+        kv = rng.choice([1, 1, 2, 4])
+        qh = kv * rng.choice([1, 2, 6, 12])
+        half = rng.choice([1, 2, 7, 16, 32, 32, 33, 64])
+        case = oapq.make_case(t, h=h, q_heads=qh, kv_heads=kv, half=half, seed=seed + i, realistic=rng.random() < 0.8)
+        print(f"attention_pre_quant case {i}: t {t} h {h} heads {qh}+{kv}+{kv} half {half}", flush=True)
+        check_apq(case, run_apq(case, cuda))
