@@ -3,7 +3,28 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include <atomic>
+
 namespace pto {
+
+// Host side: set-up that has to happen once on every device the library launches on (a kernel's attributes belong to
+// the device its code object is loaded on).  f must be idempotent: two threads that arrive together both run it.
+class DeviceOnce {
+    std::atomic<uint64_t> done_{0}; // one bit per device ordinal
+public:
+    template <class F>
+    hipError_t run(F&& f)
+    {
+        int dev = 0;
+        hipError_t e = hipGetDevice(&dev);
+        if (e != hipSuccess) return e;
+        const uint64_t bit = 1ull << (dev & 63);
+        if (done_.load(std::memory_order_acquire) & bit) return hipSuccess;
+        if ((e = f()) != hipSuccess) return e;
+        done_.fetch_or(bit, std::memory_order_release);
+        return hipSuccess;
+    }
+};
 
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));

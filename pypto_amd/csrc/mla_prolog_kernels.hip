@@ -625,22 +625,21 @@ void fused_prolog_bind(MlaPrologArgs& m, PrologArgs& p, void* ws)
 
 static hipError_t set_lds_limits()
 {
-    static bool done = false;
-    if (done) return hipSuccess;
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(mla_xa_kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
-                                       4 * XA_K * XROW2);
-    if (e != hipSuccess) return e;
-    e = hipFuncSetAttribute(reinterpret_cast<const void*>(mla_qb_kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
-                            mla_qb_lds_bytes(MAX_R));
-    if (e != hipSuccess) return e;
-    e = hipFuncSetAttribute(reinterpret_cast<const void*>(mla_qb16_kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
-                            4 * XA_K * XROW2);
-    if (e != hipSuccess) return e;
-    e = hipFuncSetAttribute(reinterpret_cast<const void*>(fused_qb_kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
-                            mla_qb_lds_bytes(MAX_R) > prolog_q_lds_bytes(QMAX_R) ? mla_qb_lds_bytes(MAX_R) : prolog_q_lds_bytes(QMAX_R));
-    if (e != hipSuccess) return e;
-    done = true;
-    return hipSuccess;
+    static DeviceOnce once;
+    return once.run([] {
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(mla_xa_kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                           4 * XA_K * XROW2);
+        if (e != hipSuccess) return e;
+        e = hipFuncSetAttribute(reinterpret_cast<const void*>(mla_qb_kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                mla_qb_lds_bytes(MAX_R));
+        if (e != hipSuccess) return e;
+        e = hipFuncSetAttribute(reinterpret_cast<const void*>(mla_qb16_kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                4 * XA_K * XROW2);
+        if (e != hipSuccess) return e;
+        e = hipFuncSetAttribute(reinterpret_cast<const void*>(fused_qb_kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                mla_qb_lds_bytes(MAX_R) > prolog_q_lds_bytes(QMAX_R) ? mla_qb_lds_bytes(MAX_R) : prolog_q_lds_bytes(QMAX_R));
+        return e;
+    });
 }
 
 // p == nullptr: the MLA prolog on its own; otherwise the fused operator (m and p bound by fused_prolog_bind)

@@ -139,14 +139,13 @@ hipError_t prolog_launch(const PrologArgs& a, hipStream_t stream)
     if (a.t == 0) return hipSuccess;
     const int ttiles = (a.t + PTOK - 1) / PTOK;
     hipError_t e;
-    static bool attr_done = false;
+    static DeviceOnce attr_done;
     constexpr int xw_lds_max = XW_K * (PD + 128) * 2;
-    if (!attr_done) {
-        e = hipFuncSetAttribute(reinterpret_cast<const void*>(prolog_qx_kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
-                                prolog_q_lds_bytes(QMAX_R) > xw_lds_max ? prolog_q_lds_bytes(QMAX_R) : xw_lds_max);
-        if (e != hipSuccess) return e;
-        attr_done = true;
-    }
+    e = attr_done.run([] {
+        return hipFuncSetAttribute(reinterpret_cast<const void*>(prolog_qx_kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                   prolog_q_lds_bytes(QMAX_R) > xw_lds_max ? prolog_q_lds_bytes(QMAX_R) : xw_lds_max);
+    });
+    if (e != hipSuccess) return e;
     {
         const int xw_lds = XW_K * (PD + a.n) * 2;
         const int smem = prolog_q_lds_bytes(a.r) > xw_lds ? prolog_q_lds_bytes(a.r) : xw_lds;

@@ -535,15 +535,15 @@ __global__ __launch_bounds__(128) void sfa_combine_kernel(const void* __restrict
 
 int num_cus()
 {
-    static int cached = 0;
-    if (cached == 0) {
-        int dev = 0, n = 0;
-        if (hipGetDevice(&dev) != hipSuccess ||
-            hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0)
-            n = 256;
-        cached = n;
+    static std::atomic<int> cached[64]; // per device ordinal; 0 = not asked yet
+    int dev = 0, n = 0;
+    if (hipGetDevice(&dev) != hipSuccess) return 256;
+    n = cached[dev & 63].load(std::memory_order_relaxed);
+    if (n == 0) {
+        if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) n = 256;
+        cached[dev & 63].store(n, std::memory_order_relaxed);
     }
-    return cached;
+    return n;
 }
 
 } // namespace
@@ -582,13 +582,14 @@ hipError_t sfa_launch(const SfaArgs& a, hipStream_t stream)
     args.bt_cached = smem_bytes + a.bt_stride * 4 <= LDS_LIMIT ? 1 : 0;
     if (args.bt_cached) smem_bytes += a.bt_stride * 4;
     if (smem_bytes < HEADS_PER_WG * OUT_ROW) smem_bytes = HEADS_PER_WG * OUT_ROW; // epilogue staging
-    static bool attr_done[2] = {false, false};
+    static DeviceOnce attr_done[2];
     auto kern = a.quant ? sfa_decode_kernel<true> : sfa_decode_kernel<false>;
-    if (!attr_done[a.quant]) {
-        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
-                                           hipFuncAttributeMaxDynamicSharedMemorySize, LDS_LIMIT);
+    {
+        hipError_t e = attr_done[a.quant].run([&] {
+            return hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                       LDS_LIMIT);
+        });
         if (e != hipSuccess) return e;
-        attr_done[a.quant] = true;
     }
     const int hgroups = (a.nq + HEADS_PER_WG - 1) / HEADS_PER_WG;
     dim3 grid(a.nsplit, t, hgroups);

@@ -1,12 +1,13 @@
 #include "timing.h"
 
+#include <atomic>
 #include <mutex>
 #include <utility>
 #include <vector>
 
 namespace pto {
 namespace {
-bool g_on = false;
+std::atomic<bool> g_on{false};
 std::mutex g_mu;
 std::vector<std::pair<hipEvent_t, hipEvent_t>> g_recs[KID_COUNT];
 hipEvent_t g_open[KID_COUNT];
