@@ -24,6 +24,8 @@
 //                    through LDS; dequantisation and the query's rotary embedding in registers
 //   mla_wuk_kernel   per (head, 128 outputs): q_b[:, head, :128] @ w_uk[head]
 #include <hip/hip_runtime.h>
+
+#include <algorithm>
 #include <stdint.h>
 
 #include "common.h"
@@ -544,35 +546,73 @@ __global__ __launch_bounds__(1024) void fused_qb_kernel(MlaPrologArgs m, PrologA
 }
 
 // ------------------------------------------------------------------------------------------------ q_b[:, head, :128] @ w_uk[head]
-// grid (heads, 512 / 128, token tiles of 32), 256 lanes: wave w owns outputs [32 w, 32 w + 32) of the tile
+// grid (heads, 512 / 128, z), 256 lanes: wave w owns outputs [32 w, 32 w + 32) of the tile.  The head's 128 x 128 weight
+// tile stays in LDS while the workgroup walks the token tiles z, z + gridDim.z, ... (one at decode sizes; at prefill
+// sizes the weights are then read once per workgroup instead of once per 32 tokens); the next tile's operand rows are
+// requested before the current tile's products.
 __global__ __launch_bounds__(256) void mla_wuk_kernel(MlaPrologArgs a)
 {
+    constexpr int OROW = 128 * 2 + 16; // bytes per LDS row of the 32 x 128 bf16 output tile (padded)
     __shared__ __align__(16) uint8_t wl[MNOPE * TROW];
+    __shared__ __align__(16) uint8_t bt[MTOK * OROW]; // the token tile's operand rows
+    __shared__ __align__(16) uint8_t ot[MTOK * OROW]; // its outputs
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int l32 = lane & 31, hl = lane >> 5;
-    const int head = blockIdx.x, ct = blockIdx.y, tok0 = blockIdx.z * MTOK;
+    const int head = blockIdx.x, ct = blockIdx.y;
+    const int ttiles = (a.t + MTOK - 1) / MTOK;
     const uint16_t* src = a.w_uk + (int64_t)head * MNOPE * MC + ct * 128;
-    const int gt = tok0 + l32;
-    u32x4 bx[MNOPE / 16];
-    load_b_rows<MNOPE / 16>(bx, a.qb_nope + ((int64_t)min(gt, a.t - 1) * a.n + head) * MNOPE, lane);
+    // a tile's operand rows: 32 tokens x 256 bytes, fetched once by the workgroup in 16-byte pieces (16 lanes per row) and
+    // handed to the waves through LDS - a wave loading its own operand would fetch a different row with every lane pair,
+    // which costs the texture addresser a cycle per row and instruction, four times over for the four waves
+    const int prow = tid >> 4, pcol = tid & 15;
+    auto fetch = [&](u32x4 (&q)[2], int tt) {
+#pragma unroll
+        for (int i = 0; i < 2; ++i)
+            q[i] = *reinterpret_cast<const u32x4*>(a.qb_nope + ((int64_t)min(tt * MTOK + prow + 16 * i, a.t - 1) * a.n + head) * MNOPE +
+                                                   8 * pcol);
+    };
+    auto park = [&](const u32x4 (&q)[2]) {
+#pragma unroll
+        for (int i = 0; i < 2; ++i) *reinterpret_cast<u32x4*>(bt + (prow + 16 * i) * OROW + 16 * pcol) = q[i];
+    };
+    u32x4 q0[2];
+    fetch(q0, blockIdx.z);
 #pragma unroll
     for (int i = tid; i < MNOPE * 16; i += 256) {
         const int k = i >> 4, c = i & 15;
         *reinterpret_cast<u32x4*>(wl + k * TROW + c * 16) = *reinterpret_cast<const u32x4*>(src + (int64_t)k * MC + c * 8);
     }
+    park(q0);
     __syncthreads();
-    f32x16 acc;
+    for (int tt = blockIdx.z; tt < ttiles; tt += gridDim.z) {
+        // the rows of the tile after this one, if there is one (uniform over the workgroup)
+        const bool more = tt + (int)gridDim.z < ttiles;
+        u32x4 qn[2];
+        if (more) fetch(qn, tt + gridDim.z);
+        u32x4 bx[MNOPE / 16];
 #pragma unroll
-    for (int e = 0; e < 16; ++e) acc[e] = 0.f;
-    gemm_tr_tile<MNOPE / 16, TROW>(acc, wl, 32 * wave, bx, lane);
-    if (gt < a.t) {
-        uint16_t* out = a.q_nope + ((int64_t)gt * a.n + head) * MC + ct * 128 + 32 * wave + 4 * hl;
+        for (int ks = 0; ks < MNOPE / 16; ++ks) bx[ks] = *reinterpret_cast<const u32x4*>(bt + l32 * OROW + (ks * 16 + 8 * hl) * 2);
+        f32x16 acc;
+#pragma unroll
+        for (int e = 0; e < 16; ++e) acc[e] = 0.f;
+        gemm_tr_tile<MNOPE / 16, TROW>(acc, wl, 32 * wave, bx, lane);
+        // through LDS, so that a token's 128 outputs leave as one 256-byte run (16 lanes x 16 bytes)
 #pragma unroll
         for (int e4 = 0; e4 < 4; ++e4) {
             const u32x2 pk = {(uint32_t)f32_to_bf16(acc[4 * e4]) | ((uint32_t)f32_to_bf16(acc[4 * e4 + 1]) << 16),
                               (uint32_t)f32_to_bf16(acc[4 * e4 + 2]) | ((uint32_t)f32_to_bf16(acc[4 * e4 + 3]) << 16)};
-            *reinterpret_cast<u32x2*>(out + 8 * e4) = pk;
+            *reinterpret_cast<u32x2*>(ot + l32 * OROW + (32 * wave + 8 * e4 + 4 * hl) * 2) = pk;
         }
+        __syncthreads(); // outputs parked; every wave is done with the operand rows
+#pragma unroll
+        for (int i = 0; i < 2; ++i) {
+            const int tok = prow + 16 * i;
+            if (tt * MTOK + tok < a.t)
+                *reinterpret_cast<u32x4*>(a.q_nope + ((int64_t)(tt * MTOK + tok) * a.n + head) * MC + ct * 128 + 8 * pcol) =
+                    *reinterpret_cast<const u32x4*>(ot + tok * OROW + 16 * pcol);
+        }
+        if (more) park(qn);
+        __syncthreads();
     }
 }
 
@@ -679,7 +719,9 @@ static hipError_t launch_prologs(const MlaPrologArgs& a, const PrologArgs* p, hi
     if ((e = hipGetLastError()) != hipSuccess) return e;
     {
         ScopedKernelTimer tm(KID_MLA_WUK, stream);
-        hipLaunchKernelGGL(mla_wuk_kernel, dim3(a.n, MC / 128, ttiles), dim3(256), 0, stream, a);
+        // token tiles per workgroup: one while that leaves the grid at about a thousand workgroups or fewer, more beyond
+        const int zdim = std::min(ttiles, std::max(1, 1024 / (a.n * (MC / 128))));
+        hipLaunchKernelGGL(mla_wuk_kernel, dim3(a.n, MC / 128, zdim), dim3(256), 0, stream, a);
     }
     return hipGetLastError();
 }
