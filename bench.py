@@ -50,7 +50,7 @@ def parse():
     ap.add_argument("--cpu-seqs", type=int, default=8, help="sequences of the workload timed on the CPU oracle")
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--packed", action="store_true", help="use the packed 656-byte-row attention entry point")
-    ap.add_argument("--workload", choices=["v32", "gqa", "select_experts", "indexer_prolog", "mla_prolog", "mla_indexer_prolog", "decode_layer", "attention_pre_quant"], default="v32",
+    ap.add_argument("--workload", choices=["v32", "gqa", "select_experts", "indexer_prolog", "mla_prolog", "mla_indexer_prolog", "decode_layer", "attention_pre_quant", "sfa_prefill"], default="v32",
                     help="v32 (default): the headline DeepSeek-V3.2 indexer + sparse attention decode step; gqa: GLM-4.5 "
                          "paged GQA decode (batch 64, 96/8 heads, contexts U[4096, 32768]); select_experts: GLM-4.5 "
                          "router (8192 tokens x 160 experts); attention_pre_quant: GLM-4.5 fused attention prolog")
@@ -469,6 +469,40 @@ def bench_attention_pre_quant(args, torch, lib, dev):
     }))
 
 
+def bench_sfa_prefill(args, torch, lib, dev):
+    """The prefill entry of sparse flash attention at the reference's prefill case (sfa_bf16_b1_s256_seq64K_int8_p,
+    models/deepseek_v32_exp/deepseekv32_sparse_flash_attention_quant.py:498): one sequence of `ctx` cached tokens, 256
+    query tokens (`--s1`), 128 heads, every query token with its own 2048 selected rows (random, distinct)."""
+    from pypto_amd.deepseek_v32_exp.sparse_flash_attention_quant_impl import SaTileShapeConfig, sparse_flash_attention_quant_p
+    s1 = args.s1 if args.s1 > 1 else 256
+    w = make_workload(torch, dev, 1, args.ctx, s1, 1)
+    g = torch.Generator(device=dev).manual_seed(1)
+    topk = torch.stack([torch.randperm(args.ctx, generator=g, device=dev)[:2048] for _ in range(s1)]).to(torch.int32).contiguous()
+    c = w["sets"][0]
+    cfg = SaTileShapeConfig()
+    scale = 192 ** -0.5
+
+    def step(i):
+        sparse_flash_attention_quant_p(w["q_nope"], w["q_rope"], c["kn"], c["kr"], c["ks"], topk, w["table"], w["act"],
+                                       w["out"], 128, 1, scale, 2048, 128, w["pages_per_seq"], cfg)
+
+    ms, kernels = timed(torch, lib, step, args)
+    flops = s1 * 2048 * 128 * (2 * 576 + 2 * 512)
+    us = kernels.get("sfa_decode_kernel", 0.0)
+    print(json.dumps({
+        "metric": "prefill query tokens/sec, V3.2 sparse flash attention", "value": round(s1 / (ms * 1e-3), 1), "unit": "tokens/s",
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms, 4), "higher_is_better": True,
+        "scaling": "weak", "vs_baseline": None, "dtype": "int8+bf16", "data": "synthetic",
+        "launch": "hip graph replay" if args.graph else "eager",
+        "config": {"workload": f"sparse flash attention, prefill entry, 1 sequence of {args.ctx} cached tokens, {s1} query tokens, "
+                               f"128 heads, top-2048 per query token, int8 paged MLA cache"},
+        "roofline": {"kernel": "sfa_decode_kernel", "bound": "mfma", "achieved": round(flops / us / 1e6, 1) if us else None,
+                     "peak": 2500.0, "unit": "TFLOP/s", "frac": round(flops / us / 1e6 / 2500.0, 4) if us else None,
+                     "traffic": None, "work_per_launch": flops, "us_per_launch": round(us, 2)},
+        "kernels": [{"kernel": k, "us": round(u, 2)} for k, u in kernels.items()], "cpu_baseline": None,
+    }))
+
+
 def bench_decode_layer(args, torch, lib, dev):
     """The attention front end of one DeepSeek-V3.2 decode layer as three chained calls on shared buffers: the fused MLA +
     indexer prolog writes the query tensors and the new cache rows (the last position of every sequence), the lightning
@@ -562,6 +596,8 @@ def main():
         return bench_decode_layer(args, torch, lib, dev)
     if args.workload == "attention_pre_quant":
         return bench_attention_pre_quant(args, torch, lib, dev)
+    if args.workload == "sfa_prefill":
+        return bench_sfa_prefill(args, torch, lib, dev)
     b, ctx, s1 = args.batch, args.ctx, args.s1
     scale = 192 ** -0.5
     nbuf = 3
