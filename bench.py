@@ -736,14 +736,20 @@ def time_cpu_oracle(torch, w, n_seq, scale):
     idx_q, idx_qs, idx_w = w["idx_q"][:t].cpu(), w["idx_qs"][:t].cpu(), w["idx_w"][:t].cpu()
     q = torch.cat([w["q_nope"][:t * 128].cpu().reshape(n_seq, s1, 128, 512),
                    w["q_rope"][:t * 128].cpu().reshape(n_seq, s1, 128, 64)], dim=-1)
-    t0 = time.perf_counter()
-    tk = oi.lightning_indexer(idx_q, idx_qs, host["idx_k"], host["idx_ks"], idx_w, act, table, s1, 2048)
-    out = osfa.attention_no_flash(q, host["kn"], host["kr"], host["ks"], tk.reshape(t, 2048), table, act, 128, scale,
-                                  2048)
+    def one_pass():
+        tk = oi.lightning_indexer(idx_q, idx_qs, host["idx_k"], host["idx_ks"], idx_w, act, table, s1, 2048)
+        return osfa.attention_no_flash(q, host["kn"], host["kr"], host["ks"], tk.reshape(t, 2048), table, act, 128, scale,
+                                       2048)
+
+    one_pass()  # untimed: first touch of the host copies, thread pool start-up
+    passes, t0 = 0, time.perf_counter()
+    while passes < 3 or time.perf_counter() - t0 < 10.0:
+        one_pass()
+        passes += 1
     dt = time.perf_counter() - t0
-    return {"value": round(t / dt, 2), "unit": "tokens/s", "cores": torch.get_num_threads(), "kind": "port",
-            "sample": f"first {n_seq} of the {w['b']} sequences of the same workload, one pass "
-                      f"({dt:.2f} s): oracle.indexer.lightning_indexer + oracle.sfa.attention_no_flash",
+    return {"value": round(passes * t / dt, 2), "unit": "tokens/s", "cores": torch.get_num_threads(), "kind": "port",
+            "sample": f"first {n_seq} of the {w['b']} sequences of the same workload, {passes} passes after an untimed one "
+                      f"({dt:.1f} s): oracle.indexer.lightning_indexer + oracle.sfa.attention_no_flash",
             "host_cpus": os.cpu_count()}
 
 
