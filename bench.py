@@ -50,7 +50,7 @@ def parse():
     ap.add_argument("--cpu-seqs", type=int, default=8, help="sequences of the workload timed on the CPU oracle")
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--packed", action="store_true", help="use the packed 656-byte-row attention entry point")
-    ap.add_argument("--workload", choices=["v32", "gqa", "select_experts", "indexer_prolog", "mla_prolog", "mla_indexer_prolog", "decode_layer", "attention_pre_quant", "sfa_prefill"], default="v32",
+    ap.add_argument("--workload", choices=["v32", "gqa", "select_experts", "indexer_prolog", "mla_prolog", "mla_indexer_prolog", "decode_layer", "attention_pre_quant", "sfa_prefill", "paged_gather"], default="v32",
                     help="v32 (default): the headline DeepSeek-V3.2 indexer + sparse attention decode step; gqa: GLM-4.5 "
                          "paged GQA decode (batch 64, 96/8 heads, contexts U[4096, 32768]); select_experts: GLM-4.5 "
                          "router (8192 tokens x 160 experts); attention_pre_quant: GLM-4.5 fused attention prolog")
@@ -503,6 +503,55 @@ def bench_sfa_prefill(args, torch, lib, dev):
     }))
 
 
+def bench_paged_gather(args, torch, lib, dev):
+    """Standalone paged gather at the attention's own gather shape: batch 32 sequences of --ctx cached tokens in pages
+    of 128, packed 656-byte cache rows (512 int8 + 64 bf16 + 4 fp32), 2048 random distinct logical indices per sequence
+    -> 65536 rows of 656 bytes.  Three caches are rotated so that no step finds its rows in the last-level cache."""
+    from pypto_amd.experimental import paged_gather
+    b, k, bs, hidden = args.batch, 2048, 128, 656
+    g = torch.Generator(device=dev).manual_seed(0)
+    per = -(-args.ctx // bs)
+    table = torch.randperm(b * per, generator=g, device=dev).to(torch.int32).reshape(b, per)
+    idx = torch.stack([torch.randperm(args.ctx, generator=g, device=dev)[:k] for _ in range(b)]).to(torch.int32)
+    caches = [torch.randint(-127, 128, (b * per * bs, hidden), generator=g, device=dev, dtype=torch.int8)
+              for _ in range(3)]
+    out = torch.empty((b * k, hidden), dtype=torch.int8, device=dev)
+
+    def step(i):
+        paged_gather(caches[i % len(caches)], idx, table, bs, out=out)
+
+    ms, kernels = timed(torch, lib, step, args, nsets=len(caches))
+    rows = b * k
+    work = rows * (2 * hidden + 4)
+    us = kernels["paged_gather_kernel"]
+    achieved = work / us / 1e3
+    cpu = None
+    if not args.no_cpu:
+        from oracle import paged
+        src, ix, tb = caches[0][:per * bs * 4].cpu(), idx[:4].cpu(), (table[:4] % (per * 4)).cpu()
+        paged.paged_gather(src, ix[0], tb[0], bs)
+        t0, n = time.perf_counter(), 0
+        while time.perf_counter() - t0 < 10.0:
+            for i in range(4):
+                paged.paged_gather(src, ix[i], tb[i], bs)
+            n += 4 * k
+        cpu = {"value": round(n / (time.perf_counter() - t0), 1), "unit": "rows/s", "cores": torch.get_num_threads(),
+               "kind": "port", "sample": "4 sequences' 2048-row gathers out of a 4-sequence cache of the same row "
+                                         "width, repeated for ten seconds after an untimed pass"}
+    print(json.dumps({
+        "metric": "gathered cache rows/sec + achieved HBM GB/s (% of peak), paged gather of 656-byte rows",
+        "value": round(rows / (ms * 1e-3), 1), "unit": "rows/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(ms, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "u8",
+        "data": "synthetic",
+        "config": {"workload": f"paged gather, batch {b} x {k} logical indices over {args.ctx} cached tokens each, "
+                               f"pages of {bs}, rows of {hidden} bytes"},
+        "roofline": {"kernel": "paged_gather_kernel", "bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS,
+                     "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None,
+                     "work_per_launch": work, "us_per_launch": round(us, 2)},
+        "kernels": [{"kernel": n, "us": round(u, 2)} for n, u in kernels.items()], "cpu_baseline": cpu,
+    }))
+
+
 def bench_decode_layer(args, torch, lib, dev):
     """The attention front end of one DeepSeek-V3.2 decode layer as three chained calls on shared buffers: the fused MLA +
     indexer prolog writes the query tensors and the new cache rows (the last position of every sequence), the lightning
@@ -596,6 +645,8 @@ def main():
         return bench_decode_layer(args, torch, lib, dev)
     if args.workload == "attention_pre_quant":
         return bench_attention_pre_quant(args, torch, lib, dev)
+    if args.workload == "paged_gather":
+        return bench_paged_gather(args, torch, lib, dev)
     if args.workload == "sfa_prefill":
         return bench_sfa_prefill(args, torch, lib, dev)
     b, ctx, s1 = args.batch, args.ctx, args.s1

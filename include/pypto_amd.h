@@ -315,6 +315,33 @@ int pto_mla_indexer_prolog_quant_launch(const PtoTensorDesc* tensors, uint32_t n
                                         const PtoMlaIndexerPrologParams* params, void* workspace,
                                         uint64_t workspace_bytes, void* hip_stream);
 
+/*
+ * gather_in_ub(param, indices, block_table, block_size, axis=-2) and
+ * gather_in_l1(src, indices, block_table, block_size, size, is_b_matrix, is_trans)
+ * (python/pypto/experimental/gather.py:18-84; semantics
+ * framework/src/interface/interpreter/calculator/calc_torch.cpp:1870-1981):
+ *   out[j, :size] = src[ block_table[idx[j] / block_size] * block_size + idx[j] % block_size , :size ].
+ * The reference operators take one index row and one page-table row ([1, k], [1, nblk]); here b such pairs are
+ * gathered in one launch, row i of indices through row i of block_table, output rows in index order.
+ * tensors[4] or tensors[5], in order:
+ *   0 src         [N, hidden]   INT8 | INT32 | INT64 | FP16 | FP32 | BF16
+ *   1 indices     [b, k]        INT32 | INT64
+ *   2 block_table [b, nblk]     INT32 | INT64
+ *   3 out         [b*k, size]   dtype of src (output)
+ *   4 status      [1]           INT32 (optional, in/out): incremented once per entry the reference's interpreter would
+ *                               reject (index outside [0, nblk*block_size), negative page, row outside src;
+ *                               calc_torch.cpp:1916-1950).  Such an entry's output row is written as zeros.
+ * `size` (gather_in_l1's column count; operation_impl.cpp:1705-1712) must be <= hidden; 0 means all columns.
+ * The layout hints is_b_matrix / is_trans and `axis` describe Ascend buffers and have no counterpart.  No workspace.
+ */
+typedef struct {
+    int32_t block_size;
+    int32_t size;
+} PtoPagedGatherParams;
+uint64_t pto_paged_gather_workspace(const PtoTensorDesc* tensors, uint32_t n_tensors, const PtoPagedGatherParams* params);
+int pto_paged_gather_launch(const PtoTensorDesc* tensors, uint32_t n_tensors, const PtoPagedGatherParams* params,
+                            void* workspace, uint64_t workspace_bytes, void* hip_stream);
+
 /* Message of the calling thread's most recent failed call ("" if none).  Replaces the message strings
  * the reference's binding layer returns (python/src/bindings/runtime.cpp:270-335). */
 const char* pto_last_error(void);
@@ -327,7 +354,8 @@ const char* pto_last_error(void);
  * Kernel ids: 0 indexer_score_kernel, 1 indexer_topk_kernel, 2 sfa_decode_kernel, 3 sfa_combine_kernel,
  * 4 indexer_select_kernel, 5 select_experts_kernel, 6 gqa_decode_kernel, 7 gqa_combine_kernel, 8 apq_norm_kernel,
  * 9 prolog_qx_kernel, 10 apq_gemm_kernel, 11 prolog_k_kernel, 12 mla_xa_kernel, 13 mla_norm_kernel (fused_norm_kernel in the fused
- * prolog), 14 mla_qb_kernel (fused_qb_kernel in the fused prolog), 15 mla_wuk_kernel, 16 apq_head_kernel
+ * prolog), 14 mla_qb_kernel (fused_qb_kernel in the fused prolog), 15 mla_wuk_kernel, 16 apq_head_kernel,
+ * 17 paged_gather_kernel
  * (pto_kernel_name returns "" past the last id).
  * Off by default; not for use under graph capture.
  */

@@ -67,6 +67,10 @@ class AttentionPreQuantParams(ctypes.Structure):
     _fields_ = [("eps", ctypes.c_float)]
 
 
+class PagedGatherParams(ctypes.Structure):
+    _fields_ = [("block_size", ctypes.c_int32), ("size", ctypes.c_int32)]
+
+
 _OPS = {
     "sfa_quant": SfaParams,
     "sfa_antiquant": SfaParams,
@@ -77,6 +81,7 @@ _OPS = {
     "mla_prolog_quant": MlaPrologParams,
     "mla_indexer_prolog_quant": MlaIndexerPrologParams,
     "attention_pre_quant": AttentionPreQuantParams,
+    "paged_gather": PagedGatherParams,
 }
 
 # C status -> Python exception type wrapped by FeError

@@ -11,7 +11,7 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 INCLUDE = os.path.join(os.path.dirname(HERE), "include")
 LIB_PATH = os.path.join(HERE, "libpypto_amd.so")
-SOURCES = ["api.cpp", "timing.cpp", "sfa_kernels.hip", "indexer_kernels.hip", "select_experts_kernels.hip", "gqa_kernels.hip", "prolog_kernels.hip", "mla_prolog_kernels.hip", "attention_pre_kernels.hip"]
+SOURCES = ["api.cpp", "timing.cpp", "sfa_kernels.hip", "indexer_kernels.hip", "select_experts_kernels.hip", "gqa_kernels.hip", "prolog_kernels.hip", "mla_prolog_kernels.hip", "attention_pre_kernels.hip", "gather_kernels.hip"]
 
 HIPCC_FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-shared", "-x", "hip",

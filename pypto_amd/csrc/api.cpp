@@ -338,6 +338,59 @@ int plan_attention_pre(const PtoTensorDesc* ts, uint32_t n, const PtoAttentionPr
     return PTO_OK;
 }
 
+int plan_paged_gather(const PtoTensorDesc* ts, uint32_t n, const PtoPagedGatherParams* p, pto::GatherArgs* a)
+{
+    const char* op = "paged_gather";
+    if (ts == nullptr || (n != 4 && n != 5)) return fail(PTO_ERR_ARG_COUNT, "%s: expected 4 or 5 tensors, got %u", op, n);
+    if (p == nullptr) return fail(PTO_ERR_PARAM, "%s: params is null", op);
+    if (p->block_size <= 0) return fail(PTO_ERR_PARAM, "%s: block_size must be positive, got %d", op, p->block_size);
+    if (p->size < 0) return fail(PTO_ERR_PARAM, "%s: size must not be negative, got %d", op, p->size);
+    int64_t esize;
+    switch (ts[0].dataType) {
+        case PTO_DT_INT8: esize = 1; break;
+        case PTO_DT_FP16: case PTO_DT_BF16: esize = 2; break;
+        case PTO_DT_INT32: case PTO_DT_FP32: esize = 4; break;
+        case PTO_DT_INT64: esize = 8; break;
+        default: return fail(PTO_ERR_DTYPE, "%s: src has an unsupported dtype (%d)", op, ts[0].dataType);
+    }
+    for (int i = 1; i <= 2; ++i)
+        if (ts[i].dataType != PTO_DT_INT32 && ts[i].dataType != PTO_DT_INT64)
+            return fail(PTO_ERR_DTYPE, "%s: %s must be int32 or int64, got %s", op, i == 1 ? "indices" : "block_table",
+                        dtype_name(ts[i].dataType));
+    int rc;
+    if ((rc = check_tensor(op, ts[0], "src", ts[0].dataType, 2))) return rc;
+    if ((rc = check_tensor(op, ts[1], "indices", ts[1].dataType, 2))) return rc;
+    if ((rc = check_tensor(op, ts[2], "block_table", ts[2].dataType, 2))) return rc;
+    if ((rc = check_tensor(op, ts[3], "out", ts[0].dataType, 2))) return rc; // out and src share a dtype
+    if (n == 5) {
+        if ((rc = check_tensor(op, ts[4], "status", PTO_DT_INT32, 1))) return rc;
+        if (ts[4].shape[0] != 1) return fail(PTO_ERR_SHAPE, "%s: status must hold one word", op);
+    }
+    const int64_t hidden = ts[0].shape[1], b = ts[1].shape[0], k = ts[1].shape[1];
+    const int64_t size = p->size > 0 ? p->size : hidden;
+    if (size > hidden) return fail(PTO_ERR_PARAM, "%s: size (%lld) exceeds the source row width (%lld)", op, (long long)size, (long long)hidden);
+    if (ts[2].shape[0] != b) return fail(PTO_ERR_SHAPE, "%s: block_table has %lld rows, indices has %lld", op, (long long)ts[2].shape[0], (long long)b);
+    if (k > 0 && b > 0x7fffffffffffLL / k) return fail(PTO_ERR_SHAPE, "%s: too many indices", op);
+    if (ts[3].shape[0] != b * k || ts[3].shape[1] != size)
+        return fail(PTO_ERR_SHAPE, "%s: out must be [%lld, %lld], got [%lld, %lld]", op, (long long)(b * k), (long long)size,
+                    (long long)ts[3].shape[0], (long long)ts[3].shape[1]);
+    a->src = ts[0].addr;
+    a->indices = ts[1].addr;
+    a->block_table = ts[2].addr;
+    a->out = ts[3].addr;
+    a->status = n == 5 ? static_cast<int32_t*>(ts[4].addr) : nullptr;
+    a->rows = b * k;
+    a->k = k > 0 ? k : 1;
+    a->nblk = ts[2].shape[1];
+    a->block_size = p->block_size;
+    a->n_src = ts[0].shape[0];
+    a->src_pitch = hidden * esize;
+    a->row_bytes = size * esize;
+    a->idx64 = ts[1].dataType == PTO_DT_INT64;
+    a->bt64 = ts[2].dataType == PTO_DT_INT64;
+    return PTO_OK;
+}
+
 int plan_select_experts(const PtoTensorDesc* ts, uint32_t n, const PtoSelectExpertsParams* p, pto::SelectExpertsArgs* a)
 {
     const char* op = "select_experts";
@@ -816,6 +869,19 @@ int pto_gqa_decode_launch(const PtoTensorDesc* tensors, uint32_t n_tensors, cons
     return PTO_OK;
 }
 
+uint64_t pto_paged_gather_workspace(const PtoTensorDesc*, uint32_t, const PtoPagedGatherParams*) { return 0; }
+
+int pto_paged_gather_launch(const PtoTensorDesc* tensors, uint32_t n_tensors, const PtoPagedGatherParams* params, void*,
+                            uint64_t, void* hip_stream)
+{
+    pto::GatherArgs a;
+    int rc = plan_paged_gather(tensors, n_tensors, params, &a);
+    if (rc) return rc;
+    hipError_t e = pto::paged_gather_launch(a, static_cast<hipStream_t>(hip_stream));
+    if (e != hipSuccess) return fail(PTO_ERR_HIP, "paged_gather: HIP launch failed: %s", hipGetErrorString(e));
+    return PTO_OK;
+}
+
 uint64_t pto_select_experts_workspace(const PtoTensorDesc*, uint32_t, const PtoSelectExpertsParams*) { return 0; }
 
 int pto_select_experts_launch(const PtoTensorDesc* tensors, uint32_t n_tensors, const PtoSelectExpertsParams* params,
@@ -911,7 +977,7 @@ const char* pto_kernel_name(int kernel_id)
                                   "sfa_combine_kernel", "indexer_select_kernel", "select_experts_kernel",
                                   "gqa_decode_kernel", "gqa_combine_kernel", "apq_norm_kernel", "prolog_qx_kernel", "apq_gemm_kernel",
                                   "prolog_k_kernel", "mla_xa_kernel", "mla_norm_kernel", "mla_qb_kernel",
-                                  "mla_wuk_kernel", "apq_head_kernel"};
+                                  "mla_wuk_kernel", "apq_head_kernel", "paged_gather_kernel"};
     return kernel_id >= 0 && kernel_id < pto::KID_COUNT ? names[kernel_id] : "";
 }
 

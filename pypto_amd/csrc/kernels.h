@@ -202,4 +202,18 @@ uint64_t attention_pre_workspace_bytes(int64_t t, int64_t h, int64_t n_out);
 void attention_pre_bind_workspace(AttnPreArgs& a, void* workspace);
 hipError_t attention_pre_launch(const AttnPreArgs& a, hipStream_t stream);
 
+// ---------------------------------------------------------------- paged row gather
+struct GatherArgs {
+    const void* src;         // [n_src, hidden], any element type
+    const void* indices;     // [b, k] int32 or int64 logical token indices
+    const void* block_table; // [b, nblk] int32 or int64 physical page of each logical page
+    void* out;               // [b * k, size]
+    int32_t* status;         // optional: incremented once per entry that addresses no source row
+    int64_t rows, k, nblk, block_size, n_src;
+    int64_t src_pitch, row_bytes; // bytes between source rows; bytes copied per row (= output pitch)
+    bool idx64, bt64;
+};
+
+hipError_t paged_gather_launch(const GatherArgs& a, hipStream_t stream);
+
 } // namespace pto

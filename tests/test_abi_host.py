@@ -216,3 +216,31 @@ def test_attention_pre_quant_validation_and_workspace(lib):
     assert rc == -3 and "cos must have rank 3" in msg
     assert launch_rc(lib, "attention_pre_quant", apq_specs(t=0), p)[0] == 0     # nothing to do, nothing launched
     assert launch_rc(lib, "attention_pre_quant", apq_specs(), AttentionPreQuantParams(float("nan")))[0] == -4
+
+
+def test_paged_gather_validation(lib):
+    from pypto_amd._runtime import PagedGatherParams
+    INT64 = 4
+
+    def specs(src=(INT8, (1024, 656)), idx=(INT32, (2, 16)), bt=(INT32, (2, 4)), out=(INT8, (32, 656))):
+        return [src, idx, bt, out]
+    p = PagedGatherParams(128, 0)
+    assert lib.pto_paged_gather_workspace(descs(specs()), 4, ctypes.byref(p)) == 0
+    rc, msg = launch_rc(lib, "paged_gather", specs()[:3], p)
+    assert rc == -1 and "4 or 5 tensors" in msg
+    rc, msg = launch_rc(lib, "paged_gather", specs(idx=(FP16, (2, 16))), p)
+    assert rc == -2 and "indices must be int32 or int64" in msg
+    rc, msg = launch_rc(lib, "paged_gather", specs(out=(FP16, (32, 656))), p)
+    assert rc == -2 and "out must be int8" in msg
+    rc, msg = launch_rc(lib, "paged_gather", specs(bt=(INT64, (3, 4))), p)
+    assert rc == -3 and "block_table has 3 rows" in msg
+    rc, msg = launch_rc(lib, "paged_gather", specs(out=(INT8, (31, 656))), p)
+    assert rc == -3 and "out must be [32, 656]" in msg
+    rc, msg = launch_rc(lib, "paged_gather", specs(out=(INT8, (32, 700))), PagedGatherParams(128, 700))
+    assert rc == -4 and "exceeds the source row width" in msg
+    assert launch_rc(lib, "paged_gather", specs(), PagedGatherParams(0, 0))[0] == -4
+    assert launch_rc(lib, "paged_gather", specs(), PagedGatherParams(128, -1))[0] == -4
+    rc, msg = launch_rc(lib, "paged_gather", specs() + [(INT32, (2,))], p)
+    assert rc == -3 and "status must hold one word" in msg
+    # nothing to gather: accepted, nothing launched
+    assert launch_rc(lib, "paged_gather", specs(idx=(INT32, (2, 0)), out=(INT8, (0, 656))), p)[0] == 0
