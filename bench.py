@@ -35,6 +35,9 @@ MEASURED_TRAFFIC_BYTES = {
     "indexer_select_kernel": 10.6e6 + 0.8e6,
     "indexer_topk_kernel": 1.2e6 + 0.3e6,
 }
+# same counters and factors on the default shapes of --workload gqa and --workload paged_gather
+GQA_TRAFFIC_BYTES = 5150.7e6 + 65.8e6
+PAGED_GATHER_TRAFFIC_BYTES = 51.4e6 + 43.0e6
 
 
 def parse():
@@ -209,7 +212,8 @@ def bench_gqa(args, torch, lib, dev):
         "config": {"workload": f"paged GQA decode attention, batch {b}, {nq}/{nkv} heads x {d}, bf16 KV, block {bs}, "
                                f"{tokens} cached tokens in total"},
         "roofline": {"kernel": "gqa_decode_kernel", "bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS,
-                     "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None,
+                     "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": GQA_TRAFFIC_BYTES,
+                     "traffic_unit": "bytes per launch (rocprofv3 FETCH_SIZE + WRITE_SIZE, calibrated)",
                      "work_per_launch": work, "us_per_launch": round(us, 2)},
         "kernels": [{"kernel": n, "us": round(u, 2)} for n, u in kernels.items()], "cpu_baseline": None,
     }))
@@ -546,7 +550,9 @@ def bench_paged_gather(args, torch, lib, dev):
         "config": {"workload": f"paged gather, batch {b} x {k} logical indices over {args.ctx} cached tokens each, "
                                f"pages of {bs}, rows of {hidden} bytes"},
         "roofline": {"kernel": "paged_gather_kernel", "bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS,
-                     "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None,
+                     "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4),
+                     "traffic": PAGED_GATHER_TRAFFIC_BYTES if (b, args.ctx) == (32, 65536) else None,
+                     "traffic_unit": "bytes per launch (rocprofv3 FETCH_SIZE + WRITE_SIZE, calibrated)",
                      "work_per_launch": work, "us_per_launch": round(us, 2)},
         "kernels": [{"kernel": n, "us": round(u, 2)} for n, u in kernels.items()], "cpu_baseline": cpu,
     }))
