@@ -321,12 +321,14 @@ __global__ __attribute__((amdgpu_flat_work_group_size(512, 512), amdgpu_waves_pe
         uint8_t* stage = smem + (it & 1) * STAGE;
         const uint32_t valid = tmask[it];
         // half of S^T[token, head] = K[token, :] . Q[head, :] (k-steps of parity kh)
-        f32x16 s, s2; // even / odd k-steps: two independent accumulation chains keep the matrix core busy
+        // One accumulation chain: a second one (even / odd k-steps) saves the few cycles a dependent MFMA waits for its
+        // predecessor, but its 16 registers are worth more as two further operand reads in flight.
+        f32x16 s;
 #pragma unroll
-        for (int r = 0; r < 16; ++r) s[r] = s2[r] = 0.f;
+        for (int r = 0; r < 16; ++r) s[r] = 0.f;
         {
             // operand reads run AHEAD k-steps ahead of the MFMAs that use them
-            constexpr int AHEAD = 2, N = KSTEPS / 2;
+            constexpr int AHEAD = 4, N = KSTEPS / 2;
             bf16x8 kf[N], qp[N];
             auto fetch = [&](int i) {
                 kf[i] = *reinterpret_cast<const bf16x8*>(stage + s_off[i & 1] + (i >> 1) * 128);
@@ -338,10 +340,7 @@ __global__ __attribute__((amdgpu_flat_work_group_size(512, 512), amdgpu_waves_pe
             for (int i = 0; i < N; ++i) {
                 if (i + AHEAD < N) fetch(i + AHEAD);
                 const bf16x8 qi = i < NREG_KSTEPS ? q[i < NREG_KSTEPS ? i : 0] : qp[i];
-                if (i & 1)
-                    s2 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf[i], qi, s2, 0, 0, 0);
-                else
-                    s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf[i], qi, s, 0, 0, 0);
+                s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf[i], qi, s, 0, 0, 0);
             }
             // issue order: AHEAD fetches, then (MFMA, fetch) pairs, then the last MFMAs; a fetch is one LDS read
             // for a k-step whose Q fragment is in registers and two for a parked one
@@ -357,8 +356,6 @@ __global__ __attribute__((amdgpu_flat_work_group_size(512, 512), amdgpu_waves_pe
                 __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
             }
             __builtin_amdgcn_sched_group_barrier(0x008, AHEAD, 0);
-#pragma unroll
-            for (int r = 0; r < 16; ++r) s[r] += s2[r];
         }
 #pragma unroll
         for (int g = 0; g < 4; ++g)
