@@ -381,7 +381,12 @@ __global__ __attribute__((amdgpu_flat_work_group_size(512, 512), amdgpu_waves_pe
                 }
                 mx = fmaxf(mx, s[r]);
             }
-            mx = fmaxf(mx, __shfl_xor(mx, 32)) * c_log2;
+            {
+                // maximum over both halves of the wavefront without a trip through LDS: v_permlane32_swap exchanges the
+                // upper half of its first operand with the lower half of its second
+                const auto sw = __builtin_amdgcn_permlane32_swap(__builtin_bit_cast(unsigned, mx), __builtin_bit_cast(unsigned, mx), false, false);
+                mx = fmaxf(__builtin_bit_cast(float, (unsigned)sw[0]), __builtin_bit_cast(float, (unsigned)sw[1])) * c_log2;
+            }
             // The reference exponent only follows the running maximum when it has grown by more than 2^8: until
             // then P~ = 2^(z - m_run) may exceed 1 (by at most 2^8, no issue for bf16 or the fp32 sums), which
             // makes the rescale of the 128 accumulator registers a rare event.  Every P~, l and O stay relative to
