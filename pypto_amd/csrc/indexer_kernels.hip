@@ -351,15 +351,60 @@ __global__ void indexer_fill_kernel(int32_t* p, int n, int32_t v)
     if (i < n) p[i] = v;
 }
 
+// One step of a wavefront scan in the vector unit's own lane network (no trip through LDS): the value of the lane
+// CTRL names (row_shr:n = 0x110 + n within a row of 16 lanes, row_bcast15 = 0x142 / row_bcast31 = 0x143 across rows,
+// limited to the rows of ROW_MASK), IDENT where there is no such lane.
+template <int CTRL, int ROW_MASK>
+__device__ __forceinline__ uint32_t dpp_from(uint32_t v, uint32_t ident)
+{
+    return (uint32_t)__builtin_amdgcn_update_dpp((int)ident, (int)v, CTRL, ROW_MASK, 0xf, false);
+}
+
+// wavefront-wide inclusive prefix sum: lane l gets v[0] + .. + v[l]
+__device__ __forceinline__ uint32_t wave_prefix_sum(uint32_t v)
+{
+    v += dpp_from<0x111, 0xf>(v, 0u);
+    v += dpp_from<0x112, 0xf>(v, 0u);
+    v += dpp_from<0x114, 0xf>(v, 0u);
+    v += dpp_from<0x118, 0xf>(v, 0u);
+    v += dpp_from<0x142, 0xa>(v, 0u); // rows 1 and 3 add the totals of rows 0 and 2
+    v += dpp_from<0x143, 0xc>(v, 0u); // rows 2 and 3 add the total of rows 0 and 1
+    return v;
+}
+
+// wavefront-wide minimum / maximum, the same value in every lane
+__device__ __forceinline__ uint32_t wave_min(uint32_t v)
+{
+    v = min(v, dpp_from<0x111, 0xf>(v, 0xffffffffu));
+    v = min(v, dpp_from<0x112, 0xf>(v, 0xffffffffu));
+    v = min(v, dpp_from<0x114, 0xf>(v, 0xffffffffu));
+    v = min(v, dpp_from<0x118, 0xf>(v, 0xffffffffu));
+    v = min(v, dpp_from<0x142, 0xa>(v, 0xffffffffu));
+    v = min(v, dpp_from<0x143, 0xc>(v, 0xffffffffu));
+    return (uint32_t)__builtin_amdgcn_readlane((int)v, 63);
+}
+
+__device__ __forceinline__ uint32_t wave_max(uint32_t v)
+{
+    v = max(v, dpp_from<0x111, 0xf>(v, 0u));
+    v = max(v, dpp_from<0x112, 0xf>(v, 0u));
+    v = max(v, dpp_from<0x114, 0xf>(v, 0u));
+    v = max(v, dpp_from<0x118, 0xf>(v, 0u));
+    v = max(v, dpp_from<0x142, 0xa>(v, 0u));
+    v = max(v, dpp_from<0x143, 0xc>(v, 0u));
+    return (uint32_t)__builtin_amdgcn_readlane((int)v, 63);
+}
+
 // block-wide inclusive suffix sum (lane t gets sum of v[t .. nthreads-1]); tmp holds one word per wavefront
 template <int NWAVES>
 __device__ __forceinline__ uint32_t block_suffix_sum(uint32_t v, uint32_t* tmp)
 {
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-#pragma unroll
-    for (int d = 1; d < 64; d <<= 1) {
-        const uint32_t o = __shfl_down(v, d);
-        if (lane + d < 64) v += o;
+    {
+        // suffix = wavefront total - exclusive prefix (unsigned arithmetic, exact)
+        const uint32_t incl = wave_prefix_sum(v);
+        const uint32_t total = (uint32_t)__builtin_amdgcn_readlane((int)incl, 63);
+        v = total - incl + v;
     }
     __syncthreads();
     if (lane == 0) tmp[wave] = v;
@@ -575,11 +620,8 @@ __device__ __forceinline__ void order_and_write(uint64_t* cand, uint32_t m, uint
             kmax = max(kmax, (uint32_t)(w[h] >> 32));
         }
     }
-#pragma unroll
-    for (int d = 1; d < 64; d <<= 1) {
-        kmin = min(kmin, (uint32_t)__shfl_xor((int)kmin, d));
-        kmax = max(kmax, (uint32_t)__shfl_xor((int)kmax, d));
-    }
+    kmin = wave_min(kmin);
+    kmax = wave_max(kmax);
     if ((tid & 63) == 0) {
         atomicMin(&tmp[14], kmin);
         atomicMax(&tmp[15], kmax);
