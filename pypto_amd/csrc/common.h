@@ -35,6 +35,27 @@ typedef int32_t i32x4 __attribute__((ext_vector_type(4)));
 typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 
+// Wavefront-wide maximum of non-negative or arbitrary floats, the same value in every lane, in the vector unit's own lane
+// network (DPP row_shr steps inside the rows of 16 lanes, row_bcast15 / row_bcast31 across them) instead of six
+// dependent permutes through LDS.  The maximum does not depend on the order, so the result is the butterfly's.
+template <int CTRL, int ROW_MASK>
+__device__ __forceinline__ float dpp_from_f32(float v, float ident)
+{
+    return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(__builtin_bit_cast(int, ident), __builtin_bit_cast(int, v),
+                                                                 CTRL, ROW_MASK, 0xf, false));
+}
+__device__ __forceinline__ float wave_max_f32(float v)
+{
+    const float lo = -__builtin_inff();
+    v = fmaxf(v, dpp_from_f32<0x111, 0xf>(v, lo));
+    v = fmaxf(v, dpp_from_f32<0x112, 0xf>(v, lo));
+    v = fmaxf(v, dpp_from_f32<0x114, 0xf>(v, lo));
+    v = fmaxf(v, dpp_from_f32<0x118, 0xf>(v, lo));
+    v = fmaxf(v, dpp_from_f32<0x142, 0xa>(v, lo));
+    v = fmaxf(v, dpp_from_f32<0x143, 0xc>(v, lo));
+    return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), 63));
+}
+
 // Two fp32 -> one dword holding two bf16 (round to nearest even), low half = a.
 __device__ __forceinline__ uint32_t pack_bf16x2(float a, float b)
 {

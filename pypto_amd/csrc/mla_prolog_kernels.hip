@@ -211,12 +211,7 @@ __device__ __forceinline__ float wave_sum(float v)
     for (int d = 1; d < 64; d <<= 1) v += __shfl_xor(v, d);
     return v;
 }
-__device__ __forceinline__ float wave_max(float v)
-{
-#pragma unroll
-    for (int d = 1; d < 64; d <<= 1) v = fmaxf(v, __shfl_xor(v, d));
-    return v;
-}
+__device__ __forceinline__ float wave_max(float v) { return wave_max_f32(v); }
 
 // one workgroup of 256 lanes per token
 __device__ __forceinline__ void mla_norm_body(const MlaPrologArgs& a, int tok)

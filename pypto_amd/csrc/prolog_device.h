@@ -258,8 +258,7 @@ __device__ __forceinline__ float block_sum128(float v, float* red)
 }
 __device__ __forceinline__ float block_max128(float v, float* red)
 {
-#pragma unroll
-    for (int d = 1; d < 64; d <<= 1) v = fmaxf(v, __shfl_xor(v, d));
+    v = wave_max_f32(v);
     __syncthreads();
     if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = v;
     __syncthreads();
