@@ -6,11 +6,15 @@
  * operator is a workspace-query / launch pair over one flat tensor list, the calling convention of the
  * reference's ahead-of-time kernel bundle ABI (framework/include/tile_fwk_bundle/pypto_bundle_api.h:30-51):
  * the tensor list holds every operand, outputs included, in the positional order of the Python entry
- * point it replaces; the launch is asynchronous on the caller's HIP stream; 0 means success.
+ * point it replaces; the launch is asynchronous on the caller's HIP stream unless `sync` is non-zero, in which case
+ * it returns after the stream has drained (pypto_bundle_api.h:41-44: "sync!=0 waits for completion"); 0 means success.
+ * Besides the reference's (workspace, stream, sync) a launch takes `workspace_bytes`, so that a short workspace is
+ * refused instead of overrun.
  *
  * Tensor descriptors use the reference's layout (pypto_bundle_api.h:30-35) and its DataType numbering
  * (framework/include/tilefwk/data_type.h:33-65).  All tensors are dense row-major device memory on the
- * current device.  No entry point synchronises the stream; none allocates device memory: scratch comes
+ * current device.  With sync = 0 no entry point synchronises the stream (a launch can be captured into a HIP graph);
+ * none allocates device memory: scratch comes
  * from the caller through `workspace` (reference: python/src/bindings/runtime.cpp:697-702, where the
  * workspace is a torch allocation made by the caller's side of the binding).
  */
@@ -84,7 +88,7 @@ typedef struct {
  */
 uint64_t pto_sfa_quant_workspace(const PtoTensorDesc* tensors, uint32_t n_tensors, const PtoSfaParams* params);
 int pto_sfa_quant_launch(const PtoTensorDesc* tensors, uint32_t n_tensors, const PtoSfaParams* params,
-                         void* workspace, uint64_t workspace_bytes, void* hip_stream);
+                         void* workspace, uint64_t workspace_bytes, void* hip_stream, int sync);
 
 /*
  * sparse_attention_antiquant_d / _p / _d_950
@@ -100,7 +104,7 @@ int pto_sfa_quant_launch(const PtoTensorDesc* tensors, uint32_t n_tensors, const
  */
 uint64_t pto_sfa_antiquant_workspace(const PtoTensorDesc* tensors, uint32_t n_tensors, const PtoSfaParams* params);
 int pto_sfa_antiquant_launch(const PtoTensorDesc* tensors, uint32_t n_tensors, const PtoSfaParams* params,
-                             void* workspace, uint64_t workspace_bytes, void* hip_stream);
+                             void* workspace, uint64_t workspace_bytes, void* hip_stream, int sync);
 
 /*
  * lightning_indexer_decode (models/deepseek_v32_exp/lightning_indexer_quant_impl.py:226-238).
@@ -117,7 +121,7 @@ int pto_sfa_antiquant_launch(const PtoTensorDesc* tensors, uint32_t n_tensors, c
 uint64_t pto_lightning_indexer_workspace(const PtoTensorDesc* tensors, uint32_t n_tensors,
                                          const PtoIndexerParams* params);
 int pto_lightning_indexer_launch(const PtoTensorDesc* tensors, uint32_t n_tensors, const PtoIndexerParams* params,
-                                 void* workspace, uint64_t workspace_bytes, void* hip_stream);
+                                 void* workspace, uint64_t workspace_bytes, void* hip_stream, int sync);
 
 /* Scalar arguments of select_experts (models/glm_v4_5/glm_select_experts.py:317-330: top_k, renormalize, topk_group,
  * num_expert_group).  routed_scaling_factor and fill_neg_inf come from the reference's generalised gating golden
@@ -145,7 +149,7 @@ typedef struct {
 uint64_t pto_select_experts_workspace(const PtoTensorDesc* tensors, uint32_t n_tensors,
                                       const PtoSelectExpertsParams* params);
 int pto_select_experts_launch(const PtoTensorDesc* tensors, uint32_t n_tensors, const PtoSelectExpertsParams* params,
-                              void* workspace, uint64_t workspace_bytes, void* hip_stream);
+                              void* workspace, uint64_t workspace_bytes, void* hip_stream, int sync);
 
 /* Scalar arguments of the GLM-4.5 paged decode attention (models/glm_v4_5/glm_attention.py:1585-1594: softmax_scale; the
  * trailing tile_config holds Ascend tiling knobs and has no counterpart here). */
@@ -168,7 +172,7 @@ typedef struct {
  */
 uint64_t pto_gqa_decode_workspace(const PtoTensorDesc* tensors, uint32_t n_tensors, const PtoGqaParams* params);
 int pto_gqa_decode_launch(const PtoTensorDesc* tensors, uint32_t n_tensors, const PtoGqaParams* params, void* workspace,
-                          uint64_t workspace_bytes, void* hip_stream);
+                          uint64_t workspace_bytes, void* hip_stream, int sync);
 
 /* Scalar arguments of lightning_indexer_prolog_quant: attrs.eps of the LayerNorm
  * (models/deepseek_v32_exp/lightning_indexer_prolog_quant_impl.py:84-88; the layout strings are fixed "TND" / "PA_BSND",
@@ -205,7 +209,7 @@ typedef struct {
 uint64_t pto_indexer_prolog_workspace(const PtoTensorDesc* tensors, uint32_t n_tensors,
                                       const PtoIndexerPrologParams* params);
 int pto_indexer_prolog_launch(const PtoTensorDesc* tensors, uint32_t n_tensors, const PtoIndexerPrologParams* params,
-                              void* workspace, uint64_t workspace_bytes, void* hip_stream);
+                              void* workspace, uint64_t workspace_bytes, void* hip_stream, int sync);
 
 /* Scalar argument of attention_pre_quant: the epsilon of its three RmsNorms, a constant 1e-5 inside the reference kernel
  * (models/glm_v4_5/glm_attention_pre_quant.py:301). */
@@ -243,7 +247,7 @@ uint64_t pto_attention_pre_quant_workspace(const PtoTensorDesc* tensors, uint32_
                                            const PtoAttentionPreQuantParams* params);
 int pto_attention_pre_quant_launch(const PtoTensorDesc* tensors, uint32_t n_tensors,
                                    const PtoAttentionPreQuantParams* params, void* workspace, uint64_t workspace_bytes,
-                                   void* hip_stream);
+                                   void* hip_stream, int sync);
 
 /* Scalar arguments of mla_prolog_quant_d / mla_prolog_quant_p: the two RmsNorm epsilons and the cache mode
  * (models/deepseek_v32_exp/mla_prolog_quant_impl.py:866-871; tile_config and rope_cfg hold Ascend tiling knobs). */
@@ -285,7 +289,7 @@ typedef struct {
 uint64_t pto_mla_prolog_quant_workspace(const PtoTensorDesc* tensors, uint32_t n_tensors,
                                         const PtoMlaPrologParams* params);
 int pto_mla_prolog_quant_launch(const PtoTensorDesc* tensors, uint32_t n_tensors, const PtoMlaPrologParams* params,
-                                void* workspace, uint64_t workspace_bytes, void* hip_stream);
+                                void* workspace, uint64_t workspace_bytes, void* hip_stream, int sync);
 
 /* Scalar arguments of mla_indexer_prolog_quant_d / _p: the MLA prolog's two epsilons and cache mode, and ip_attrs.eps of
  * the indexer's LayerNorm (models/deepseek_v32_exp/mla_indexer_prolog_quant_impl.py:521-527). */
@@ -313,7 +317,7 @@ uint64_t pto_mla_indexer_prolog_quant_workspace(const PtoTensorDesc* tensors, ui
                                                 const PtoMlaIndexerPrologParams* params);
 int pto_mla_indexer_prolog_quant_launch(const PtoTensorDesc* tensors, uint32_t n_tensors,
                                         const PtoMlaIndexerPrologParams* params, void* workspace,
-                                        uint64_t workspace_bytes, void* hip_stream);
+                                        uint64_t workspace_bytes, void* hip_stream, int sync);
 
 /*
  * gather_in_ub(param, indices, block_table, block_size, axis=-2) and
@@ -340,7 +344,7 @@ typedef struct {
 } PtoPagedGatherParams;
 uint64_t pto_paged_gather_workspace(const PtoTensorDesc* tensors, uint32_t n_tensors, const PtoPagedGatherParams* params);
 int pto_paged_gather_launch(const PtoTensorDesc* tensors, uint32_t n_tensors, const PtoPagedGatherParams* params,
-                            void* workspace, uint64_t workspace_bytes, void* hip_stream);
+                            void* workspace, uint64_t workspace_bytes, void* hip_stream, int sync);
 
 /* Message of the calling thread's most recent failed call ("" if none).  Replaces the message strings
  * the reference's binding layer returns (python/src/bindings/runtime.cpp:270-335). */

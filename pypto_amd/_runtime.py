@@ -113,7 +113,7 @@ def load_library():
             ln = getattr(lib, f"pto_{op}_launch")
             ln.restype = ctypes.c_int
             ln.argtypes = [ctypes.POINTER(TensorDesc), ctypes.c_uint32, ctypes.POINTER(ptype), ctypes.c_void_p,
-                           ctypes.c_uint64, ctypes.c_void_p]
+                           ctypes.c_uint64, ctypes.c_void_p, ctypes.c_int]
         lib.pto_last_error.restype = ctypes.c_char_p
         lib.pto_last_error.argtypes = []
         lib.pto_abi_version.restype = ctypes.c_int
@@ -195,7 +195,7 @@ def _launch_on_current_device(dev, ws_fn, launch_fn, descs, n, params):
     ws_bytes = ws_fn(descs, n, p)
     ws = torch.empty(ws_bytes, dtype=torch.uint8, device=dev) if ws_bytes else None
     return launch_fn(descs, n, p, ws.data_ptr() if ws is not None else None, ws_bytes,
-                     torch.cuda.current_stream(dev).cuda_stream)
+                     torch.cuda.current_stream(dev).cuda_stream, 0)
 
 
 def launch(op, tensors, params):

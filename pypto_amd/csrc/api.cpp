@@ -730,6 +730,17 @@ int plan_fused_prolog(const PtoTensorDesc* ts, uint32_t n, const PtoMlaIndexerPr
     return PTO_OK;
 }
 
+// The exported launches: the asynchronous launch, then - when the caller asks for it, as the reference's bundle launch
+// allows (framework/include/tile_fwk_bundle/pypto_bundle_api.h:41-44, "sync != 0 waits for completion") - a wait for
+// the stream.
+int finish_launch(const char* op, int rc, void* hip_stream, int sync)
+{
+    if (rc != PTO_OK || sync == 0) return rc;
+    hipError_t e = hipStreamSynchronize(static_cast<hipStream_t>(hip_stream));
+    if (e != hipSuccess) return fail(PTO_ERR_HIP, "%s: waiting for the stream failed: %s", op, hipGetErrorString(e));
+    return PTO_OK;
+}
+
 } // namespace
 
 extern "C" {
@@ -741,7 +752,7 @@ uint64_t pto_mla_indexer_prolog_quant_workspace(const PtoTensorDesc* tensors, ui
     return plan_fused_prolog(tensors, n_tensors, params, nullptr, &plan) == PTO_OK ? plan.ws_bytes : 0;
 }
 
-int pto_mla_indexer_prolog_quant_launch(const PtoTensorDesc* tensors, uint32_t n_tensors,
+static int mla_indexer_prolog_quant_launch_async(const PtoTensorDesc* tensors, uint32_t n_tensors,
                                         const PtoMlaIndexerPrologParams* params, void* workspace,
                                         uint64_t workspace_bytes, void* hip_stream)
 {
@@ -776,7 +787,7 @@ uint64_t pto_mla_prolog_quant_workspace(const PtoTensorDesc* tensors, uint32_t n
     return plan_mla_prolog(tensors, n_tensors, params, &plan) == PTO_OK ? plan.ws_bytes : 0;
 }
 
-int pto_mla_prolog_quant_launch(const PtoTensorDesc* tensors, uint32_t n_tensors, const PtoMlaPrologParams* params,
+static int mla_prolog_quant_launch_async(const PtoTensorDesc* tensors, uint32_t n_tensors, const PtoMlaPrologParams* params,
                                 void* workspace, uint64_t workspace_bytes, void* hip_stream)
 {
     const char* op = "mla_prolog_quant";
@@ -800,7 +811,7 @@ uint64_t pto_indexer_prolog_workspace(const PtoTensorDesc* tensors, uint32_t n_t
     return plan_prolog(tensors, n_tensors, params, &plan) == PTO_OK ? plan.ws_bytes : 0;
 }
 
-int pto_indexer_prolog_launch(const PtoTensorDesc* tensors, uint32_t n_tensors, const PtoIndexerPrologParams* params,
+static int indexer_prolog_launch_async(const PtoTensorDesc* tensors, uint32_t n_tensors, const PtoIndexerPrologParams* params,
                               void* workspace, uint64_t workspace_bytes, void* hip_stream)
 {
     const char* op = "lightning_indexer_prolog_quant";
@@ -824,7 +835,7 @@ uint64_t pto_attention_pre_quant_workspace(const PtoTensorDesc* tensors, uint32_
     return plan_attention_pre(tensors, n_tensors, params, &plan) == PTO_OK ? plan.ws_bytes : 0;
 }
 
-int pto_attention_pre_quant_launch(const PtoTensorDesc* tensors, uint32_t n_tensors,
+static int attention_pre_quant_launch_async(const PtoTensorDesc* tensors, uint32_t n_tensors,
                                    const PtoAttentionPreQuantParams* params, void* workspace, uint64_t workspace_bytes,
                                    void* hip_stream)
 {
@@ -848,7 +859,7 @@ uint64_t pto_gqa_decode_workspace(const PtoTensorDesc* tensors, uint32_t n_tenso
     return plan_gqa(tensors, n_tensors, params, &plan) == PTO_OK ? plan.ws_bytes : 0;
 }
 
-int pto_gqa_decode_launch(const PtoTensorDesc* tensors, uint32_t n_tensors, const PtoGqaParams* params, void* workspace,
+static int gqa_decode_launch_async(const PtoTensorDesc* tensors, uint32_t n_tensors, const PtoGqaParams* params, void* workspace,
                           uint64_t workspace_bytes, void* hip_stream)
 {
     const char* op = "attention";
@@ -871,7 +882,7 @@ int pto_gqa_decode_launch(const PtoTensorDesc* tensors, uint32_t n_tensors, cons
 
 uint64_t pto_paged_gather_workspace(const PtoTensorDesc*, uint32_t, const PtoPagedGatherParams*) { return 0; }
 
-int pto_paged_gather_launch(const PtoTensorDesc* tensors, uint32_t n_tensors, const PtoPagedGatherParams* params, void*,
+static int paged_gather_launch_async(const PtoTensorDesc* tensors, uint32_t n_tensors, const PtoPagedGatherParams* params, void*,
                             uint64_t, void* hip_stream)
 {
     pto::GatherArgs a;
@@ -884,7 +895,7 @@ int pto_paged_gather_launch(const PtoTensorDesc* tensors, uint32_t n_tensors, co
 
 uint64_t pto_select_experts_workspace(const PtoTensorDesc*, uint32_t, const PtoSelectExpertsParams*) { return 0; }
 
-int pto_select_experts_launch(const PtoTensorDesc* tensors, uint32_t n_tensors, const PtoSelectExpertsParams* params,
+static int select_experts_launch_async(const PtoTensorDesc* tensors, uint32_t n_tensors, const PtoSelectExpertsParams* params,
                               void*, uint64_t, void* hip_stream)
 {
     pto::SelectExpertsArgs a;
@@ -901,7 +912,7 @@ uint64_t pto_sfa_quant_workspace(const PtoTensorDesc* tensors, uint32_t n_tensor
     return plan_sfa_quant(tensors, n_tensors, params, &plan) == PTO_OK ? plan.ws_bytes : 0;
 }
 
-int pto_sfa_quant_launch(const PtoTensorDesc* tensors, uint32_t n_tensors, const PtoSfaParams* params, void* workspace,
+static int sfa_quant_launch_async(const PtoTensorDesc* tensors, uint32_t n_tensors, const PtoSfaParams* params, void* workspace,
                          uint64_t workspace_bytes, void* hip_stream)
 {
     SfaPlan plan;
@@ -916,7 +927,7 @@ uint64_t pto_sfa_antiquant_workspace(const PtoTensorDesc* tensors, uint32_t n_te
     return plan_sfa_antiquant(tensors, n_tensors, params, &plan) == PTO_OK ? plan.ws_bytes : 0;
 }
 
-int pto_sfa_antiquant_launch(const PtoTensorDesc* tensors, uint32_t n_tensors, const PtoSfaParams* params,
+static int sfa_antiquant_launch_async(const PtoTensorDesc* tensors, uint32_t n_tensors, const PtoSfaParams* params,
                              void* workspace, uint64_t workspace_bytes, void* hip_stream)
 {
     SfaPlan plan;
@@ -932,7 +943,7 @@ uint64_t pto_lightning_indexer_workspace(const PtoTensorDesc* tensors, uint32_t 
     return plan_indexer(tensors, n_tensors, params, &plan) == PTO_OK ? plan.ws_bytes : 0;
 }
 
-int pto_lightning_indexer_launch(const PtoTensorDesc* tensors, uint32_t n_tensors, const PtoIndexerParams* params,
+static int lightning_indexer_launch_async(const PtoTensorDesc* tensors, uint32_t n_tensors, const PtoIndexerParams* params,
                                  void* workspace, uint64_t workspace_bytes, void* hip_stream)
 {
     const char* op = "lightning_indexer_decode";
@@ -947,6 +958,25 @@ int pto_lightning_indexer_launch(const PtoTensorDesc* tensors, uint32_t n_tensor
     if (e != hipSuccess) return fail(PTO_ERR_HIP, "%s: HIP launch failed: %s", op, hipGetErrorString(e));
     return PTO_OK;
 }
+
+#define PTO_EXPORT_LAUNCH(op, ParamsT)                                                                                \
+    int pto_##op##_launch(const PtoTensorDesc* tensors, uint32_t n_tensors, const ParamsT* params, void* workspace,  \
+                          uint64_t workspace_bytes, void* hip_stream, int sync)                                      \
+    {                                                                                                                 \
+        return finish_launch(#op, op##_launch_async(tensors, n_tensors, params, workspace, workspace_bytes, hip_stream), \
+                             hip_stream, sync);                                                                       \
+    }
+PTO_EXPORT_LAUNCH(mla_indexer_prolog_quant, PtoMlaIndexerPrologParams)
+PTO_EXPORT_LAUNCH(mla_prolog_quant, PtoMlaPrologParams)
+PTO_EXPORT_LAUNCH(indexer_prolog, PtoIndexerPrologParams)
+PTO_EXPORT_LAUNCH(attention_pre_quant, PtoAttentionPreQuantParams)
+PTO_EXPORT_LAUNCH(gqa_decode, PtoGqaParams)
+PTO_EXPORT_LAUNCH(paged_gather, PtoPagedGatherParams)
+PTO_EXPORT_LAUNCH(select_experts, PtoSelectExpertsParams)
+PTO_EXPORT_LAUNCH(sfa_quant, PtoSfaParams)
+PTO_EXPORT_LAUNCH(sfa_antiquant, PtoSfaParams)
+PTO_EXPORT_LAUNCH(lightning_indexer, PtoIndexerParams)
+#undef PTO_EXPORT_LAUNCH
 
 int pto_kernel_timing_enable(int on)
 {
@@ -983,6 +1013,6 @@ const char* pto_kernel_name(int kernel_id)
 
 const char* pto_last_error(void) { return g_last_error.c_str(); }
 
-int pto_abi_version(void) { return 1; }
+int pto_abi_version(void) { return 2; }
 
 } // extern "C"

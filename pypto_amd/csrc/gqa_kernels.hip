@@ -278,6 +278,13 @@ __global__ __launch_bounds__(128) void gqa_combine_kernel(GqaArgs a)
     *reinterpret_cast<u32x2*>(static_cast<uint16_t*>(a.out) + head_row * GD + d0) = pk;
 }
 
+// attn_res <- 0 (cache without pages)
+__global__ void gqa_zero_kernel(uint32_t* out, int64_t n_words)
+{
+    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n_words) out[i] = 0u;
+}
+
 } // namespace
 
 void gqa_pick_chunk(int max_ctx, int forced_chunk, int* chunk, int* nsplit)
@@ -301,6 +308,12 @@ hipError_t gqa_launch(const GqaArgs& a, hipStream_t stream)
 {
     const int64_t t = (int64_t)a.b * a.s1;
     if (t == 0 || a.nq == 0) return hipSuccess;
+    if (a.n_blocks == 0) { // a cache without pages holds no token: every output row is zero (and no kernel reads the cache)
+        const int64_t words = t * a.nq * 128 / 2;
+        hipLaunchKernelGGL(gqa_zero_kernel, dim3((unsigned)((words + 255) / 256)), dim3(256), 0, stream,
+                           static_cast<uint32_t*>(a.out), words);
+        return hipGetLastError();
+    }
     {
         ScopedKernelTimer timer(KID_GQA_DECODE, stream);
         hipLaunchKernelGGL(gqa_decode_kernel, dim3(a.nsplit, a.nkv * a.hsub, (unsigned)t), dim3(256), 0, stream, a);

@@ -58,7 +58,7 @@ __global__ __launch_bounds__(256) void indexer_score_kernel(IndexerArgs a)
     const int l16 = lane & 15, g = lane >> 4;
     const int bi = blockIdx.y;
     const int sgrp = blockIdx.z; // group of S1 consecutive query tokens of the sequence
-    const int L = a.act_seq[bi];
+    const int L = min(a.act_seq[bi], a.max_ctx); // keys past the page table's reach do not exist
     if (blockIdx.x * (CHUNK * PASSES) >= L) return;
     const int row0 = bi * a.s1 + sgrp * S1;
 
@@ -210,7 +210,7 @@ __global__ __launch_bounds__(256, S1 == 1 ? 3 : 2) void indexer_score_paged_kern
         const int32_t* bt = a.block_table + (int64_t)bi * a.bt_stride;
         pg_mine = bt[min(mytok / bs, a.bt_stride - 1)];
         pg_first = bt[0];
-        L = a.act_seq[bi];
+        L = min(a.act_seq[bi], a.max_ctx); // keys past the page table's reach do not exist
     };
     fetch();
     if (listed) {
@@ -420,7 +420,7 @@ __device__ __forceinline__ uint32_t block_suffix_sum(uint32_t v, uint32_t* tmp)
 // first ones of the launch order and spread evenly over the CUs (when every sequence fills its spans the list is the
 // identity and changes nothing).  256 lanes per workgroup.
 __global__ __launch_bounds__(256) void indexer_zero_kernel(uint32_t* p, int n, const int32_t* act_seq, int b, int pchunks,
-                                                           uint32_t* span_list)
+                                                           int max_ctx, uint32_t* span_list)
 {
     const int i = blockIdx.x * blockDim.x + threadIdx.x;
     if (i < n) p[i] = 0u;
@@ -433,7 +433,7 @@ __global__ __launch_bounds__(256) void indexer_zero_kernel(uint32_t* p, int n, c
         const int seq = base + tid;
         uint32_t cnt = 0;
         if (seq < b) {
-            const int L = act_seq[seq];
+            const int L = min(act_seq[seq], max_ctx);
             cnt = L > 0 ? (uint32_t)min((L + CHUNK * PPASSES - 1) / (CHUNK * PPASSES), pchunks) : 0u;
         }
         const uint32_t suffix = block_suffix_sum<4>(cnt, tmp); // sum over lanes tid .. 255
@@ -447,11 +447,12 @@ __global__ __launch_bounds__(256) void indexer_zero_kernel(uint32_t* p, int n, c
     if (tid == 0) span_list[0] = base_off;
 }
 
-// Valid length of query token `row`'s score row.
-__device__ __forceinline__ int row_length(const int32_t* act_seq, int row, int s1, int cap)
+// Valid length of query token `row`'s score row: the sequence's length, cut to what the page table can address
+// (the score kernels write no score beyond that), less the query tokens that come after this one.
+__device__ __forceinline__ int row_length(const int32_t* act_seq, int row, int s1, int max_ctx)
 {
     const int bi = row / s1, si = row - bi * s1;
-    return min(max(act_seq[bi] - (s1 - 1 - si), 0), cap);
+    return max(min(act_seq[bi], max_ctx) - (s1 - 1 - si), 0);
 }
 
 // grid (chunks of SEL_CHUNK scores, query tokens), 256 lanes
@@ -470,7 +471,7 @@ __global__ __launch_bounds__(256) void indexer_select_kernel(IndexerArgs a)
     f32x4 v[4];
 #pragma unroll
     for (int j = 0; j < 4; ++j) v[j] = *reinterpret_cast<const f32x4*>(x + min(i_begin + 4 * (j * 256 + tid), a.score_stride - 4));
-    const int n = row_length(a.act_seq, row, a.s1, a.score_stride);
+    const int n = row_length(a.act_seq, row, a.s1, a.max_ctx);
     if (i_begin >= n) return;
     if (tid == 0) s_bin = 0xffffffffu; // n <= k: no threshold bin, everything is a winner
 
@@ -700,7 +701,7 @@ __global__ __launch_bounds__(1024) void indexer_topk_kernel(IndexerArgs a)
     static_assert(MAX_K == 2048 && TIE_CAP >= 2048, "two winners and two early ties per lane");
     const uint64_t w0 = wsrc[tid], w1 = wsrc[tid + 1024];
     const uint64_t t0 = tsrc[tid], t1 = tsrc[tid + 1024];
-    const int n = row_length(a.act_seq, row, a.s1, a.score_stride);
+    const int n = row_length(a.act_seq, row, a.s1, a.max_ctx);
     const int k = a.k;
     const uint32_t n_gt = min(a.counters[(int64_t)row * 4], (uint32_t)MAX_K);
     const uint32_t n_tie = a.counters[(int64_t)row * 4 + 1];
@@ -779,7 +780,7 @@ hipError_t indexer_launch(const IndexerArgs& a, hipStream_t stream)
     const int t = a.b * a.s1;
     if (t == 0) return hipSuccess;
     const int max_ctx = a.bt_stride * a.block_size;
-    if (max_ctx == 0) { // a page table without columns: no key can be addressed, every slot is -1
+    if (max_ctx == 0 || a.n_blocks == 0) { // a page table without columns, or a cache without pages: no key exists, every slot is -1
         const int n = t * a.k;
         hipLaunchKernelGGL(indexer_fill_kernel, dim3((n + 255) / 256), dim3(256), 0, stream, a.topk_res, n, -1);
         return hipGetLastError();
@@ -788,10 +789,11 @@ hipError_t indexer_launch(const IndexerArgs& a, hipStream_t stream)
     const int pchunks = (max_ctx + CHUNK * PPASSES - 1) / (CHUNK * PPASSES);
     const int nzero = t * (NBINS + 4);
     IndexerArgs args = a;
+    args.max_ctx = max_ctx;
     const bool paged = a.block_size % 128 == 0;
     if (!paged || (int64_t)a.b * pchunks > SPAN_LIST_CAP || pchunks > 1024) args.span_list = nullptr;
     hipLaunchKernelGGL(indexer_zero_kernel, dim3((nzero + 255) / 256), dim3(256), 0, stream, a.hist, nzero, a.act_seq, a.b,
-                       pchunks, args.span_list);
+                       pchunks, max_ctx, args.span_list);
     {
         ScopedKernelTimer tm(KID_INDEXER_SCORE, stream);
         const bool pow2 = (a.block_size & (a.block_size - 1)) == 0;
@@ -802,21 +804,21 @@ hipError_t indexer_launch(const IndexerArgs& a, hipStream_t stream)
                 hipLaunchKernelGGL(indexer_score_paged_kernel<1>, dim3(pchunks, a.b, a.s1), dim3(256), 0, stream, args);
         } else if (a.s1 % 2 == 0) {
             auto kern = pow2 ? indexer_score_kernel<2, true> : indexer_score_kernel<2, false>;
-            hipLaunchKernelGGL(kern, dim3(chunks, a.b, a.s1 / 2), dim3(256), 0, stream, a);
+            hipLaunchKernelGGL(kern, dim3(chunks, a.b, a.s1 / 2), dim3(256), 0, stream, args);
         } else {
             auto kern = pow2 ? indexer_score_kernel<1, true> : indexer_score_kernel<1, false>;
-            hipLaunchKernelGGL(kern, dim3(chunks, a.b, a.s1), dim3(256), 0, stream, a);
+            hipLaunchKernelGGL(kern, dim3(chunks, a.b, a.s1), dim3(256), 0, stream, args);
         }
     }
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) return e;
     {
         ScopedKernelTimer tm(KID_INDEXER_SELECT, stream);
-        hipLaunchKernelGGL(indexer_select_kernel, dim3((max_ctx + SEL_CHUNK - 1) / SEL_CHUNK, t), dim3(256), 0, stream, a);
+        hipLaunchKernelGGL(indexer_select_kernel, dim3((max_ctx + SEL_CHUNK - 1) / SEL_CHUNK, t), dim3(256), 0, stream, args);
     }
     {
         ScopedKernelTimer tm(KID_INDEXER_TOPK, stream);
-        hipLaunchKernelGGL(indexer_topk_kernel, dim3(t), dim3(1024), 0, stream, a);
+        hipLaunchKernelGGL(indexer_topk_kernel, dim3(t), dim3(1024), 0, stream, args);
     }
     return hipGetLastError();
 }

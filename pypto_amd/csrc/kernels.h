@@ -52,6 +52,7 @@ struct IndexerArgs {
                                  // that holds keys; nullptr when the grid is too large for the list
     int64_t n_blocks;
     int32_t b, s1, nh, block_size, bt_stride, k, score_stride;
+    int32_t max_ctx; // set by indexer_launch: bt_stride * block_size, the longest sequence the page table can address
 };
 
 constexpr int SPAN_LIST_CAP = 16384;

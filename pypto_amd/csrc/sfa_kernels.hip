@@ -9,21 +9,22 @@
 //   P~ = exp(S - m) rounded to bf16 un-normalised, l summed in fp32 from the unrounded values
 //   O = (sum P~ V) / l, one rounding to bf16
 //
-// Work decomposition.  One workgroup (4 wavefronts) owns one (query token, KV split, group of 64 heads): it
-// walks its share of the token's top-k list in tiles of 32 selected cache rows.  Per tile all 256 lanes
-// gather the rows (8-byte loads, a wavefront covers the 512 int8 of one row per instruction), dequantise in
-// registers and store the tile row-major to LDS (16-byte chunks XOR-swizzled with the row, no padding).
-// Wavefronts pair up on 32 heads: wave (hg, kh) holds the Q columns of the k-steps with parity kh (B operand
-// of v_mfma_f32_32x32x16_bf16, 72 registers), computes its half of S^T = K Q^T, swaps the fp32 partial with
-// its partner through LDS, and both run the same softmax (one head per lane: row statistics are in-lane
-// reductions plus one cross-half exchange).  The rounded P~ registers are directly the B operand of
-// O^T = V^T P~, of which wave kh accumulates the 32-column blocks of parity kh (128 accumulator registers).
-// The V^T operand is read from the same row-major tile with ds_read_b64_tr_b16 (LDS transpose read: a 16-lane
-// group fetches 4 rows x 16 columns and each lane receives 4 rows of one column).  The LDS tile is double
-// buffered: tile i+1 is dequantised while tile i is in the matrix cores.  64 heads per workgroup (not 128)
-// keeps Q + O at 200 of the 512 registers per lane, which leaves room to overlap loads, dequant and MFMA.
+// Work decomposition.  One workgroup of eight wavefronts owns one (query token, KV split, group of 128 heads) and
+// walks its share of the token's top-k list in tiles of 32 selected cache rows; every gathered row is dequantised
+// once for all 128 heads.  The dequantised tile sits row-major in LDS (16-byte chunks XOR-swizzled with the row),
+// double buffered, and serves as K (row reads) and as V (transposing reads, ds_read_b64_tr_b16).  All eight
+// wavefronts issue MFMAs (v_mfma_f32_32x32x16_bf16), two per SIMD, and each has two roles:
+//   * scores: wave (hg, kh) computes S^T = K Q^T for the 32 heads of group hg over the k-steps of parity kh; its
+//     Q slice is the B operand, resident in registers but for a few k-steps parked in LDS;
+//   * values: wave (hh, dq) accumulates O^T = V^T P~ for the 64 heads of half hh and 128 of the 512 value
+//     columns (128 accumulator registers); every V^T fragment read from LDS feeds two MFMAs.
+// Between the two, per tile: the kh = 1 wave of a pair hands its partial S to the kh = 0 wave through LDS; the
+// kh = 0 wave runs the online softmax (one head per lane) and leaves P~ (bf16, already in B-operand order), the
+// rescale factors and a flag in LDS for the value role; meanwhile the kh = 1 waves - the producers - dequantise
+// the next tile out of the registers its gather landed in, store it to the other LDS stage and issue the
+// gather of the tile after.  Two workgroup barriers per tile.
 //
-// KV splits write un-normalised fp32 partial outputs plus (m, l); sfa_combine_kernel merges them.
+// KV splits write their output normalised by their own sum as fp16 plus (m, l); sfa_combine_kernel merges them.
 #include "common.h"
 #include "kernels.h"
 #include "timing.h"
@@ -38,19 +39,38 @@ constexpr int KSTEPS = (DN + DR) / 16; // 36 MFMA k-steps for S, 18 per wave of 
 constexpr int KROW = (DN + DR) * 2;    // 1152 bytes per tile row = 72 chunks of 16 bytes
 constexpr int STAGE = T * KROW;        // 36864
 constexpr int MAX_SPLIT_TOKENS = 2048; // largest share of a top-k list one workgroup may own
-constexpr int NREG_KSTEPS = 12;        // of a wave's 18 k-steps of Q, these stay in registers ...
-constexpr int NPARK = KSTEPS / 2 - NREG_KSTEPS; // ... and these are parked in LDS (16 bytes per lane each)
-// LDS layout: two tile stages | S exchange | parked Q | per-split arrays sized by SfaArgs::split_cap
-// (validity words, rows) | this sequence's page table (when it fits)
+constexpr int HEADS_PER_WG = 128;
+// of a wave's 18 k-steps of Q, NREG stay in registers and the others are parked in LDS (16 bytes per lane each);
+// the producers hold a gathered tile in registers as well and keep one k-step fewer
+#ifndef NREG_SM_V
+#define NREG_SM_V 12
+#define NREG_PR_V 12
+#define NR_PR_V 5
+#define S_AHEAD_V 4
+#define PV_AHEAD_V 2
+#endif
+constexpr int NREG_SM = NREG_SM_V, NREG_PR = NREG_PR_V;
+// of the 8 tile rows a pair of waves produces, the KH = 1 wave takes NR_PR and the softmax wave the others
+constexpr int NR_PR = NR_PR_V;
+constexpr int NPARK_SM = KSTEPS / 2 - NREG_SM, NPARK_PR = KSTEPS / 2 - NREG_PR;
+// LDS layout: two tile stages | partial S, 4 KB per head group | P~, 2 KB per head group | rescale factors [4][32],
+// row sums [128], flags [4] | parked Q | per-split arrays sized by SfaArgs::split_cap (validity words, rows) |
+// this sequence's page table (when it fits)
 constexpr int XBUF_OFF = 2 * STAGE;
-constexpr int QPARK_OFF = XBUF_OFF + 4 * 4096;
-constexpr int SPLIT_OFF = QPARK_OFF + 4 * NPARK * 1024; // 114688
+constexpr int PBUF_OFF = XBUF_OFF + 4 * 4096;
+constexpr int ALPHA_OFF = PBUF_OFF + 4 * 2048;
+constexpr int LSUM_OFF = ALPHA_OFF + 4 * 32 * 4;
+constexpr int FLAG_OFF = LSUM_OFF + HEADS_PER_WG * 4;
+constexpr int QPARK_OFF = FLAG_OFF + 16;
+constexpr int SPLIT_OFF = QPARK_OFF + 4 * (NPARK_SM + NPARK_PR) * 1024;
 constexpr int LDS_LIMIT = 160 * 1024;
-constexpr int OUT_ROW = DN * 4;  // epilogue staging: 64 heads x 512 fp32, reusing the front of LDS
+constexpr int OUT_ROW = DN * 4;  // epilogue staging: 64 heads x 512 fp32 per pass, reusing the front of LDS
+constexpr int OUT_HEADS = 64;
 __host__ __device__ constexpr int tmask_bytes(int cap) { return (cap / T + 2) * 4; }
 __host__ __device__ constexpr int split_bytes(int cap) { return tmask_bytes(cap) + cap * 4; }
-static_assert(64 * OUT_ROW <= LDS_LIMIT, "epilogue staging must fit");
-constexpr int HEADS_PER_WG = 64;
+static_assert(OUT_HEADS * OUT_ROW <= LDS_LIMIT, "epilogue staging must fit");
+static_assert(QPARK_OFF % 16 == 0 && SPLIT_OFF % 16 == 0, "16-byte LDS accesses");
+
 
 typedef short s16x4 __attribute__((ext_vector_type(4)));
 typedef _Float16 f16x4 __attribute__((ext_vector_type(4)));
@@ -65,47 +85,60 @@ __device__ __forceinline__ s16x4 lds_read_tr(uint8_t* p) { return __builtin_amdg
 // 4 consecutive rows of a transpose read both land on distinct banks
 __device__ __forceinline__ int swz(int t) { return ((t & 3) << 1) | ((t >> 2) & 1); }
 
-template <bool QUANT>
+// A wavefront's share of one gathered tile, in registers: NR of the tile's 32 rows (this lane's 8 columns of each), 8
+// bytes of the tile's rope columns, and one of the share's 4 NR dequantisation scales.  The two waves of a pair (same
+// head group hg) share rows 8 hg .. 8 hg + 7: the first NR_PR go to the KH = 1 wave, the others to the softmax wave.
+template <bool QUANT, int NR>
 struct RawTile;
-template <>
-struct RawTile<true> {
-    u32x2 nope[8]; // 8 rows x 8 int8 (this lane's 8 columns)
-    float sc[8];   // the rows' dequant scales for this lane's column group
-    u32x4 rope;
-    uint32_t absent;
+template <int NR>
+struct RawTile<true, NR> {
+    u32x2 nope[NR]; // NR rows x 8 int8
+    u32x2 rope;     // row tid/16, bytes 8 (tid%16) ..
+    float sc;       // lanes 0 .. 4 NR - 1: scale of (row lane/4 of the share, column group lane%4)
 };
-template <>
-struct RawTile<false> {
-    u32x4 nope[8]; // 8 rows x 8 bf16
-    u32x4 rope;
-    uint32_t absent;
+template <int NR>
+struct RawTile<false, NR> {
+    u32x4 nope[NR]; // NR rows x 8 bf16
+    u32x2 rope;
 };
 
-// Lane (wave w, lane l) fetches columns [8l, 8l+8) of tile rows 8w .. 8w+7 and one 16-byte piece of a rope row.
-// rows[] holds valid cache rows only (absent entries point at row 0); the tile's validity word says which
-// rows are absent, and their data is zeroed when it is consumed (dequant_store), so that no load has to be
-// waited for here.
-template <bool QUANT>
-__device__ __forceinline__ void load_raw(RawTile<QUANT>& r, const SfaArgs& a, const int* rows, const uint32_t* tmask,
-                                         int tile, int wave, int lane, int tid)
+// Byte offset `row * stride` of a wave-uniform row, pinned in scalar registers so that the load that follows takes a
+// scalar base and the lane's 32-bit offset (no 64-bit vector arithmetic per row).  An offset, not an address: the
+// pointer it is added to keeps its address space, and the load stays a global one.
+__device__ __forceinline__ uint64_t row_offset(uint32_t row, uint32_t stride)
 {
-    // the 8 rows are the same for every lane of the wavefront: two 16-byte LDS reads, then scalar address arithmetic
-    // (the loads take a scalar base and the lane's column offset)
-    const u32x4 ra = *reinterpret_cast<const u32x4*>(rows + tile * T + 8 * wave);
-    const u32x4 rb = *reinterpret_cast<const u32x4*>(rows + tile * T + 8 * wave + 4);
+    const uint64_t p = (uint64_t)row * stride;
+    uint32_t lo = (uint32_t)p, hi = (uint32_t)(p >> 32);
+    asm volatile("" : "+s"(lo), "+s"(hi));
+    return ((uint64_t)hi << 32) | lo;
+}
+
+// rows[] holds valid cache rows only (absent entries point at row 0); the tile's validity word says which rows are
+// absent, and their data is zeroed when it is consumed, so that no load depends on it.  All loads are unconditional.
+// The share is rows pair0 + E0 .. pair0 + E0 + NR - 1 of the tile, pair0 a multiple of 8.
+template <bool QUANT, int NR, int E0>
+__device__ __forceinline__ void load_raw(RawTile<QUANT, NR>& r, const SfaArgs& a, const int* rows, int tile, int pair0,
+                                         int lane, int tid)
+{
+    // the pair's eight rows are the same for every lane: two 16-byte LDS reads, then scalar address arithmetic
+    const u32x4 ra = *reinterpret_cast<const u32x4*>(rows + tile * T + pair0);
+    const u32x4 rb = *reinterpret_cast<const u32x4*>(rows + tile * T + pair0 + 4);
 #pragma unroll
-    for (int e = 0; e < 8; ++e) {
-        const uint32_t row = __builtin_amdgcn_readfirstlane(e < 4 ? ra[e & 3] : rb[e & 3]);
-        if constexpr (QUANT) {
-            r.nope[e] = *reinterpret_cast<const u32x2*>(a.kn + (uint64_t)row * a.kn_stride + lane * 8);
-            r.sc[e] = *reinterpret_cast<const float*>(a.ks + (uint64_t)row * a.ks_stride + (lane >> 4) * 4);
-        } else
-            r.nope[e] = *reinterpret_cast<const u32x4*>(a.kn + (uint64_t)row * a.kn_stride + lane * 16);
+    for (int e = 0; e < NR; ++e) {
+        const uint32_t row = __builtin_amdgcn_readfirstlane(E0 + e < 4 ? ra[(E0 + e) & 3] : rb[(E0 + e) & 3]);
+        const uint8_t* rp = a.kn + row_offset(row, a.kn_stride);
+        if constexpr (QUANT)
+            r.nope[e] = *reinterpret_cast<const u32x2*>(rp + lane * 8);
+        else
+            r.nope[e] = *reinterpret_cast<const u32x4*>(rp + lane * 16);
     }
-    const uint32_t row = (uint32_t)rows[tile * T + (tid >> 3)];
-    r.rope = *reinterpret_cast<const u32x4*>(a.kr + (uint64_t)row * a.kr_stride + (tid & 7) * 16);
-    const uint32_t present = tmask[tile];
-    r.absent = ((~present >> (8 * wave)) & 0xffu) | (((~present >> (tid >> 3)) & 1u) << 8);
+    const uint32_t row = (uint32_t)rows[tile * T + (tid >> 4)];
+    r.rope = *reinterpret_cast<const u32x2*>(a.kr + (uint64_t)row * a.kr_stride + (tid & 15) * 8);
+    if constexpr (QUANT) {
+        const int l = lane < 4 * NR ? lane : 0;
+        const uint32_t srow = (uint32_t)rows[tile * T + pair0 + E0 + (l >> 2)];
+        r.sc = *reinterpret_cast<const float*>(a.ks + (uint64_t)srow * a.ks_stride + (l & 3) * 4);
+    }
 }
 
 // int8 -> fp32 -> * scale with one conversion and one fma per element: byte k of w holds x + 128 (the caller
@@ -116,41 +149,40 @@ __device__ __forceinline__ float dq(uint32_t w, int k, float s, float neg128s)
     return __builtin_fmaf((float)((w >> (8 * k)) & 0xffu), s, neg128s);
 }
 
-// Dequantise rows [E0, E1) of this lane's 8 rows x 8 columns and store them into an LDS stage; with ROPE also
-// the lane's rope piece.
-template <bool QUANT, int E0, int E1, bool ROPE>
-__device__ __forceinline__ void dequant_store(const RawTile<QUANT>& r, uint8_t* stage, int wave, int lane, int tid)
+// Dequantise the share and store it, and the lane's rope piece, into an LDS stage; `present` is the tile's validity word.
+template <bool QUANT, int NR>
+__device__ __forceinline__ void dequant_store(const RawTile<QUANT, NR>& r, uint8_t* stage, uint32_t present, int row0,
+                                              int lane, int tid)
 {
+    float sc[NR];
+    if constexpr (QUANT) {
+        // the scale of (row e, this lane's group of 128 columns) sits in lane 4e + lane/16
 #pragma unroll
-    for (int e = E0; e < E1; ++e) {
-        const int t = 8 * wave + e;
+        for (int e = 0; e < NR; ++e)
+            sc[e] = __builtin_bit_cast(float, __builtin_amdgcn_ds_bpermute(4 * (4 * e + (lane >> 4)), __builtin_bit_cast(int, r.sc)));
+    }
+#pragma unroll
+    for (int e = 0; e < NR; ++e) {
+        const int t = row0 + e;
+        const bool absent = ((present >> t) & 1u) == 0u; // an absent row is stored as zeros
         u32x4 v;
         if constexpr (QUANT) {
-            uint32_t w0 = r.nope[e][0], w1 = r.nope[e][1];
-            float s = r.sc[e];
-            // keep the unpacking here: hoisted to the load, it would wait for the load right after issuing it
-            asm volatile("" : "+v"(w0), "+v"(w1), "+v"(s));
-            s = ((r.absent >> e) & 1u) ? 0.f : s; // an absent row is stored as zeros
-            w0 ^= 0x80808080u;
-            w1 ^= 0x80808080u;
+            const uint32_t w0 = r.nope[e][0] ^ 0x80808080u, w1 = r.nope[e][1] ^ 0x80808080u;
+            const float s = absent ? 0.f : sc[e];
             const float c = -128.f * s;
             v[0] = pack_bf16x2(dq(w0, 0, s, c), dq(w0, 1, s, c));
             v[1] = pack_bf16x2(dq(w0, 2, s, c), dq(w0, 3, s, c));
             v[2] = pack_bf16x2(dq(w1, 0, s, c), dq(w1, 1, s, c));
             v[3] = pack_bf16x2(dq(w1, 2, s, c), dq(w1, 3, s, c));
         } else {
-            u32x4 w = r.nope[e];
-            asm volatile("" : "+v"(w)); // as above: consume the load here, not where it was issued
-            v = ((r.absent >> e) & 1u) ? u32x4{0u, 0u, 0u, 0u} : w;
+            v = absent ? u32x4{0u, 0u, 0u, 0u} : r.nope[e];
         }
         *reinterpret_cast<u32x4*>(stage + t * KROW + ((lane ^ swz(t)) << 4)) = v;
     }
-    if constexpr (ROPE) {
-        const int t = tid >> 3;
-        u32x4 rp = r.rope;
-        asm volatile("" : "+v"(rp));
-        rp = ((r.absent >> 8) & 1u) ? u32x4{0u, 0u, 0u, 0u} : rp;
-        *reinterpret_cast<u32x4*>(stage + t * KROW + DN * 2 + (((tid & 7) ^ swz(t)) << 4)) = rp;
+    {
+        const int t = tid >> 4, piece = tid & 15;
+        const u32x2 rp = ((present >> t) & 1u) ? r.rope : u32x2{0u, 0u};
+        *reinterpret_cast<u32x2*>(stage + t * KROW + DN * 2 + (((piece >> 1) ^ swz(t)) << 4) + (piece & 1) * 8) = rp;
     }
 }
 
@@ -182,8 +214,11 @@ __device__ __forceinline__ void resolve_split(const SfaArgs& a, int bi, int tq, 
         const int idx = my_idx[j];
         int row = -1;
         if (idx >= 0 && idx < max_logical) {
-            const int page = bt_cached ? bt_lds[idx / a.block_size]
-                                       : a.block_table[(int64_t)bi * a.bt_stride + idx / a.block_size];
+            int page; // (two loads under a branch, not one load from a selected pointer: that would be a generic-address load)
+            if (bt_cached)
+                page = bt_lds[idx / a.block_size];
+            else
+                page = a.block_table[(int64_t)bi * a.bt_stride + idx / a.block_size];
             const int64_t r = (int64_t)page * a.block_size + idx % a.block_size;
             if (page >= 0 && r < a.n_rows) row = (int)r;
         }
@@ -197,6 +232,319 @@ __device__ __forceinline__ void resolve_split(const SfaArgs& a, int bi, int tq, 
     __syncthreads(); // rows[] / tmask[] ready
 }
 
+// Half of S^T[token, head] = K[token, :] . Q[head, :] for one wave: the k-steps 2*i + kh, i = 0..17.  One accumulation
+// chain; the K fragments (and the parked Q fragments) are read AHEAD k-steps before the MFMA that uses them.
+template <int NREG>
+__device__ __forceinline__ void s_partial(f32x16& s, const uint8_t* stage, const uint32_t (&s_off)[2], const bf16x8 (&q)[NREG],
+                                          const uint8_t* qpark)
+{
+    constexpr int AHEAD = S_AHEAD_V, N = KSTEPS / 2;
+    static_assert(NREG >= AHEAD && NREG <= N, "the first reads are of k-steps whose Q fragment is in registers");
+#pragma unroll
+    for (int r = 0; r < 16; ++r) s[r] = 0.f;
+    bf16x8 kf[N], qp[N];
+    auto fetch = [&](int i) {
+        kf[i] = *reinterpret_cast<const bf16x8*>(stage + s_off[i & 1] + (i >> 1) * 128);
+        if (i >= NREG) qp[i] = *reinterpret_cast<const bf16x8*>(qpark + (i - NREG) * 1024);
+    };
+#pragma unroll
+    for (int i = 0; i < AHEAD; ++i) fetch(i);
+#pragma unroll
+    for (int i = 0; i < N; ++i) {
+        if (i + AHEAD < N) fetch(i + AHEAD);
+        const bf16x8 qi = i < NREG ? q[i < NREG ? i : 0] : qp[i];
+        s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf[i], qi, s, 0, 0, 0);
+    }
+    // issue order: AHEAD fetches, then (MFMA, fetch) pairs, then the last MFMAs; a fetch is one LDS read for a
+    // k-step whose Q fragment is in registers and two for a parked one
+    __builtin_amdgcn_sched_group_barrier(0x100, AHEAD, 0);
+#pragma unroll
+    for (int i = 0; i < NREG - AHEAD; ++i) {
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+        __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+    }
+#pragma unroll
+    for (int i = NREG - AHEAD; i < N - AHEAD; ++i) {
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+        __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
+    }
+    __builtin_amdgcn_sched_group_barrier(0x008, AHEAD, 0);
+}
+
+// The body of one wavefront.  KH = 0: the softmax wave of its pair; KH = 1: the wave that hands its partial S over.
+template <bool QUANT, int KH>
+__device__ __forceinline__ void sfa_wave(const SfaArgs& a, uint8_t* smem, const uint32_t* tmask, const int* rows, int tq,
+                                         int sp, int hz, int ntiles, int tid)
+{
+    constexpr int NREG = KH ? NREG_PR : NREG_SM;
+    const int lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6); // (scalar: what follows from it is too)
+    const int l32 = lane & 31, hl = lane >> 5;
+    const int hg = wave & 3;              // scores role: heads [32 hg, 32 hg + 32) of the workgroup's 128, k-steps of parity KH
+    const int hh = wave & 1, dq = wave >> 1; // values role: heads [64 hh, 64 hh + 64), value columns [128 dq, 128 dq + 128)
+    const int last = ntiles - 1;
+    const int head0 = hz * HEADS_PER_WG;
+    const int head = head0 + hg * 32 + l32;
+    const bool head_ok = head < a.nq;
+    const bool s_active = head0 + hg * 32 < a.nq;
+    const bool pv_active = head0 + hh * 64 < a.nq;
+
+    // Production: this wave's share of every tile (rows row0 .. row0 + NR - 1 and 8 bytes of the rope columns).  The
+    // share of tile i+1 is dequantised out of `raw` and stored between the two MFMA phases of tile i, and `raw` is
+    // refilled at once with the share of tile i+2 (past the end the last tile is loaded again and stored into a stage
+    // nobody reads: every path has the same loads in flight).
+    constexpr int NR = KH ? NR_PR : 8 - NR_PR, E0 = KH ? 0 : NR_PR;
+    const int pair0 = 8 * hg, row0 = pair0 + E0;
+    RawTile<QUANT, NR> raw;
+    if (ntiles > 0) load_raw<QUANT, NR, E0>(raw, a, rows, 0, pair0, lane, tid);
+
+    // this lane's query head and its Q slice: k-steps 2*i + KH, i = 0..17 (0..15 nope, 16..17 rope); B operand
+    // layout: head = column, 8 consecutive k per half-wave.  Lanes past the last head reuse head 0's rows,
+    // their results are never written.
+    bf16x8 q[NREG];
+    uint8_t* qpark = smem + QPARK_OFF + (KH ? 4 * NPARK_SM * 1024 + hg * (NPARK_PR * 1024) : hg * (NPARK_SM * 1024)) + lane * 16;
+    {
+        const int64_t qrow = (int64_t)tq * a.nq + (head_ok ? head : 0);
+        const uint32_t f = a.softmax_scale < 0.f ? 0x80008000u : 0u;
+        const u32x4 qflip = {f, f, f, f};
+        const __bf16* qn = reinterpret_cast<const __bf16*>(a.q_nope) + qrow * DN + KH * 16 + hl * 8;
+        const __bf16* qr = reinterpret_cast<const __bf16*>(a.q_rope) + qrow * DR + KH * 16 + hl * 8;
+#pragma unroll
+        for (int i = 0; i < KSTEPS / 2; ++i) {
+            // (a negative softmax_scale is applied as its magnitude to the negated query: the row statistics below are
+            // taken on the raw scores, which needs a factor that commutes with max)
+            u32x4 w = *reinterpret_cast<const u32x4*>(i < DN / 32 ? qn + i * 32 : qr + (i - DN / 32) * 32);
+            w ^= qflip;
+            const bf16x8 v = __builtin_bit_cast(bf16x8, w);
+            if (i < NREG)
+                q[i < NREG ? i : 0] = v;
+            else
+                *reinterpret_cast<bf16x8*>(qpark + (i - NREG) * 1024) = v;
+        }
+    }
+    if (ntiles > 0) {
+        dequant_store<QUANT, NR>(raw, smem, __builtin_amdgcn_readfirstlane(tmask[0]), row0, lane, tid);
+        load_raw<QUANT, NR, E0>(raw, a, rows, min(1, last), pair0, lane, tid);
+    }
+
+    f32x16 o[4][2]; // O^T blocks [value columns 32 (4 dq + i) ..][heads 64 hh + 32 hb ..]
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int hb = 0; hb < 2; ++hb)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) o[i][hb][r] = 0.f;
+    float m_run = -INFINITY; // running max of S * scale * log2(e)          (softmax wave)
+    float l_run = 0.f;       // this lane's share of sum exp                (softmax wave)
+    const float c_log2 = fabsf(a.softmax_scale) * 1.4426950408889634f;
+
+    // S operand (b128): row l32, chunk 2*ks + hl with ks = 2*i + KH -> chunk 4*i + 2*KH + hl; swizzled offsets
+    // for even and odd i
+    uint32_t s_off[2];
+    {
+        const int sw = swz(l32), c = 2 * KH + hl;
+        s_off[0] = l32 * KROW + ((c ^ sw) << 4);
+        s_off[1] = l32 * KROW + (((4 + c) ^ sw) << 4);
+    }
+    // V^T operand (transpose read): lane jj of 16-lane group G points at row 4*hl + jj/4 (+ 16*j + 8*h2), columns
+    // 32*db + 16*(G&1) + 4*(jj&3) with db = 4*dq + i -> chunk 16*dq + 4*i + 2*(G&1) + (jj&3)/2; swizzled offsets for even
+    // and odd i
+    uint32_t v_off[2];
+    {
+        const int jj = lane & 15, mh = (lane >> 4) & 1;
+        const int cl = 2 * mh + ((jj & 3) >> 1);
+        const int sw = ((jj >> 2) << 1) | hl;
+        const uint32_t base = (4 * hl + (jj >> 2)) * KROW + (jj & 1) * 8 + dq * 256;
+        v_off[0] = base + ((cl ^ sw) << 4);
+        v_off[1] = base + (((4 + cl) ^ sw) << 4);
+    }
+    uint8_t* xbuf = smem + XBUF_OFF + hg * 4096 + lane * 16;
+    uint8_t* pbuf = smem + PBUF_OFF + hg * 2048 + lane * 16;
+    float* alpha_lds = reinterpret_cast<float*>(smem + ALPHA_OFF);
+    uint32_t* flag_lds = reinterpret_cast<uint32_t*>(smem + FLAG_OFF);
+    if (tid < 4) flag_lds[tid] = 0u;
+    __syncthreads(); // tile 0 stored, Q parked
+
+    // Two barriers per tile: partial S handed over | P~ and the next tile ready.
+    for (int it = 0; it < ntiles; ++it) {
+        uint8_t* stage = smem + (it & 1) * STAGE;
+        const uint32_t valid = __builtin_amdgcn_readfirstlane(tmask[it]);
+        f32x16 s;
+        if (s_active) s_partial<NREG>(s, stage, s_off, q, qpark);
+        if (KH == 1 && s_active) {
+#pragma unroll
+            for (int g = 0; g < 4; ++g)
+                *reinterpret_cast<f32x4*>(xbuf + g * 1024) = f32x4{s[4 * g], s[4 * g + 1], s[4 * g + 2], s[4 * g + 3]};
+        }
+        __syncthreads(); // the partial S of the KH = 1 waves is in LDS
+        if (KH == 0 && s_active && valid != 0u) {
+#pragma unroll
+            for (int g = 0; g < 4; ++g) {
+                const f32x4 p = *reinterpret_cast<const f32x4*>(xbuf + g * 1024);
+                s[4 * g] += p[0];
+                s[4 * g + 1] += p[1];
+                s[4 * g + 2] += p[2];
+                s[4 * g + 3] += p[3];
+            }
+            // register r holds token 8*(r/4) + 4*hl + r%4 for head l32; statistics on the raw scores (the factor
+            // is not negative, so it commutes with max), exponent argument by one fma per score
+            float mx = -INFINITY;
+            if (valid != 0xffffffffu) {
+                // (the half-wave's shift first: the bit positions left are compile-time constants)
+                const uint32_t vh = valid >> (4 * hl);
+#pragma unroll
+                for (int r = 0; r < 16; ++r) s[r] = ((vh >> (8 * (r >> 2) + (r & 3))) & 1u) ? s[r] : -INFINITY;
+            }
+#pragma unroll
+            for (int r = 0; r < 16; ++r) mx = fmaxf(mx, s[r]);
+            {
+                // maximum over both halves of the wavefront without a trip through LDS: v_permlane32_swap exchanges the
+                // upper half of its first operand with the lower half of its second
+                const auto sw = __builtin_amdgcn_permlane32_swap(__builtin_bit_cast(unsigned, mx), __builtin_bit_cast(unsigned, mx), false, false);
+                mx = fmaxf(__builtin_bit_cast(float, (unsigned)sw[0]), __builtin_bit_cast(float, (unsigned)sw[1])) * c_log2;
+            }
+            // The reference exponent only follows the running maximum when it has grown by more than 2^8: until
+            // then P~ = 2^(z - m_run) may exceed 1 (by at most 2^8, no issue for bf16 or the fp32 sums), which
+            // makes the rescale of the accumulator registers a rare event.  Every P~, l and O stay relative to
+            // the same m_run, so the result is unchanged.
+            const float m_new = fmaxf(m_run, mx);
+            const bool rescale = __any(m_new > m_run + 8.f);
+            if (rescale) {
+                const float alpha = __builtin_amdgcn_exp2f(m_run - m_new); // 0 on the first tile (m_run = -inf)
+                l_run *= alpha;
+                m_run = m_new;
+                if (hl == 0) alpha_lds[hg * 32 + l32] = alpha;
+            }
+            if (lane == 0) flag_lds[hg] = rescale ? 1u : 0u;
+            uint32_t pb[8];
+#pragma unroll
+            for (int r = 0; r < 16; r += 2) {
+                const float p0 = __builtin_amdgcn_exp2f(__builtin_fmaf(s[r], c_log2, -m_run));
+                const float p1 = __builtin_amdgcn_exp2f(__builtin_fmaf(s[r + 1], c_log2, -m_run));
+                l_run += p0 + p1;
+                pb[r >> 1] = pack_bf16x2(p0, p1);
+            }
+            // P~ in the order the S^T registers hold the tokens: k-slot s of half hl in block j is token
+            // 16*j + 8*(s/4) + 4*hl + s%4 - which is also how the V^T fragments are read
+#pragma unroll
+            for (int j = 0; j < 2; ++j)
+                *reinterpret_cast<u32x4*>(pbuf + j * 1024) = u32x4{pb[4 * j], pb[4 * j + 1], pb[4 * j + 2], pb[4 * j + 3]};
+        }
+        {
+            // the next tile: out of the registers into the other stage, then the gather of the tile after
+            const int nx = min(it + 1, last);
+            dequant_store<QUANT, NR>(raw, smem + ((it + 1) & 1) * STAGE, __builtin_amdgcn_readfirstlane(tmask[nx]), row0, lane, tid);
+            load_raw<QUANT, NR, E0>(raw, a, rows, min(it + 2, last), pair0, lane, tid);
+        }
+        __syncthreads(); // P~ and the next tile are in LDS
+        if (pv_active && valid != 0u) {
+            // O^T[dim, head] += V^T[dim, token] . P~[token, head]
+#pragma unroll
+            for (int hb = 0; hb < 2; ++hb) {
+                const uint32_t f = __builtin_amdgcn_readfirstlane(flag_lds[2 * hh + hb]);
+                if (f) {
+                    const float alpha = alpha_lds[(2 * hh + hb) * 32 + l32];
+#pragma unroll
+                    for (int i = 0; i < 4; ++i)
+#pragma unroll
+                        for (int r = 0; r < 16; ++r) o[i][hb][r] *= alpha;
+                }
+            }
+            bf16x8 pf[2][2];
+#pragma unroll
+            for (int hb = 0; hb < 2; ++hb)
+#pragma unroll
+                for (int j = 0; j < 2; ++j)
+                    pf[hb][j] = *reinterpret_cast<const bf16x8*>(smem + PBUF_OFF + (2 * hh + hb) * 2048 + j * 1024 + lane * 16);
+            // 8 V^T fragments (token block j, column block i), two transpose reads each, feeding two MFMAs each;
+            // the reads run AHEAD fragments ahead
+            constexpr int AHEAD = PV_AHEAD_V;
+            s16x4 lo[8], hi[8];
+            auto vread = [&](int n) {
+                const int j = n >> 2, i = n & 3;
+                uint8_t* vp = stage + v_off[i & 1] + (16 * j) * KROW + (i >> 1) * 128;
+                lo[n] = lds_read_tr(vp);
+                hi[n] = lds_read_tr(vp + 8 * KROW);
+            };
+#pragma unroll
+            for (int n = 0; n < AHEAD; ++n) vread(n);
+#pragma unroll
+            for (int n = 0; n < 8; ++n) {
+                if (n + AHEAD < 8) vread(n + AHEAD);
+                const s16x8 both = __builtin_shufflevector(lo[n], hi[n], 0, 1, 2, 3, 4, 5, 6, 7);
+                const bf16x8 vf = __builtin_bit_cast(bf16x8, both);
+#pragma unroll
+                for (int hb = 0; hb < 2; ++hb)
+                    o[n & 3][hb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf, pf[hb][n >> 2], o[n & 3][hb], 0, 0, 0);
+            }
+        }
+    }
+
+    // Epilogue.  The softmax waves publish the row sums; then, 64 heads at a time, the O^T blocks go to LDS as
+    // [head][512] fp32 rows (everything but the split arrays is free now), 16-byte chunks XOR-swizzled with the
+    // head so that the 8 lanes of a b128 write hit distinct banks, and all 512 lanes copy the rows out.  Register r of
+    // o[i][hb] holds dim 32*(4*dq + i) + 8*(r/4) + 4*hl + r%4 of head 64*hh + 32*hb + l32.
+    float* lsum = reinterpret_cast<float*>(smem + LSUM_OFF);
+    if (KH == 0) {
+        const float l_tot = l_run + __shfl_xor(l_run, 32);
+        if (hl == 0) lsum[hg * 32 + l32] = s_active ? l_tot : 0.f;
+        if (a.nsplit > 1 && head_ok && hl == 0) {
+            const int64_t prow = ((int64_t)tq * a.nsplit + sp) * a.nq + head;
+            a.part_ml[prow * 2] = m_run;
+            a.part_ml[prow * 2 + 1] = l_tot;
+        }
+    }
+    __syncthreads();
+    float mul[2]; // splits hand over their normalised output as well
+#pragma unroll
+    for (int hb = 0; hb < 2; ++hb) {
+        const float l = lsum[(2 * hh + hb) * 32 + l32];
+        mul[hb] = l > 0.f ? 1.f / l : 0.f;
+    }
+    __syncthreads(); // the staging area covers the row sums
+#pragma unroll
+    for (int pass = 0; pass < 2; ++pass) {
+        if (hh == pass) {
+#pragma unroll
+            for (int hb = 0; hb < 2; ++hb) {
+                const int hrow = hb * 32 + l32;
+                uint8_t* orow = smem + hrow * OUT_ROW;
+#pragma unroll
+                for (int i = 0; i < 4; ++i)
+#pragma unroll
+                    for (int g = 0; g < 4; ++g) {
+                        const int c = 8 * (4 * dq + i) + 2 * g + hl;
+                        const f32x4 v = {o[i][hb][4 * g] * mul[hb], o[i][hb][4 * g + 1] * mul[hb], o[i][hb][4 * g + 2] * mul[hb],
+                                         o[i][hb][4 * g + 3] * mul[hb]};
+                        *reinterpret_cast<f32x4*>(orow + ((c ^ (hrow & 7)) << 4)) = v;
+                    }
+            }
+        }
+        __syncthreads();
+        // a wavefront writes 512 B (bf16 output or fp16 partial) of one row per instruction
+#pragma unroll 4
+        for (int id = tid; id < OUT_HEADS * (DN / 4); id += 512) {
+            const int hrow = id / (DN / 4), c = id % (DN / 4);
+            const int oh = head0 + pass * OUT_HEADS + hrow;
+            if (oh >= a.nq) continue;
+            const f32x4 v = *reinterpret_cast<const f32x4*>(smem + hrow * OUT_ROW + ((c ^ (hrow & 7)) << 4));
+            if (a.nsplit == 1) {
+                const u32x2 w = {pack_bf16x2(v[0], v[1]), pack_bf16x2(v[2], v[3])};
+                *reinterpret_cast<u32x2*>(reinterpret_cast<uint8_t*>(a.out) + (((int64_t)tq * a.nq + oh) * DN + c * 4) * 2) = w;
+            } else {
+                // a split's share, normalised by its own sum, in fp16: |value| <= max |V| and 2^-11 relative rounding, a
+                // quarter of the final bf16 rounding; half the bytes of fp32 for this kernel to write and the merge to read
+                const int64_t prow = ((int64_t)tq * a.nsplit + sp) * a.nq + oh;
+                const f16x4 hv = {(_Float16)v[0], (_Float16)v[1], (_Float16)v[2], (_Float16)v[3]};
+                *reinterpret_cast<f16x4*>(a.part_o + prow * DN + c * 4) = hv;
+            }
+        }
+        if (pass == 0) __syncthreads();
+    }
+}
+
+// grid (query token, KV split, group of 128 heads).  Workgroups go to the XCDs round-robin in launch order, so with the
+// token as the fastest grid dimension the splits of one token run on one XCD (when the token count is a multiple of 8)
+// and share its L2 for the token's queries.
 template <bool QUANT>
 __global__ __attribute__((amdgpu_flat_work_group_size(512, 512), amdgpu_waves_per_eu(2, 2))) void sfa_decode_kernel(
     SfaArgs a)
@@ -206,8 +554,8 @@ __global__ __attribute__((amdgpu_flat_work_group_size(512, 512), amdgpu_waves_pe
     int* rows = reinterpret_cast<int*>(smem + SPLIT_OFF + tmask_bytes(a.split_cap));
     int* bt_lds = reinterpret_cast<int*>(smem + SPLIT_OFF + split_bytes(a.split_cap));
 
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const int sp = blockIdx.x, tq = blockIdx.y, hz = blockIdx.z;
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int tq = blockIdx.x, sp = blockIdx.y, hz = blockIdx.z;
     const int bi = tq / a.s1, si = tq - bi * a.s1;
 
     int cur = a.act_seq[bi] - a.s1 + 1 + si;
@@ -215,280 +563,22 @@ __global__ __attribute__((amdgpu_flat_work_group_size(512, 512), amdgpu_waves_pe
     const int ntiles_all = (cur + T - 1) / T;
     const int per = (ntiles_all + a.nsplit - 1) / a.nsplit;
     const int tile0 = sp * per;
-    const int ntiles_real = max(min(ntiles_all, tile0 + per) - tile0, 0);
-    // an even number of tiles keeps the producer loop free of conditional loads (the odd one out is fully masked)
-    const int ntiles = (ntiles_real + 1) & ~1;
+    const int ntiles = max(min(ntiles_all, tile0 + per) - tile0, 0);
     const int tok0 = tile0 * T;
 
-    resolve_split<512>(a, bi, tq, tok0, cur, ntiles_real, ntiles, tmask, rows, bt_lds, tid, lane);
+    resolve_split<512>(a, bi, tq, tok0, cur, ntiles, (ntiles + 1) & ~1, tmask, rows, bt_lds, tid, lane);
 
-    // Both roles run the same barrier sequence: one before the first tile, then two per tile
-    // (partial S exchanged; tile consumed and next tile stored).
-    if (wave >= 4) {
-        // ---------------------------------------------------------------- producer wavefronts
-        // Gathered rows travel global -> registers -> LDS.  Two register tiles alternate so that the loads of
-        // a tile are issued two tiles before it is dequantised.
-        const int pw = wave - 4, ptid = tid - 256;
-        const int last = ntiles - 1;
-        RawTile<QUANT> raw0, raw1;
-        // (tile 0 is gathered and stored by the consumer wavefronts, which would otherwise idle here: the cold first
-        // gathers are slow to issue, and two sets of waves issue them side by side)
-        if (ntiles > 0) {
-            load_raw<QUANT>(raw1, a, rows, tmask, 1, pw, lane, ptid);
-            load_raw<QUANT>(raw0, a, rows, tmask, min(2, last), pw, lane, ptid);
-        }
-        __syncthreads();
-        // Every step stores one tile and issues the loads of another, unconditionally (past the end the last
-        // tile is loaded again and stored into a stage nobody reads): with a fixed number of loads in flight
-        // on every path the wait for a tile leaves the younger tile's loads outstanding.
-        // The store of the next tile is split around the consumers' mid-tile barrier: most of it runs beside the
-        // S MFMAs, the rest (and the loads of a later tile) beside softmax and PV.
-        auto produce = [&](int it, RawTile<QUANT>& next) {
-            uint8_t* dst = smem + ((it + 1) & 1) * STAGE;
-            dequant_store<QUANT, 0, 5, false>(next, dst, pw, lane, ptid);
-            __syncthreads();
-            dequant_store<QUANT, 5, 8, true>(next, dst, pw, lane, ptid);
-            load_raw<QUANT>(next, a, rows, tmask, min(it + 3, last), pw, lane, ptid);
-            __syncthreads();
-        };
-        for (int it = 0; it < ntiles; it += 2) {
-            produce(it, raw1);
-            produce(it + 1, raw0);
-        }
-    } else {
-    // -------------------------------------------------------------------- consumer wavefronts
-    const int l32 = lane & 31, hl = lane >> 5;
-    const int hg = wave >> 1, kh = wave & 1; // head group of 32 within the workgroup; k-step / dim-block parity
-
-    // this lane's query head and its Q slice: k-steps 2*i + kh, i = 0..17 (0..15 nope, 16..17 rope); B operand
-    // layout: head = column, 8 consecutive k per half-wave.  Lanes past the last head reuse head 0's rows,
-    // their results are never written.
-    const int head = hz * HEADS_PER_WG + hg * 32 + l32;
-    const bool head_ok = head < a.nq;
-    const bool wave_active = hz * HEADS_PER_WG + hg * 32 < a.nq;
-    // 12 k-steps stay in registers; the other 6 (4 nope, 2 rope) are parked in LDS and read back by the same lane
-    // every tile, which keeps the consumer inside its 256 registers.
-    bf16x8 q[NREG_KSTEPS];
-    uint8_t* qpark = smem + QPARK_OFF + wave * (NPARK * 1024) + lane * 16;
-    RawTile<QUANT> first; // tile 0: wave w takes rows 8w .. 8w + 7, as producer wave w does for the later tiles
-    if (ntiles > 0) load_raw<QUANT>(first, a, rows, tmask, 0, wave, lane, tid);
-    {
-        const int64_t qrow = (int64_t)tq * a.nq + (head_ok ? head : 0);
-        const __bf16* qn = reinterpret_cast<const __bf16*>(a.q_nope) + qrow * DN + kh * 16 + hl * 8;
-        const __bf16* qr = reinterpret_cast<const __bf16*>(a.q_rope) + qrow * DR + kh * 16 + hl * 8;
-#pragma unroll
-        for (int i = 0; i < KSTEPS / 2; ++i) {
-            const bf16x8 v = *reinterpret_cast<const bf16x8*>(i < DN / 32 ? qn + i * 32 : qr + (i - DN / 32) * 32);
-            if (i < NREG_KSTEPS)
-                q[i < NREG_KSTEPS ? i : 0] = v;
-            else
-                *reinterpret_cast<bf16x8*>(qpark + (i - NREG_KSTEPS) * 1024) = v;
-        }
-    }
-
-    f32x16 o[8]; // O^T blocks db = 2*i + kh: dims [32*db, 32*db + 32) x 32 heads
-#pragma unroll
-    for (int i = 0; i < 8; ++i)
-#pragma unroll
-        for (int r = 0; r < 16; ++r) o[i][r] = 0.f;
-    float m_run = -INFINITY; // running max of S * scale * log2(e)
-    float l_run = 0.f;       // this lane's share of sum exp
-    const float c_log2 = a.softmax_scale * 1.4426950408889634f;
-
-    // S operand (b128): row l32, chunk 2*ks + hl with ks = 2*i + kh -> chunk 4*i + 2*kh + hl; swizzled offsets
-    // for even and odd i
-    uint32_t s_off[2];
-    {
-        const int sw = swz(l32), c = 2 * kh + hl;
-        s_off[0] = l32 * KROW + ((c ^ sw) << 4);
-        s_off[1] = l32 * KROW + (((4 + c) ^ sw) << 4);
-    }
-    // V^T operand (transpose read): lane jj of 16-lane group G points at row 4*hl + jj/4 (+ 16*j + 8*h2),
-    // columns 32*db + 16*(G&1) + 4*(jj&3) with db = 2*i + kh -> chunk 8*i + 4*kh + 2*(G&1) + (jj&3)/2
-    uint32_t v_off;
-    {
-        const int jj = lane & 15, mh = (lane >> 4) & 1;
-        const int cl = 4 * kh + 2 * mh + ((jj & 3) >> 1);
-        const int sw = ((jj >> 2) << 1) | hl;
-        v_off = (4 * hl + (jj >> 2)) * KROW + (jj & 1) * 8 + ((cl ^ sw) << 4);
-    }
-    uint8_t* xmine = smem + XBUF_OFF + wave * 4096 + lane * 16;
-
-    if (ntiles > 0) dequant_store<QUANT, 0, 8, true>(first, smem, wave, lane, tid);
-    __syncthreads(); // tile 0 stored
-
-    for (int it = 0; it < ntiles; ++it) {
-        uint8_t* stage = smem + (it & 1) * STAGE;
-        const uint32_t valid = tmask[it];
-        // half of S^T[token, head] = K[token, :] . Q[head, :] (k-steps of parity kh)
-        // One accumulation chain: a second one (even / odd k-steps) saves the few cycles a dependent MFMA waits for its
-        // predecessor, but its 16 registers are worth more as two further operand reads in flight.
-        f32x16 s;
-#pragma unroll
-        for (int r = 0; r < 16; ++r) s[r] = 0.f;
-        {
-            // operand reads run AHEAD k-steps ahead of the MFMAs that use them
-            constexpr int AHEAD = 4, N = KSTEPS / 2;
-            bf16x8 kf[N], qp[N];
-            auto fetch = [&](int i) {
-                kf[i] = *reinterpret_cast<const bf16x8*>(stage + s_off[i & 1] + (i >> 1) * 128);
-                if (i >= NREG_KSTEPS) qp[i] = *reinterpret_cast<const bf16x8*>(qpark + (i - NREG_KSTEPS) * 1024);
-            };
-#pragma unroll
-            for (int i = 0; i < AHEAD; ++i) fetch(i);
-#pragma unroll
-            for (int i = 0; i < N; ++i) {
-                if (i + AHEAD < N) fetch(i + AHEAD);
-                const bf16x8 qi = i < NREG_KSTEPS ? q[i < NREG_KSTEPS ? i : 0] : qp[i];
-                s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf[i], qi, s, 0, 0, 0);
-            }
-            // issue order: AHEAD fetches, then (MFMA, fetch) pairs, then the last MFMAs; a fetch is one LDS read
-            // for a k-step whose Q fragment is in registers and two for a parked one
-            __builtin_amdgcn_sched_group_barrier(0x100, AHEAD, 0);
-#pragma unroll
-            for (int i = 0; i < NREG_KSTEPS - AHEAD; ++i) {
-                __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-                __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
-            }
-#pragma unroll
-            for (int i = NREG_KSTEPS - AHEAD; i < N - AHEAD; ++i) {
-                __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-                __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
-            }
-            __builtin_amdgcn_sched_group_barrier(0x008, AHEAD, 0);
-        }
-#pragma unroll
-        for (int g = 0; g < 4; ++g)
-            *reinterpret_cast<f32x4*>(xmine + g * 1024) = f32x4{s[4 * g], s[4 * g + 1], s[4 * g + 2], s[4 * g + 3]};
-        __syncthreads(); // partial S of both waves of each pair is in LDS
-#pragma unroll
-        for (int g = 0; g < 4; ++g) {
-            const f32x4 p = *reinterpret_cast<const f32x4*>(xmine + (kh ? -4096 : 4096) + g * 1024);
-            s[4 * g] += p[0];
-            s[4 * g + 1] += p[1];
-            s[4 * g + 2] += p[2];
-            s[4 * g + 3] += p[3];
-        }
-        if (wave_active && valid != 0u) {
-            // register r holds token 8*(r/4) + 4*hl + r%4 for head l32; statistics on the raw scores
-            // (softmax_scale > 0 commutes with max), exponent argument by one fma per score
-            float mx = -INFINITY;
-#pragma unroll
-            for (int r = 0; r < 16; ++r) {
-                if (valid != 0xffffffffu) {
-                    const int tok = 8 * (r >> 2) + 4 * hl + (r & 3);
-                    s[r] = ((valid >> tok) & 1u) ? s[r] : -INFINITY;
-                }
-                mx = fmaxf(mx, s[r]);
-            }
-            {
-                // maximum over both halves of the wavefront without a trip through LDS: v_permlane32_swap exchanges the
-                // upper half of its first operand with the lower half of its second
-                const auto sw = __builtin_amdgcn_permlane32_swap(__builtin_bit_cast(unsigned, mx), __builtin_bit_cast(unsigned, mx), false, false);
-                mx = fmaxf(__builtin_bit_cast(float, (unsigned)sw[0]), __builtin_bit_cast(float, (unsigned)sw[1])) * c_log2;
-            }
-            // The reference exponent only follows the running maximum when it has grown by more than 2^8: until
-            // then P~ = 2^(z - m_run) may exceed 1 (by at most 2^8, no issue for bf16 or the fp32 sums), which
-            // makes the rescale of the 128 accumulator registers a rare event.  Every P~, l and O stay relative to
-            // the same m_run, so the result is unchanged.
-            const float m_new = fmaxf(m_run, mx);
-            if (__any(m_new > m_run + 8.f)) {
-                const float alpha = __builtin_amdgcn_exp2f(m_run - m_new); // 0 on the first tile (m_run = -inf)
-                l_run *= alpha;
-#pragma unroll
-                for (int i = 0; i < 8; ++i)
-#pragma unroll
-                    for (int r = 0; r < 16; ++r) o[i][r] *= alpha;
-                m_run = m_new;
-            }
-            uint32_t pb[8];
-#pragma unroll
-            for (int r = 0; r < 16; r += 2) {
-                const float p0 = __builtin_amdgcn_exp2f(__builtin_fmaf(s[r], c_log2, -m_run));
-                const float p1 = __builtin_amdgcn_exp2f(__builtin_fmaf(s[r + 1], c_log2, -m_run));
-                l_run += p0 + p1;
-                pb[r >> 1] = pack_bf16x2(p0, p1);
-            }
-            // O^T[dim, head] += V^T[dim, token] . P~[token, head]; k-slot s of half hl in block j is token
-            // 16*j + 8*(s/4) + 4*hl + s%4, the order in which the S^T registers hold the tokens
-            {
-                bf16x8 pf[2];
-#pragma unroll
-                for (int j = 0; j < 2; ++j) {
-                    u32x4 pw = {pb[4 * j], pb[4 * j + 1], pb[4 * j + 2], pb[4 * j + 3]};
-                    pf[j] = __builtin_bit_cast(bf16x8, pw);
-                }
-                // 16 MFMAs (j, i); their two transpose reads each run AHEAD MFMAs ahead
-                constexpr int AHEAD = 3;
-                s16x4 lo[16], hi[16];
-                auto vread = [&](int n) {
-                    uint8_t* vp = stage + v_off + (16 * (n >> 3)) * KROW + (n & 7) * 128;
-                    lo[n] = lds_read_tr(vp);
-                    hi[n] = lds_read_tr(vp + 8 * KROW);
-                };
-#pragma unroll
-                for (int n = 0; n < AHEAD; ++n) vread(n);
-#pragma unroll
-                for (int n = 0; n < 16; ++n) {
-                    if (n + AHEAD < 16) vread(n + AHEAD);
-                    const s16x8 both = __builtin_shufflevector(lo[n], hi[n], 0, 1, 2, 3, 4, 5, 6, 7);
-                    o[n & 7] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, both), pf[n >> 3],
-                                                                       o[n & 7], 0, 0, 0);
-                }
-                __builtin_amdgcn_sched_group_barrier(0x100, 2 * AHEAD, 0);
-#pragma unroll
-                for (int n = 0; n < 16 - AHEAD; ++n) {
-                    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0); // one MFMA
-                    __builtin_amdgcn_sched_group_barrier(0x100, 2, 0); // two LDS reads
-                }
-                __builtin_amdgcn_sched_group_barrier(0x008, AHEAD, 0);
-            }
-        }
-        __syncthreads(); // tile consumed: its stage and the exchange buffer may be overwritten
-    }
-
-    // Epilogue, part 1: O^T blocks -> LDS as [head][512] fp32 rows (the tile stages are free now), 16-byte
-    // chunks XOR-swizzled with the head so that the 8 lanes of a b128 write hit distinct banks.  Register r of
-    // o[i] holds dim 32*(2*i + kh) + 8*(r/4) + 4*hl + r%4 of head l32.
-    const float l_tot = l_run + __shfl_xor(l_run, 32);
-    const float mul = l_tot > 0.f ? 1.f / l_tot : 0.f; // splits hand over their normalised output as well
-    const int hrow = hg * 32 + l32;
-    uint8_t* orow = smem + hrow * OUT_ROW;
-#pragma unroll
-    for (int i = 0; i < 8; ++i)
-#pragma unroll
-        for (int g = 0; g < 4; ++g) {
-            const int c = 8 * (2 * i + kh) + 2 * g + hl;
-            const f32x4 v = {o[i][4 * g] * mul, o[i][4 * g + 1] * mul, o[i][4 * g + 2] * mul, o[i][4 * g + 3] * mul};
-            *reinterpret_cast<f32x4*>(orow + ((c ^ (hrow & 7)) << 4)) = v;
-        }
-    if (a.nsplit > 1 && head_ok && hl == 0 && kh == 0) {
-        const int64_t prow = ((int64_t)tq * a.nsplit + sp) * a.nq + head;
-        a.part_ml[prow * 2] = m_run;
-        a.part_ml[prow * 2 + 1] = l_tot;
-    }
-    } // consumer
-    __syncthreads();
-
-    // Epilogue, part 2: all 512 lanes copy the 64 rows out, a wavefront writing 1 KB (fp32 partial) or 512 B
-    // (bf16 output) of one row per instruction.
-#pragma unroll 4
-    for (int id = tid; id < HEADS_PER_WG * (DN / 4); id += 512) {
-        const int hrow = id / (DN / 4), c = id % (DN / 4);
-        const int head = hz * HEADS_PER_WG + hrow;
-        if (head >= a.nq) continue;
-        const f32x4 v = *reinterpret_cast<const f32x4*>(smem + hrow * OUT_ROW + ((c ^ (hrow & 7)) << 4));
-        if (a.nsplit == 1) {
-            const u32x2 w = {pack_bf16x2(v[0], v[1]), pack_bf16x2(v[2], v[3])};
-            *reinterpret_cast<u32x2*>(reinterpret_cast<uint8_t*>(a.out) + (((int64_t)tq * a.nq + head) * DN + c * 4) * 2) = w;
-        } else {
-            // a split's share, normalised by its own sum, in fp16: |value| <= max |V| and 2^-11 relative rounding, a
-            // quarter of the final bf16 rounding; half the bytes of fp32 for this kernel to write and the merge to read
-            const int64_t prow = ((int64_t)tq * a.nsplit + sp) * a.nq + head;
-            const f16x4 hv = {(_Float16)v[0], (_Float16)v[1], (_Float16)v[2], (_Float16)v[3]};
-            *reinterpret_cast<f16x4*>(a.part_o + prow * DN + c * 4) = hv;
-        }
-    }
+    // Both kinds of wavefront run the same barrier sequence: one before the first tile, two per tile, the epilogue's.
+#if defined(ONLY_KH0)
+    sfa_wave<QUANT, 0>(a, smem, tmask, rows, tq, sp, hz, ntiles, tid);
+#elif defined(ONLY_KH1)
+    sfa_wave<QUANT, 1>(a, smem, tmask, rows, tq, sp, hz, ntiles, tid);
+#else
+    if (tid < 256)
+        sfa_wave<QUANT, 0>(a, smem, tmask, rows, tq, sp, hz, ntiles, tid);
+    else
+        sfa_wave<QUANT, 1>(a, smem, tmask, rows, tq, sp, hz, ntiles, tid);
+#endif
 }
 
 // attention_out <- 0 (cache without rows: every selected entry is absent)
@@ -583,7 +673,7 @@ hipError_t sfa_launch(const SfaArgs& a, hipStream_t stream)
     int smem_bytes = SPLIT_OFF + split_bytes(args.split_cap);
     args.bt_cached = smem_bytes + a.bt_stride * 4 <= LDS_LIMIT ? 1 : 0;
     if (args.bt_cached) smem_bytes += a.bt_stride * 4;
-    if (smem_bytes < HEADS_PER_WG * OUT_ROW) smem_bytes = HEADS_PER_WG * OUT_ROW; // epilogue staging
+    if (smem_bytes < OUT_HEADS * OUT_ROW) smem_bytes = OUT_HEADS * OUT_ROW; // epilogue staging
     static DeviceOnce attr_done[2];
     auto kern = a.quant ? sfa_decode_kernel<true> : sfa_decode_kernel<false>;
     {
@@ -594,7 +684,7 @@ hipError_t sfa_launch(const SfaArgs& a, hipStream_t stream)
         if (e != hipSuccess) return e;
     }
     const int hgroups = (a.nq + HEADS_PER_WG - 1) / HEADS_PER_WG;
-    dim3 grid(a.nsplit, t, hgroups);
+    dim3 grid(t, a.nsplit, hgroups);
     {
         ScopedKernelTimer tm(KID_SFA_DECODE, stream);
         hipLaunchKernelGGL(kern, grid, dim3(512), smem_bytes, stream, args);

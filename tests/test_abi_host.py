@@ -51,7 +51,7 @@ def test_every_declared_symbol_is_exported(lib):
             "pto_last_error"} <= names
     for n in names:
         assert hasattr(lib, n), f"{n} declared in the header but not exported"
-    assert lib.pto_abi_version() == 1
+    assert lib.pto_abi_version() == 2
 
 
 def test_tensor_desc_layout_matches_the_reference_abi():
@@ -75,7 +75,7 @@ def test_sfa_workspace_query(lib):
 
 def launch_rc(lib, op, specs, params, ws=None, ws_bytes=0):
     fn = getattr(lib, f"pto_{op}_launch")
-    rc = fn(descs(specs), len(specs), ctypes.byref(params), ws, ws_bytes, None)
+    rc = fn(descs(specs), len(specs), ctypes.byref(params), ws, ws_bytes, None, 0)
     return rc, lib.pto_last_error().decode()
 
 
@@ -104,7 +104,7 @@ def test_sfa_validation_codes(lib):
     rc, msg = launch_rc(lib, "sfa_quant", sfa_specs(), p)  # needs a workspace, none given
     assert rc == -5 and "workspace" in msg
     null = descs(sfa_specs()); null[3].addr = None
-    assert lib.pto_sfa_quant_launch(null, 9, ctypes.byref(p), None, 0, None) == -6
+    assert lib.pto_sfa_quant_launch(null, 9, ctypes.byref(p), None, 0, None, 0) == -6
     assert lib.pto_sfa_quant_workspace(descs(sfa_specs()), 9, None) == 0  # query reports failure as 0
 
 

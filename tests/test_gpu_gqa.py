@@ -88,7 +88,7 @@ def test_forced_chunks_agree(cuda):
         n = lib.pto_gqa_decode_workspace(d, 6, ctypes.byref(p))
         assert (n == 0) == (chunk == 4096)
         ws = torch.empty(max(n, 1), dtype=torch.uint8, device=cuda)
-        rc = lib.pto_gqa_decode_launch(d, 6, ctypes.byref(p), ws.data_ptr(), n, torch.cuda.current_stream().cuda_stream)
+        rc = lib.pto_gqa_decode_launch(d, 6, ctypes.byref(p), ws.data_ptr(), n, torch.cuda.current_stream().cuda_stream, 0)
         assert rc == 0, lib.pto_last_error()
         torch.cuda.synchronize()
         check(out.cpu(), case, f"chunk {chunk}")

@@ -144,7 +144,7 @@ def test_forced_kv_splits_agree(cuda):
         n = lib.pto_sfa_quant_workspace(d, 9, ctypes.byref(p))
         assert (n == 0) == (splits == 1)
         ws = torch.empty(max(n, 1), dtype=torch.uint8, device=dev)
-        rc = lib.pto_sfa_quant_launch(d, 9, ctypes.byref(p), ws.data_ptr(), n, torch.cuda.current_stream().cuda_stream)
+        rc = lib.pto_sfa_quant_launch(d, 9, ctypes.byref(p), ws.data_ptr(), n, torch.cuda.current_stream().cuda_stream, 0)
         assert rc == 0, lib.pto_last_error()
         torch.cuda.synchronize()
         outs.append(out.cpu())
