@@ -14,15 +14,19 @@
 // once for all 128 heads.  The dequantised tile sits row-major in LDS (16-byte chunks XOR-swizzled with the row),
 // double buffered, and serves as K (row reads) and as V (transposing reads, ds_read_b64_tr_b16).  All eight
 // wavefronts issue MFMAs (v_mfma_f32_32x32x16_bf16), two per SIMD, and each has two roles:
-//   * scores: wave (hg, kh) computes S^T = K Q^T for the 32 heads of group hg over the k-steps of parity kh; its
-//     Q slice is the B operand, resident in registers but for a few k-steps parked in LDS;
+//   * scores: wave (hg, kh) computes S^T = K Q^T for the 32 heads of group hg over half of the 576-wide
+//     contraction (nope columns [256 kh, 256 kh + 256) and rope columns [32 kh, 32 kh + 32)); its Q slice is the B
+//     operand, resident in registers but for a few k-steps parked in LDS;
 //   * values: wave (hh, dq) accumulates O^T = V^T P~ for the 64 heads of half hh and 128 of the 512 value
 //     columns (128 accumulator registers); every V^T fragment read from LDS feeds two MFMAs.
 // Between the two, per tile: the kh = 1 wave of a pair hands its partial S to the kh = 0 wave through LDS; the
 // kh = 0 wave runs the online softmax (one head per lane) and leaves P~ (bf16, already in B-operand order), the
-// rescale factors and a flag in LDS for the value role; meanwhile the kh = 1 waves - the producers - dequantise
-// the next tile out of the registers its gather landed in, store it to the other LDS stage and issue the
-// gather of the tile after.  Two workgroup barriers per tile.
+// rescale factors and a flag in LDS for the value role; and every wave produces its share of the next tile (four of
+// the 32 rows): dequantises it out of the registers its gather landed in, stores it to the other LDS stage and issues
+// the gather of the tile after.  Two workgroup barriers per tile.  All waves run the same phase at the same time on
+// purpose: two waves of a SIMD issuing MFMAs keep the matrix pipe fed (one wave alone gets its LDS operands at half
+// the rate), and two waves issuing vector work fill the vector port (one wave alone issues at about half its rate);
+// running the phases of two wave groups one barrier interval apart was measured and is slower.
 //
 // KV splits write their output normalised by their own sum as fp16 plus (m, l); sfa_combine_kernel merges them.
 #include "common.h"
@@ -40,18 +44,15 @@ constexpr int KROW = (DN + DR) * 2;    // 1152 bytes per tile row = 72 chunks of
 constexpr int STAGE = T * KROW;        // 36864
 constexpr int MAX_SPLIT_TOKENS = 2048; // largest share of a top-k list one workgroup may own
 constexpr int HEADS_PER_WG = 128;
-// of a wave's 18 k-steps of Q, NREG stay in registers and the others are parked in LDS (16 bytes per lane each);
-// the producers hold a gathered tile in registers as well and keep one k-step fewer
-#ifndef NREG_SM_V
-#define NREG_SM_V 12
-#define NREG_PR_V 12
-#define NR_PR_V 5
-#define S_AHEAD_V 4
-#define PV_AHEAD_V 2
-#endif
-constexpr int NREG_SM = NREG_SM_V, NREG_PR = NREG_PR_V;
+// of a wave's 18 k-steps of Q, NREG stay in registers and the others are parked in LDS (16 bytes per lane each): with
+// the 128 accumulator registers of the values role, the wave's share of a gathered tile and the operand fragments in
+// flight this is what fits the 256 registers a wave has at two waves per SIMD without spilling
+constexpr int NREG_SM = 12, NREG_PR = 12;
 // of the 8 tile rows a pair of waves produces, the KH = 1 wave takes NR_PR and the softmax wave the others
-constexpr int NR_PR = NR_PR_V;
+constexpr int NR_PR = 4;
+// operand fragments read ahead of the MFMA that uses them, in the scores and in the values phase (deeper costs
+// registers the kernel does not have)
+constexpr int S_AHEAD = 2, PV_AHEAD = 1;
 constexpr int NPARK_SM = KSTEPS / 2 - NREG_SM, NPARK_PR = KSTEPS / 2 - NREG_PR;
 // LDS layout: two tile stages | partial S, 4 KB per head group | P~, 2 KB per head group | rescale factors [4][32],
 // row sums [128], flags [4] | parked Q | per-split arrays sized by SfaArgs::split_cap (validity words, rows) |
@@ -66,10 +67,13 @@ constexpr int SPLIT_OFF = QPARK_OFF + 4 * (NPARK_SM + NPARK_PR) * 1024;
 constexpr int LDS_LIMIT = 160 * 1024;
 constexpr int OUT_ROW = DN * 4;  // epilogue staging: 64 heads x 512 fp32 per pass, reusing the front of LDS
 constexpr int OUT_HEADS = 64;
+constexpr int QPITCH = 272;      // start-up staging of Q: 128 heads x 256 bytes per round, padded against bank conflicts
+static_assert(HEADS_PER_WG * QPITCH <= STAGE, "a round of Q fits one tile stage");
 __host__ __device__ constexpr int tmask_bytes(int cap) { return (cap / T + 2) * 4; }
 __host__ __device__ constexpr int split_bytes(int cap) { return tmask_bytes(cap) + cap * 4; }
 static_assert(OUT_HEADS * OUT_ROW <= LDS_LIMIT, "epilogue staging must fit");
 static_assert(QPARK_OFF % 16 == 0 && SPLIT_OFF % 16 == 0, "16-byte LDS accesses");
+static_assert(SPLIT_OFF + split_bytes(MAX_SPLIT_TOKENS) <= LDS_LIMIT, "a whole top-k list must fit one workgroup");
 
 
 typedef short s16x4 __attribute__((ext_vector_type(4)));
@@ -150,34 +154,70 @@ __device__ __forceinline__ float dq(uint32_t w, int k, float s, float neg128s)
 }
 
 // Dequantise the share and store it, and the lane's rope piece, into an LDS stage; `present` is the tile's validity word.
+// Two rows at a time, instruction class by instruction class (16 conversions, 16 multiply-adds, 8 packs): a wave issues
+// a vector instruction that depends on the one before it at half the rate of an independent one, and the scheduler,
+// left alone, emits each element's conversion - multiply-add - pack chain back to back.
 template <bool QUANT, int NR>
 __device__ __forceinline__ void dequant_store(const RawTile<QUANT, NR>& r, uint8_t* stage, uint32_t present, int row0,
                                               int lane, int tid)
 {
     float sc[NR];
     if constexpr (QUANT) {
-        // the scale of (row e, this lane's group of 128 columns) sits in lane 4e + lane/16
+        // the scale of (row e, this lane's group of 128 columns) sits in lane 4e + lane/16; an absent row is stored as
+        // zeros (scale 0)
 #pragma unroll
         for (int e = 0; e < NR; ++e)
             sc[e] = __builtin_bit_cast(float, __builtin_amdgcn_ds_bpermute(4 * (4 * e + (lane >> 4)), __builtin_bit_cast(int, r.sc)));
+#pragma unroll
+        for (int e = 0; e < NR; ++e) sc[e] = ((present >> (row0 + e)) & 1u) ? sc[e] : 0.f;
     }
 #pragma unroll
-    for (int e = 0; e < NR; ++e) {
-        const int t = row0 + e;
-        const bool absent = ((present >> t) & 1u) == 0u; // an absent row is stored as zeros
-        u32x4 v;
+    for (int e0 = 0; e0 < NR; e0 += 2) {
+        constexpr int G = 2;
         if constexpr (QUANT) {
-            const uint32_t w0 = r.nope[e][0] ^ 0x80808080u, w1 = r.nope[e][1] ^ 0x80808080u;
-            const float s = absent ? 0.f : sc[e];
-            const float c = -128.f * s;
-            v[0] = pack_bf16x2(dq(w0, 0, s, c), dq(w0, 1, s, c));
-            v[1] = pack_bf16x2(dq(w0, 2, s, c), dq(w0, 3, s, c));
-            v[2] = pack_bf16x2(dq(w1, 0, s, c), dq(w1, 1, s, c));
-            v[3] = pack_bf16x2(dq(w1, 2, s, c), dq(w1, 3, s, c));
+            float f[G][8], c[G];
+            uint32_t pk[G][4];
+#pragma unroll
+            for (int g = 0; g < G; ++g) {
+                if (e0 + g >= NR) break;
+                const uint32_t w0 = r.nope[e0 + g][0] ^ 0x80808080u, w1 = r.nope[e0 + g][1] ^ 0x80808080u;
+                c[g] = -128.f * sc[e0 + g];
+#pragma unroll
+                for (int k = 0; k < 4; ++k) {
+                    f[g][k] = (float)((w0 >> (8 * k)) & 0xffu);
+                    f[g][4 + k] = (float)((w1 >> (8 * k)) & 0xffu);
+                }
+            }
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int g = 0; g < G; ++g) {
+                if (e0 + g >= NR) break;
+#pragma unroll
+                for (int k = 0; k < 8; ++k) f[g][k] = __builtin_fmaf(f[g][k], sc[e0 + g], c[g]);
+            }
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int g = 0; g < G; ++g) {
+                if (e0 + g >= NR) break;
+#pragma unroll
+                for (int k = 0; k < 4; ++k) pk[g][k] = pack_bf16x2(f[g][2 * k], f[g][2 * k + 1]);
+            }
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int g = 0; g < G; ++g) {
+                if (e0 + g >= NR) break;
+                const int t = row0 + e0 + g;
+                *reinterpret_cast<u32x4*>(stage + t * KROW + ((lane ^ swz(t)) << 4)) = u32x4{pk[g][0], pk[g][1], pk[g][2], pk[g][3]};
+            }
         } else {
-            v = absent ? u32x4{0u, 0u, 0u, 0u} : r.nope[e];
+#pragma unroll
+            for (int g = 0; g < G; ++g) {
+                if (e0 + g >= NR) break;
+                const int t = row0 + e0 + g;
+                const u32x4 v = ((present >> t) & 1u) ? r.nope[e0 + g] : u32x4{0u, 0u, 0u, 0u};
+                *reinterpret_cast<u32x4*>(stage + t * KROW + ((lane ^ swz(t)) << 4)) = v;
+            }
         }
-        *reinterpret_cast<u32x4*>(stage + t * KROW + ((lane ^ swz(t)) << 4)) = v;
     }
     {
         const int t = tid >> 4, piece = tid & 15;
@@ -186,32 +226,65 @@ __device__ __forceinline__ void dequant_store(const RawTile<QUANT, NR>& r, uint8
     }
 }
 
-// Resolves a workgroup's share of a token's top-k list: logical indices -> physical cache rows (absent entries: row 0
-// and a cleared bit in the tile's validity word), in LDS.  NT lanes.
-template <int NT>
-__device__ __forceinline__ void resolve_split(const SfaArgs& a, int bi, int tq, int tok0, int cur, int ntiles_real,
-                                              int ntiles, uint32_t* tmask, int* rows, int* bt_lds, int tid,
-                                              int lane)
+// A workgroup's share of a token's top-k list: tiles [tile0, tile0 + ntiles) of the first `cur` entries.
+struct SplitRange {
+    int cur, tile0, ntiles;
+};
+__device__ __forceinline__ SplitRange split_range(int cur, int nsplit, int sp)
 {
-    // this sequence's page table -> LDS (saves one dependent global load per selected token)
-    const bool bt_cached = a.bt_cached != 0;
-    if (bt_cached)
-        for (int i = tid; i < a.bt_stride; i += NT) bt_lds[i] = a.block_table[(int64_t)bi * a.bt_stride + i];
-    // logical top-k entries of this split
-    const int64_t max_logical = (int64_t)a.bt_stride * a.block_size;
-    int my_idx[MAX_SPLIT_TOKENS / NT];
+    const int ntiles_all = (cur + T - 1) / T;
+    const int per = (ntiles_all + nsplit - 1) / nsplit;
+    const int tile0 = sp * per;
+    return {cur, tile0, max(min(ntiles_all, tile0 + per) - tile0, 0)};
+}
+
+// Resolves the workgroup's share: logical indices -> physical cache rows (absent entries: row 0 and a cleared bit in
+// the tile's validity word), in LDS.  NT lanes.  The sequence's length, its page table and the share's top-k entries
+// are requested together: the entries are fetched for the share a full list would give (the usual case) and only
+// fetched again if the length, once known, moves the share.  `between` runs after those requests and before the first
+// wait for them.  Returns the share.
+template <int NT, class Between>
+__device__ __forceinline__ SplitRange resolve_split(const SfaArgs& a, int bi, int si, int tq, int sp, uint32_t* tmask,
+                                                    int* rows, int* bt_lds, int tid, int lane, Between&& between)
+{
+    constexpr int PER_LANE = MAX_SPLIT_TOKENS / NT;
+    const int32_t* list = a.topk_idx + (int64_t)tq * a.topk_stride;
+    const SplitRange guess = split_range(a.topk, a.nsplit, sp);
+    int my_idx[PER_LANE];
+    auto fetch = [&](int tok0) {
 #pragma unroll
-    for (int j = 0; j < MAX_SPLIT_TOKENS / NT; ++j) {
-        const int i = tid + NT * j, g = tok0 + i;
-        my_idx[j] = -1;
-        if (i < ntiles_real * T && g < cur) my_idx[j] = a.topk_idx[(int64_t)tq * a.topk_stride + g];
+        for (int j = 0; j < PER_LANE; ++j)
+            if (NT * j < a.split_cap) my_idx[j] = list[min(tok0 + tid + NT * j, a.topk - 1)];
+    };
+    fetch(guess.tile0 * T);
+    const int act = a.act_seq[bi];
+    // this sequence's page table -> LDS (saves one dependent global load per selected token); a table that fits LDS
+    // has at most BT_PER_LANE entries per lane
+    constexpr int BT_PER_LANE = (LDS_LIMIT - SPLIT_OFF) / 4 / NT + 1;
+    const bool bt_cached = a.bt_cached != 0;
+    int btv[BT_PER_LANE];
+    if (bt_cached) {
+#pragma unroll
+        for (int j = 0; j < BT_PER_LANE; ++j)
+            if (tid + NT * j < a.bt_stride) btv[j] = a.block_table[(int64_t)bi * a.bt_stride + tid + NT * j];
     }
+    between(); // the caller's own loads, behind the ones above and ahead of the first wait for them
+    if (bt_cached) {
+#pragma unroll
+        for (int j = 0; j < BT_PER_LANE; ++j)
+            if (tid + NT * j < a.bt_stride) bt_lds[tid + NT * j] = btv[j];
+    }
+    const SplitRange r = split_range(min(max(act - a.s1 + 1 + si, 0), a.topk), a.nsplit, sp);
+    if (r.tile0 != guess.tile0) fetch(r.tile0 * T); // block-uniform
+    const int tok0 = r.tile0 * T;
+    const int ntiles_even = (r.ntiles + 1) & ~1; // whole wavefronts of entries
+    const int64_t max_logical = (int64_t)a.bt_stride * a.block_size;
     __syncthreads();
 #pragma unroll
-    for (int j = 0; j < MAX_SPLIT_TOKENS / NT; ++j) {
+    for (int j = 0; j < PER_LANE; ++j) {
         const int i = tid + NT * j;
-        if (i >= ntiles * T) break; // wave-uniform: tiles are 32 wide, waves 64
-        const int idx = my_idx[j];
+        if (i >= ntiles_even * T) break; // wave-uniform: tiles are 32 wide, waves 64
+        const int idx = (i < r.ntiles * T && tok0 + i < r.cur) ? my_idx[j] : -1;
         int row = -1;
         if (idx >= 0 && idx < max_logical) {
             int page; // (two loads under a branch, not one load from a selected pointer: that would be a generic-address load)
@@ -219,8 +292,8 @@ __device__ __forceinline__ void resolve_split(const SfaArgs& a, int bi, int tq, 
                 page = bt_lds[idx / a.block_size];
             else
                 page = a.block_table[(int64_t)bi * a.bt_stride + idx / a.block_size];
-            const int64_t r = (int64_t)page * a.block_size + idx % a.block_size;
-            if (page >= 0 && r < a.n_rows) row = (int)r;
+            const int64_t pr = (int64_t)page * a.block_size + idx % a.block_size;
+            if (page >= 0 && pr < a.n_rows) row = (int)pr;
         }
         rows[i] = max(row, 0);
         const uint64_t present = __ballot(row >= 0);
@@ -230,21 +303,24 @@ __device__ __forceinline__ void resolve_split(const SfaArgs& a, int bi, int tq, 
         }
     }
     __syncthreads(); // rows[] / tmask[] ready
+    return r;
 }
 
-// Half of S^T[token, head] = K[token, :] . Q[head, :] for one wave: the k-steps 2*i + kh, i = 0..17.  One accumulation
+// Half of S^T[token, head] = K[token, :] . Q[head, :] for one wave: its 18 k-steps (kstep_of).  One accumulation
 // chain; the K fragments (and the parked Q fragments) are read AHEAD k-steps before the MFMA that uses them.
-template <int NREG>
-__device__ __forceinline__ void s_partial(f32x16& s, const uint8_t* stage, const uint32_t (&s_off)[2], const bf16x8 (&q)[NREG],
+template <int NREG, int KH>
+__device__ __forceinline__ void s_partial(f32x16& s, const uint8_t* stage, const uint32_t (&s_off)[4], const bf16x8 (&q)[NREG],
                                           const uint8_t* qpark)
 {
-    constexpr int AHEAD = S_AHEAD_V, N = KSTEPS / 2;
+    constexpr int AHEAD = S_AHEAD, N = KSTEPS / 2;
     static_assert(NREG >= AHEAD && NREG <= N, "the first reads are of k-steps whose Q fragment is in registers");
 #pragma unroll
     for (int r = 0; r < 16; ++r) s[r] = 0.f;
     bf16x8 kf[N], qp[N];
     auto fetch = [&](int i) {
-        kf[i] = *reinterpret_cast<const bf16x8*>(stage + s_off[i & 1] + (i >> 1) * 128);
+        // nope k-step 16 KH + i: chunks 32 KH + 2 i + hl; rope k-step 32 + 2 KH + (i - 16): chunks 64 + 2 (2 KH + i - 16) + hl
+        kf[i] = *reinterpret_cast<const bf16x8*>(i < 16 ? stage + s_off[i & 3] + KH * 512 + (i >> 2) * 128
+                                                        : stage + s_off[2 * KH + i - 16] + DN * 2);
         if (i >= NREG) qp[i] = *reinterpret_cast<const bf16x8*>(qpark + (i - NREG) * 1024);
     };
 #pragma unroll
@@ -273,20 +349,47 @@ __device__ __forceinline__ void s_partial(f32x16& s, const uint8_t* stage, const
 
 // The body of one wavefront.  KH = 0: the softmax wave of its pair; KH = 1: the wave that hands its partial S over.
 template <bool QUANT, int KH>
-__device__ __forceinline__ void sfa_wave(const SfaArgs& a, uint8_t* smem, const uint32_t* tmask, const int* rows, int tq,
-                                         int sp, int hz, int ntiles, int tid)
+__device__ __forceinline__ void sfa_wave(const SfaArgs& a, uint8_t* smem, uint32_t* tmask, int* rows, int* bt_lds, int tid)
 {
+    const int tq = blockIdx.x, sp = blockIdx.y, hz = blockIdx.z;
+    const int bi = tq / a.s1, si = tq - bi * a.s1;
     constexpr int NREG = KH ? NREG_PR : NREG_SM;
     const int lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6); // (scalar: what follows from it is too)
     const int l32 = lane & 31, hl = lane >> 5;
-    const int hg = wave & 3;              // scores role: heads [32 hg, 32 hg + 32) of the workgroup's 128, k-steps of parity KH
+    const int hg = wave & 3;              // scores role: heads [32 hg, 32 hg + 32) of the workgroup's 128, contraction half KH = wave / 4
     const int hh = wave & 1, dq = wave >> 1; // values role: heads [64 hh, 64 hh + 64), value columns [128 dq, 128 dq + 128)
-    const int last = ntiles - 1;
     const int head0 = hz * HEADS_PER_WG;
     const int head = head0 + hg * 32 + l32;
     const bool head_ok = head < a.nq;
     const bool s_active = head0 + hg * 32 < a.nq;
     const bool pv_active = head0 + hh * 64 < a.nq;
+
+    // The query of the workgroup's 128 heads, requested right behind the few loads the look-up of the share starts with
+    // (it is the largest piece of the start-up traffic and depends on nothing).  Fetched as whole cache lines - in each of four rounds of 128 nope
+    // columns a lane takes four 16-byte pieces, 16 consecutive lanes one head's 256 bytes; then the rope columns, two
+    // pieces per lane - because a load in operand layout (a lane pair per head) costs the texture addresser one line per
+    // lane pair.  The operand layout is made on the way through LDS further down.
+    u32x4 qraw[4][4], qraw_rope[2];
+    auto request_q = [&]() {
+        const int64_t qrow0 = (int64_t)tq * a.nq;
+#pragma unroll
+        for (int r = 0; r < 4; ++r)
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const int p = tid + 512 * j;
+                const int64_t row = qrow0 + min(head0 + (p >> 4), a.nq - 1);
+                qraw[r][j] = *reinterpret_cast<const u32x4*>(reinterpret_cast<const __bf16*>(a.q_nope) + row * DN + 128 * r + 8 * (p & 15));
+            }
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+            const int p = tid + 512 * j;
+            const int64_t row = qrow0 + min(head0 + (p >> 3), a.nq - 1);
+            qraw_rope[j] = *reinterpret_cast<const u32x4*>(reinterpret_cast<const __bf16*>(a.q_rope) + row * DR + 8 * (p & 7));
+        }
+    };
+
+    const SplitRange share = resolve_split<512>(a, bi, si, tq, sp, tmask, rows, bt_lds, tid, lane, request_q);
+    const int ntiles = share.ntiles, last = ntiles - 1;
 
     // Production: this wave's share of every tile (rows row0 .. row0 + NR - 1 and 8 bytes of the rope columns).  The
     // share of tile i+1 is dequantised out of `raw` and stored between the two MFMA phases of tile i, and `raw` is
@@ -297,29 +400,60 @@ __device__ __forceinline__ void sfa_wave(const SfaArgs& a, uint8_t* smem, const 
     RawTile<QUANT, NR> raw;
     if (ntiles > 0) load_raw<QUANT, NR, E0>(raw, a, rows, 0, pair0, lane, tid);
 
-    // this lane's query head and its Q slice: k-steps 2*i + KH, i = 0..17 (0..15 nope, 16..17 rope); B operand
-    // layout: head = column, 8 consecutive k per half-wave.  Lanes past the last head reuse head 0's rows,
-    // their results are never written.
+    // Q into operand layout: this lane's head (hg, l32) and its slice - the 16 k-steps of nope columns
+    // [256 KH, 256 KH + 256) and the 2 of rope columns [32 KH, 32 KH + 32); B operand layout: head = column, 8
+    // consecutive k per half-wave.  Five rounds through the two (still unused) tile stages, alternately: a round's
+    // 128 columns of all heads are written row-major (pitch QPITCH) while the round before is read.
     bf16x8 q[NREG];
     uint8_t* qpark = smem + QPARK_OFF + (KH ? 4 * NPARK_SM * 1024 + hg * (NPARK_PR * 1024) : hg * (NPARK_SM * 1024)) + lane * 16;
     {
-        const int64_t qrow = (int64_t)tq * a.nq + (head_ok ? head : 0);
+        // (a negative softmax_scale is applied as its magnitude to the negated query: the row statistics below are
+        // taken on the raw scores, which needs a factor that commutes with max)
         const uint32_t f = a.softmax_scale < 0.f ? 0x80008000u : 0u;
         const u32x4 qflip = {f, f, f, f};
-        const __bf16* qn = reinterpret_cast<const __bf16*>(a.q_nope) + qrow * DN + KH * 16 + hl * 8;
-        const __bf16* qr = reinterpret_cast<const __bf16*>(a.q_rope) + qrow * DR + KH * 16 + hl * 8;
-#pragma unroll
-        for (int i = 0; i < KSTEPS / 2; ++i) {
-            // (a negative softmax_scale is applied as its magnitude to the negated query: the row statistics below are
-            // taken on the raw scores, which needs a factor that commutes with max)
-            u32x4 w = *reinterpret_cast<const u32x4*>(i < DN / 32 ? qn + i * 32 : qr + (i - DN / 32) * 32);
-            w ^= qflip;
-            const bf16x8 v = __builtin_bit_cast(bf16x8, w);
+        auto keep = [&](int i, u32x4 w) { // k-step i of this wave's 18
+            const bf16x8 v = __builtin_bit_cast(bf16x8, w ^ qflip);
             if (i < NREG)
                 q[i < NREG ? i : 0] = v;
             else
                 *reinterpret_cast<bf16x8*>(qpark + (i - NREG) * 1024) = v;
+        };
+        auto put = [&](int r) {
+            uint8_t* buf = smem + (r & 1) * STAGE;
+            if (r < 4) {
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    const int p = tid + 512 * j;
+                    *reinterpret_cast<u32x4*>(buf + (p >> 4) * QPITCH + (p & 15) * 16) = qraw[r < 4 ? r : 0][j];
+                }
+            } else {
+#pragma unroll
+                for (int j = 0; j < 2; ++j) {
+                    const int p = tid + 512 * j;
+                    *reinterpret_cast<u32x4*>(buf + (p >> 3) * QPITCH + (p & 7) * 16) = qraw_rope[j];
+                }
+            }
+        };
+        auto take = [&](int r) {
+            const uint8_t* row = smem + (r & 1) * STAGE + (hg * 32 + l32) * QPITCH + hl * 16;
+            if (r < 4) {
+                if ((r >> 1) == KH) {
+#pragma unroll
+                    for (int kk = 0; kk < 8; ++kk) keep(8 * (r & 1) + kk, *reinterpret_cast<const u32x4*>(row + kk * 32));
+                }
+            } else {
+#pragma unroll
+                for (int j = 0; j < 2; ++j) keep(16 + j, *reinterpret_cast<const u32x4*>(row + (2 * KH + j) * 32));
+            }
+        };
+        put(0);
+#pragma unroll
+        for (int r = 0; r < 5; ++r) {
+            __syncthreads();
+            take(r);
+            if (r + 1 < 5) put(r + 1);
         }
+        __syncthreads(); // the stages are free for the tiles
     }
     if (ntiles > 0) {
         dequant_store<QUANT, NR>(raw, smem, __builtin_amdgcn_readfirstlane(tmask[0]), row0, lane, tid);
@@ -335,15 +469,17 @@ __device__ __forceinline__ void sfa_wave(const SfaArgs& a, uint8_t* smem, const 
             for (int r = 0; r < 16; ++r) o[i][hb][r] = 0.f;
     float m_run = -INFINITY; // running max of S * scale * log2(e)          (softmax wave)
     float l_run = 0.f;       // this lane's share of sum exp                (softmax wave)
-    const float c_log2 = fabsf(a.softmax_scale) * 1.4426950408889634f;
+    // (never exactly zero: a masked score is -inf, and -inf * 0 would be NaN; 2^(s * 1e-30) is 1 for every finite s, so
+    // a zero scale still gives every attended row the same weight)
+    const float c_log2 = fmaxf(fabsf(a.softmax_scale) * 1.4426950408889634f, 1e-30f);
 
-    // S operand (b128): row l32, chunk 2*ks + hl with ks = 2*i + KH -> chunk 4*i + 2*KH + hl; swizzled offsets
-    // for even and odd i
-    uint32_t s_off[2];
+    // S operand (b128): row l32, chunk 2*ks + hl of k-step ks; swizzled offsets of the four chunk positions 2 m + hl
+    // inside a group of eight chunks
+    uint32_t s_off[4];
     {
-        const int sw = swz(l32), c = 2 * KH + hl;
-        s_off[0] = l32 * KROW + ((c ^ sw) << 4);
-        s_off[1] = l32 * KROW + (((4 + c) ^ sw) << 4);
+        const int sw = swz(l32);
+#pragma unroll
+        for (int m = 0; m < 4; ++m) s_off[m] = l32 * KROW + (((2 * m + hl) ^ sw) << 4);
     }
     // V^T operand (transpose read): lane jj of 16-lane group G points at row 4*hl + jj/4 (+ 16*j + 8*h2), columns
     // 32*db + 16*(G&1) + 4*(jj&3) with db = 4*dq + i -> chunk 16*dq + 4*i + 2*(G&1) + (jj&3)/2; swizzled offsets for even
@@ -369,7 +505,7 @@ __device__ __forceinline__ void sfa_wave(const SfaArgs& a, uint8_t* smem, const 
         uint8_t* stage = smem + (it & 1) * STAGE;
         const uint32_t valid = __builtin_amdgcn_readfirstlane(tmask[it]);
         f32x16 s;
-        if (s_active) s_partial<NREG>(s, stage, s_off, q, qpark);
+        if (s_active) s_partial<NREG, KH>(s, stage, s_off, q, qpark);
         if (KH == 1 && s_active) {
 #pragma unroll
             for (int g = 0; g < 4; ++g)
@@ -457,7 +593,7 @@ __device__ __forceinline__ void sfa_wave(const SfaArgs& a, uint8_t* smem, const 
                     pf[hb][j] = *reinterpret_cast<const bf16x8*>(smem + PBUF_OFF + (2 * hh + hb) * 2048 + j * 1024 + lane * 16);
             // 8 V^T fragments (token block j, column block i), two transpose reads each, feeding two MFMAs each;
             // the reads run AHEAD fragments ahead
-            constexpr int AHEAD = PV_AHEAD_V;
+            constexpr int AHEAD = PV_AHEAD;
             s16x4 lo[8], hi[8];
             auto vread = [&](int n) {
                 const int j = n >> 2, i = n & 3;
@@ -554,31 +690,13 @@ __global__ __attribute__((amdgpu_flat_work_group_size(512, 512), amdgpu_waves_pe
     int* rows = reinterpret_cast<int*>(smem + SPLIT_OFF + tmask_bytes(a.split_cap));
     int* bt_lds = reinterpret_cast<int*>(smem + SPLIT_OFF + split_bytes(a.split_cap));
 
-    const int tid = threadIdx.x, lane = tid & 63;
-    const int tq = blockIdx.x, sp = blockIdx.y, hz = blockIdx.z;
-    const int bi = tq / a.s1, si = tq - bi * a.s1;
-
-    int cur = a.act_seq[bi] - a.s1 + 1 + si;
-    cur = min(max(cur, 0), a.topk);
-    const int ntiles_all = (cur + T - 1) / T;
-    const int per = (ntiles_all + a.nsplit - 1) / a.nsplit;
-    const int tile0 = sp * per;
-    const int ntiles = max(min(ntiles_all, tile0 + per) - tile0, 0);
-    const int tok0 = tile0 * T;
-
-    resolve_split<512>(a, bi, tq, tok0, cur, ntiles, (ntiles + 1) & ~1, tmask, rows, bt_lds, tid, lane);
+    const int tid = threadIdx.x;
 
     // Both kinds of wavefront run the same barrier sequence: one before the first tile, two per tile, the epilogue's.
-#if defined(ONLY_KH0)
-    sfa_wave<QUANT, 0>(a, smem, tmask, rows, tq, sp, hz, ntiles, tid);
-#elif defined(ONLY_KH1)
-    sfa_wave<QUANT, 1>(a, smem, tmask, rows, tq, sp, hz, ntiles, tid);
-#else
     if (tid < 256)
-        sfa_wave<QUANT, 0>(a, smem, tmask, rows, tq, sp, hz, ntiles, tid);
+        sfa_wave<QUANT, 0>(a, smem, tmask, rows, bt_lds, tid);
     else
-        sfa_wave<QUANT, 1>(a, smem, tmask, rows, tq, sp, hz, ntiles, tid);
-#endif
+        sfa_wave<QUANT, 1>(a, smem, tmask, rows, bt_lds, tid);
 }
 
 // attention_out <- 0 (cache without rows: every selected entry is absent)
@@ -589,40 +707,53 @@ __global__ void sfa_zero_kernel(uint32_t* out, int64_t n_words)
 }
 
 // out[row, :] = sum_s (2^(m_s - M) l_s / L) o_s[row, :] with L = sum_s 2^(m_s - M) l_s and o_s the split's normalised
-// output; one block of 128 lanes per output row.  Splits are taken four at a time, every load of a group requested
-// before any is used (splits past the last are the last again with weight 0).
-__global__ __launch_bounds__(128) void sfa_combine_kernel(const void* __restrict__ part_o_fp16,
+// output; one wavefront per output row (a lane owns 8 of the 512 values, 16 bytes of every split's fp16 row), four rows
+// per workgroup.  Splits are taken eight at a time, every load of a group requested before any is used (splits past
+// the last are the last again with weight 0).
+__global__ __launch_bounds__(256) void sfa_combine_kernel(const void* __restrict__ part_o_fp16,
                                                           const float* __restrict__ part_ml, void* out, int nq,
-                                                          int nsplit)
+                                                          int nsplit, int n_rows)
 {
     const _Float16* part_o = static_cast<const _Float16*>(part_o_fp16); // (a plain pointer type keeps the symbol readable)
-    const int row = blockIdx.x; // tq * nq + head
+    const int lane = threadIdx.x & 63;
+    const int row = blockIdx.x * 4 + (threadIdx.x >> 6); // tq * nq + head
+    if (row >= n_rows) return;
     const int tq = row / nq, head = row - tq * nq;
-    float M = -INFINITY;
-    for (int s = 0; s < nsplit; ++s) M = fmaxf(M, part_ml[(((int64_t)tq * nsplit + s) * nq + head) * 2]);
-    float L = 0.f;
-    f32x4 acc = {0.f, 0.f, 0.f, 0.f};
-    if (M > -INFINITY) {
-        for (int s0 = 0; s0 < nsplit; s0 += 4) {
-            f16x4 v[4];
-            float w[4];
+    constexpr int G = 8;
+    float acc[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+    float M = -INFINITY, L = 0.f;
+    for (int s0 = 0; s0 < nsplit; s0 += G) {
+        f16x8 v[G];
+        float m[G], l[G];
 #pragma unroll
-            for (int j = 0; j < 4; ++j) {
-                const int64_t prow = ((int64_t)tq * nsplit + min(s0 + j, nsplit - 1)) * nq + head;
-                v[j] = *reinterpret_cast<const f16x4*>(part_o + prow * DN + threadIdx.x * 4);
-                const float m = part_ml[prow * 2], l = part_ml[prow * 2 + 1];
-                w[j] = (s0 + j < nsplit && l > 0.f) ? exp2f(m - M) * l : 0.f;
-            }
+        for (int j = 0; j < G; ++j) {
+            const int64_t prow = ((int64_t)tq * nsplit + min(s0 + j, nsplit - 1)) * nq + head;
+            v[j] = *reinterpret_cast<const f16x8*>(part_o + prow * DN + lane * 8);
+            m[j] = part_ml[prow * 2];
+            l[j] = s0 + j < nsplit ? part_ml[prow * 2 + 1] : 0.f;
+        }
+        // the group's maximum joins the running one: what was summed so far is rescaled once per group
+        float Mg = M;
 #pragma unroll
-            for (int j = 0; j < 4; ++j) {
-                L += w[j];
-                acc += f32x4{(float)v[j][0], (float)v[j][1], (float)v[j][2], (float)v[j][3]} * w[j];
-            }
+        for (int j = 0; j < G; ++j) Mg = l[j] > 0.f ? fmaxf(Mg, m[j]) : Mg;
+        if (Mg == -INFINITY) continue; // nothing attended in these splits
+        const float back = exp2f(M - Mg); // 0 while nothing has been summed (M = -inf)
+        L *= back;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) acc[e] *= back;
+        M = Mg;
+#pragma unroll
+        for (int j = 0; j < G; ++j) {
+            const float w = l[j] > 0.f ? exp2f(m[j] - M) * l[j] : 0.f;
+            L += w;
+#pragma unroll
+            for (int e = 0; e < 8; ++e) acc[e] += (float)v[j][e] * w;
         }
     }
     const float inv = L > 0.f ? 1.f / L : 0.f;
-    u32x2 v = {pack_bf16x2(acc[0] * inv, acc[1] * inv), pack_bf16x2(acc[2] * inv, acc[3] * inv)};
-    *reinterpret_cast<u32x2*>(reinterpret_cast<uint8_t*>(out) + ((int64_t)row * DN + threadIdx.x * 4) * 2) = v;
+    const u32x4 w = {pack_bf16x2(acc[0] * inv, acc[1] * inv), pack_bf16x2(acc[2] * inv, acc[3] * inv),
+                     pack_bf16x2(acc[4] * inv, acc[5] * inv), pack_bf16x2(acc[6] * inv, acc[7] * inv)};
+    *reinterpret_cast<u32x4*>(reinterpret_cast<uint8_t*>(out) + ((int64_t)row * DN + lane * 8) * 2) = w;
 }
 
 int num_cus()
@@ -693,8 +824,9 @@ hipError_t sfa_launch(const SfaArgs& a, hipStream_t stream)
     if (e != hipSuccess) return e;
     if (a.nsplit > 1) {
         ScopedKernelTimer tm(KID_SFA_COMBINE, stream);
-        hipLaunchKernelGGL(sfa_combine_kernel, dim3(t * a.nq), dim3(128), 0, stream, static_cast<const void*>(a.part_o), a.part_ml, a.out, a.nq,
-                           a.nsplit);
+        const int n_rows = t * a.nq;
+        hipLaunchKernelGGL(sfa_combine_kernel, dim3((n_rows + 3) / 4), dim3(256), 0, stream, static_cast<const void*>(a.part_o),
+                           a.part_ml, a.out, a.nq, a.nsplit, n_rows);
         e = hipGetLastError();
     }
     return e;

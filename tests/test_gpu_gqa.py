@@ -102,6 +102,37 @@ def test_full_size_config4_sample(cuda):
     check(run(case, cuda), case, "config4 sample")
 
 
+def test_full_size_config4(cuda):
+    """The benchmark's GQA configuration at its full batch of 64.  The whole output is produced on the GPU and checked
+    for finiteness and for lying inside the convex hull of each sequence's value rows; the oracle checks a sample of the
+    sequences (a sequence's result depends on its own query, pages and length only)."""
+    g = torch.Generator().manual_seed(45)
+    act = torch.randint(4096, 32769, (64,), generator=g).tolist()
+    case = gqa.make_case(64, 1, 96, 8, act, seed=45)
+    out = run(case, cuda)
+    assert torch.isfinite(out.float()).all()
+    v = case["v"].float()
+    bs = v.shape[1]
+    for bi in range(64):
+        pages = case["block_table"][bi, :(act[bi] + bs - 1) // bs].long()
+        rows = v[pages].reshape(-1, 8, 128)[:act[bi]]                      # [tokens, kv heads, 128]
+        lo, hi = rows.min(0).values, rows.max(0).values                  # [kv heads, 128]
+        o = out[bi].float().reshape(8, 12, 128)
+        assert (o >= lo[:, None] - 0.02).all() and (o <= hi[:, None] + 0.02).all(), f"sequence {bi}"
+    sel = [0, 17, 40, 63]
+    sub_case = dict(case, q=case["q"][sel].contiguous(), block_table=case["block_table"][sel].contiguous(),
+                    act_seq=[act[i] for i in sel])
+    check(out[sel].contiguous(), sub_case, "config4 (sampled sequences)")
+
+
+def test_cache_without_pages_gives_zeros(cuda):
+    # a page table with columns and positive lengths over a cache that holds no page: zero rows, no read of the cache
+    case = gqa.make_case(2, 2, 12, 1, [300, 40], seed=9)
+    case["k"] = case["k"][:0].contiguous()
+    case["v"] = case["v"][:0].contiguous()
+    assert (run(case, cuda) == 0).all()
+
+
 def test_errors(cuda):
     from pypto_amd.error import FeError
     case = gqa.make_case(1, 1, 12, 1, [100], seed=1, block_size=48)

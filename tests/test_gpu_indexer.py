@@ -137,6 +137,28 @@ def test_empty_sequences_and_empty_page_table(cuda):
     check_topk(case, run_indexer(case, cuda))
 
 
+def test_length_beyond_the_page_tables_reach_is_cut_to_it(cuda):
+    # act_seq says more tokens than the page table has entries for: keys past the table do not exist, so the answer
+    # is the oracle's on the length cut to the table's reach - and no score slot the score kernels never wrote is read
+    for s1, bs in ((1, 128), (2, 128), (2, 48)):
+        case = oi.make_case(3, s1, [5000, 700, 2500], seed=31 + s1, block_size=bs)
+        reach = case["block_table"].shape[1] * bs
+        claimed = dict(case, act_seq=[5000 + 70000, 700, 2500])  # (sequence 0 owns every column of the table)
+        cut = dict(case, act_seq=[min(a, reach) for a in claimed["act_seq"]])
+        got = run_indexer(claimed, cuda)
+        assert torch.equal(got, run_indexer(cut, cuda))
+        check_topk(cut, got)
+
+
+def test_cache_without_pages_under_a_page_table(cuda):
+    # no page in the cache but a page table with columns and positive lengths: nothing can be addressed, every slot
+    # is -1, and no kernel touches the (null) cache
+    case = oi.make_case(2, 2, [300, 40], seed=35)
+    case["key_cache"] = case["key_cache"][:0].contiguous()
+    case["k_scale"] = case["k_scale"][:0].contiguous()
+    assert (run_indexer(case, cuda) == -1).all()
+
+
 def test_coincident_scores_of_different_keys(cuda):
     # the reference generator's small integers make different keys tie exactly in the golden; the kernel may order such
     # a pair either way (its fp32 sum runs in another order), which the tolerance rule of check_topk admits

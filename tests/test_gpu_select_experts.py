@@ -48,8 +48,12 @@ def test_config2_grouped(cuda):
     # the benchmark's expert-selector configuration: 8192 tokens x 160 experts, bf16 logits, fp32 bias, 8 groups, top-4
     # groups, top-8 experts, renormalised, x 2.5
     logits, bias = ose.make_case(8192, 160, 2, logits_dtype=torch.bfloat16, bias_dtype=torch.float32)
-    check(logits, bias, 8, True, 4, 8, cuda, scale=2.5, neg=True)
-    check(logits, bias, 8, True, 4, 8, cuda, scale=2.5, neg=False)
+    # (rows whose ids differ from the golden's by a swap of two experts within 2 ulps of each other: the count is
+    # reported and held to a handful - the ids of every other row are bit-exact)
+    n_neg = check(logits, bias, 8, True, 4, 8, cuda, scale=2.5, neg=True)
+    n_zero = check(logits, bias, 8, True, 4, 8, cuda, scale=2.5, neg=False)
+    print(f"config 2: {n_neg} (-inf fill) and {n_zero} (0.0 fill) of 8192 rows used the 2-ulp swap licence")
+    assert n_neg <= 4 and n_zero <= 4
 
 
 def test_dtypes_sizes_and_flags(cuda):

@@ -190,6 +190,36 @@ def test_reference_prefill_case_b1_s256(cuda):
     assert (o >= lo - 0.02).all() and (o <= hi + 0.02).all()
 
 
+def test_negative_and_zero_softmax_scale(cuda):
+    # the scale is just an argument: a negative one turns the softmax towards the smallest scores, zero gives the mean
+    # of the attended rows
+    for scale in (-(192 ** -0.5), 0.0):
+        case = osfa.make_case(2, 32, 1, [900, 70], topk=256, seed=13, dist="bench", softmax_scale=scale)
+        full_check(run_sfa(case, cuda), case, f"scale {scale}")
+
+
+def test_reference_antiquant_case_b64_s1_2(cuda):
+    """The reference's largest packed-row case (deepseekv32_sparse_attention_antiquant.py:627-638,725): batch 64, two
+    query tokens, lengths mixed between 16K and 112K, through sparse_attention_antiquant_d_950.  The whole output is
+    produced on the GPU and checked for finiteness and for lying inside the hull of the dequantised cache; the oracle
+    checks a sample of the query tokens (a token's result depends on its own query and top-k row only)."""
+    g = torch.Generator().manual_seed(64)
+    act = [(16384, 16384, 16384, 32768, 65536)[i] for i in torch.randint(0, 5, (64,), generator=g).tolist()]
+    act[0], act[1], act[2] = 16384, 114688, 114688 - 1
+    case = osfa.make_case(64, 128, 2, act, seed=64)
+    out = run_sfa(case, cuda, packed=True, entry="d_950")
+    assert torch.isfinite(out.float()).all()
+    kn = osfa.dequant_nope(case["kn"], case["kn_scales"]).float()
+    lo, hi = kn.min(0).values, kn.max(0).values
+    o = out.float().reshape(-1, 512)
+    assert (o >= lo - 0.02).all() and (o <= hi + 0.02).all()
+    sel = [0, 1, 2, 33, 63]
+    tk = case["topk_indices"].reshape(64, 2, -1)
+    sub = dict(case, b=len(sel), q=case["q"][sel].contiguous(), topk_indices=tk[sel].reshape(2 * len(sel), -1).contiguous(),
+               block_table=case["block_table"][sel].contiguous(), act_seq=[act[i] for i in sel])
+    full_check(out[sel].contiguous(), sub, "antiquant b64 s1 2 (sampled sequences)")
+
+
 def test_bad_calls_raise_before_launch(cuda):
     from pypto_amd.deepseek_v32_exp import sparse_flash_attention_quant_impl as impl
     from pypto_amd.error import FeError
