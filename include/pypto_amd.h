@@ -91,6 +91,18 @@ int pto_sfa_quant_launch(const PtoTensorDesc* tensors, uint32_t n_tensors, const
                          void* workspace, uint64_t workspace_bytes, void* hip_stream, int sync);
 
 /*
+ * The allocation-free launch of sparse_flash_attention_quant: pto_sfa_quant_launch without the workspace arguments.
+ * It has no counterpart in the reference.  It is for callers that cannot allocate device memory - code under HIP graph
+ * capture, tight serving loops, harnesses that forbid it: the scratch the KV splits need (what
+ * pto_sfa_quant_workspace reports) lives in an array inside the library, 40 MiB on every GPU the library runs on, held
+ * until the process ends.  A problem that needs more is refused with PTO_ERR_WORKSPACE.  Every call on a GPU shares that
+ * GPU's array: calls that overlap in time on one GPU (two streams, two threads) race; calls on one stream do not.
+ * Tensors and parameters as for pto_sfa_quant_launch.
+ */
+int pto_sfa_quant_launch_noalloc(const PtoTensorDesc* tensors, uint32_t n_tensors, const PtoSfaParams* params,
+                                 void* hip_stream, int sync);
+
+/*
  * sparse_attention_antiquant_d / _p / _d_950
  * (models/deepseek_v32_exp/sparse_attention_antiquant_impl.py:287-302,358-373,739-749).
  * tensors[7], in order:

@@ -921,6 +921,24 @@ static int sfa_quant_launch_async(const PtoTensorDesc* tensors, uint32_t n_tenso
     return launch_sfa("sparse_flash_attention_quant", &plan, workspace, workspace_bytes, hip_stream);
 }
 
+int pto_sfa_quant_launch_noalloc(const PtoTensorDesc* tensors, uint32_t n_tensors, const PtoSfaParams* params,
+                                 void* hip_stream, int sync)
+{
+    const char* op = "sparse_flash_attention_quant (no-allocation entry)";
+    SfaPlan plan;
+    int rc = plan_sfa_quant(tensors, n_tensors, params, &plan);
+    if (rc) return rc;
+    if (plan.ws_bytes > pto::SFA_STATIC_SCRATCH_BYTES)
+        return fail(PTO_ERR_WORKSPACE, "%s: this problem needs %llu bytes of scratch, the library's own scratch array holds %llu; use pto_sfa_quant_launch with a workspace",
+                    op, (unsigned long long)plan.ws_bytes, (unsigned long long)pto::SFA_STATIC_SCRATCH_BYTES);
+    void* ws = nullptr;
+    if (plan.ws_bytes > 0) {
+        hipError_t e = pto::sfa_static_scratch(&ws);
+        if (e != hipSuccess) return fail(PTO_ERR_HIP, "%s: the scratch array's address is not available: %s", op, hipGetErrorString(e));
+    }
+    return finish_launch(op, launch_sfa(op, &plan, ws, plan.ws_bytes, hip_stream), hip_stream, sync);
+}
+
 uint64_t pto_sfa_antiquant_workspace(const PtoTensorDesc* tensors, uint32_t n_tensors, const PtoSfaParams* params)
 {
     SfaPlan plan;

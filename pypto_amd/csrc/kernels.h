@@ -32,6 +32,10 @@ struct SfaArgs {
 int sfa_pick_splits(int t, int nq, int topk);
 uint64_t sfa_workspace_bytes(int t, int nq, int nsplit);
 hipError_t sfa_launch(const SfaArgs& a, hipStream_t stream);
+// Device address, on the current device, of the library's own scratch array of SFA_STATIC_SCRATCH_BYTES bytes (looked up
+// once per device).  Every call on a GPU shares that GPU's array.
+constexpr uint64_t SFA_STATIC_SCRATCH_BYTES = 40ull << 20;
+hipError_t sfa_static_scratch(void** ptr);
 
 // ---------------------------------------------------------------- lightning indexer
 struct IndexerArgs {

@@ -788,6 +788,28 @@ uint64_t sfa_workspace_bytes(int t, int nq, int nsplit)
     return (uint64_t)t * nsplit * nq * (DN * sizeof(_Float16) + 2 * sizeof(float));
 }
 
+// Scratch for callers that cannot allocate (sfa_static_scratch): one array per GPU the library runs on, held until the
+// process ends.  In host code the array's name is only a handle for hipGetSymbolAddress - the device address it returns
+// is what kernels and copies are given.
+static __device__ __align__(256) unsigned char scratch[SFA_STATIC_SCRATCH_BYTES];
+
+hipError_t sfa_static_scratch(void** ptr)
+{
+    static std::atomic<void*> cached[64]; // per device ordinal: every GPU has its own copy of the array at its own address
+    int dev = 0;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return e;
+    void* p = cached[dev & 63].load(std::memory_order_acquire);
+    if (p == nullptr) {
+        e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+        if (e != hipSuccess) return e;
+        if (p == nullptr) return hipErrorInvalidSymbol;
+        cached[dev & 63].store(p, std::memory_order_release);
+    }
+    *ptr = p;
+    return hipSuccess;
+}
+
 hipError_t sfa_launch(const SfaArgs& a, hipStream_t stream)
 {
     const int t = a.b * a.s1;
