@@ -111,15 +111,18 @@ def read_kernel_times(lib):
     lib.pto_kernel_name.restype = ctypes.c_char_p
     off = ctypes.c_double(0)
     lib.pto_kernel_timing_overhead(ctypes.c_void_p(torch.cuda.current_stream().cuda_stream), ctypes.byref(off))
-    kernels = {}
+    kernels, raw = {}, {}
     for kid in range(64):
         if not lib.pto_kernel_name(kid):
             break
         ms, n = ctypes.c_double(0), ctypes.c_uint64(0)
         lib.pto_kernel_timing_read(kid, ctypes.byref(ms), ctypes.byref(n))
         if n.value:
-            kernels[lib.pto_kernel_name(kid).decode()] = max(ms.value * 1e3 / n.value - off.value * 1e3, 0.05)
+            name = lib.pto_kernel_name(kid).decode()
+            raw[name] = ms.value * 1e3 / n.value
+            kernels[name] = max(raw[name] - off.value * 1e3, 0.05)
     read_kernel_times.offset_us = off.value * 1e3
+    read_kernel_times.raw_us = raw
     return kernels
 
 
@@ -719,6 +722,20 @@ def main():
     ms_per_step = (t1 - t0) * 1e3 / args.steps
     tokens_per_s = b * s1 / (ms_per_step * 1e-3)
 
+    # the same steps once more, one event pair per step on the launch stream (torch's current stream is the stream the
+    # operators launch on): the spread of a single step, next to the mean above
+    n_single = max(args.steps, 100)
+    evs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(n_single)]
+    for i, (e0, e1) in enumerate(evs):
+        e0.record()
+        step(i)
+        e1.record()
+    torch.cuda.synchronize()
+    single = sorted(e0.elapsed_time(e1) * 1e3 for e0, e1 in evs)
+    step_us = {"median": round(single[len(single) // 2], 1), "p10": round(single[len(single) // 10], 1),
+               "p90": round(single[len(single) * 9 // 10], 1), "n": n_single,
+               "note": "one event pair per step; includes about 4 us of the pair's own offset"}
+
     # second pass over the same steps with an event pair around every kernel launch
     lib.pto_kernel_timing_enable(1)
     for i in range(args.steps):
@@ -741,14 +758,16 @@ def main():
         "sfa_decode_kernel": {"bound": "mfma", "work": sfa_flops, "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s"},
         "sfa_combine_kernel": {"bound": "hbm", "work": t * 128 * 512 * 2, "peak": HBM_PEAK_GBS, "unit": "GB/s"},
         "indexer_select_kernel": {"bound": "hbm", "work": select_bytes, "peak": HBM_PEAK_GBS, "unit": "GB/s"},
+        "indexer_zero_kernel": {"bound": "hbm", "work": t * 2052 * 4, "peak": HBM_PEAK_GBS, "unit": "GB/s"},
     }
     per_kernel = []
     for name, us in kernels.items():
         k = info[name]
         div = 1e3 if k["unit"] == "GB/s" else 1e6  # bytes/us -> GB/s is /1e3 ; flop/us -> TFLOP/s is /1e6
         achieved = k["work"] / us / div
-        per_kernel.append({"kernel": name, "us": round(us, 2), "bound": k["bound"], "achieved": round(achieved, 2),
-                           "peak": k["peak"], "unit": k["unit"], "frac": round(achieved / k["peak"], 4)})
+        per_kernel.append({"kernel": name, "us": round(us, 2), "us_event_pair": round(read_kernel_times.raw_us[name], 2),
+                           "bound": k["bound"], "achieved": round(achieved, 2), "peak": k["peak"], "unit": k["unit"],
+                           "frac": round(achieved / k["peak"], 4)})
     per_kernel.sort(key=lambda r: -r["us"])
     dom = per_kernel[0]
     default_workload = (b, ctx, s1, args.packed, args.ctx_min) == (32, 65536, 1, False, 0)
@@ -761,9 +780,26 @@ def main():
     if sfa_row:
         sfa_row["hbm_gbs"] = round(sfa_bytes / sfa_row["us"] / 1e3, 1)
 
-    cpu_baseline = None
+    # the two stages of the step against their rooflines: the indexer (all of its kernels) streams the index cache
+    # once; attention (decode + split merge) is the bf16 contraction.  The reference labels four sub-stages of its
+    # attention tile loop (Sa_V0 gather and dequantisation, Sa_C1 scores, Sa_V1 softmax, Sa_C2 values:
+    # sparse_flash_attention_quant_impl.py:147,179,261,271); here all four run inside sfa_decode_kernel.
+    idx_us = sum(us for n, us in kernels.items() if n.startswith("indexer_"))
+    sfa_us = sum(us for n, us in kernels.items() if n.startswith("sfa_"))
+    stages = [
+        {"name": "indexer", "kernels": [n for n in kernels if n.startswith("indexer_")], "us": round(idx_us, 2),
+         "bound": "hbm", "achieved": round((score_bytes + topk_bytes) / idx_us / 1e3, 1), "peak": HBM_PEAK_GBS,
+         "unit": "GB/s", "frac": round((score_bytes + topk_bytes) / idx_us / 1e3 / HBM_PEAK_GBS, 4)},
+        {"name": "sparse flash attention (Sa_V0 + Sa_C1 + Sa_V1 + Sa_C2, split merge)",
+         "kernels": [n for n in kernels if n.startswith("sfa_")], "us": round(sfa_us, 2), "bound": "mfma",
+         "achieved": round(sfa_flops / sfa_us / 1e6, 1), "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
+         "frac": round(sfa_flops / sfa_us / 1e6 / MFMA_BF16_PEAK_TFLOPS, 4)},
+    ]
+
+    cpu_baseline, cpu_as_written = None, None
     if not args.no_cpu:
         cpu_baseline = time_cpu_oracle(torch, w, min(args.cpu_seqs, b), scale)
+        cpu_as_written = time_cpu_as_written(torch, w, scale)
 
     print(json.dumps({
         "metric": "decode tokens/sec + achieved HBM GB/s (% of peak), V3.2 SFA b=32 ctx=64K",
@@ -775,7 +811,7 @@ def main():
                                f"s1 {s1}, ctx {f'U[{args.ctx_min}, {ctx}]' if args.ctx_min else ctx}, 64x128 int8 index heads, 128 heads x (512 nope + 64 rope), "
                                f"int8 paged MLA cache, block 128, {'packed 656 B rows' if args.packed else 'three cache tensors'}"},
         "roofline": roofline, "kernels": per_kernel, "event_pair_offset_us": round(read_kernel_times.offset_us, 2),
-        "cpu_baseline": cpu_baseline,
+        "step_us": step_us, "stages": stages, "cpu_baseline": cpu_baseline, "cpu_baseline_as_written": cpu_as_written,
     }))
 
 
@@ -808,6 +844,40 @@ def time_cpu_oracle(torch, w, n_seq, scale):
             "sample": f"first {n_seq} of the {w['b']} sequences of the same workload, {passes} passes after an untimed one "
                       f"({dt:.1f} s): oracle.indexer.lightning_indexer + oracle.sfa.attention_no_flash",
             "host_cpus": os.cpu_count()}
+
+
+def time_cpu_as_written(torch, w, scale):
+    """The reference's goldens the way it writes them - a Python loop over pages for the indexer, Python loops over
+    batch, query token and selected token for attention - timed once each at the tiny attention configuration (batch 1,
+    16 heads, 4096-token cache, top-256) and on the first two sequences of this workload."""
+    from oracle import indexer as oi
+    from oracle import sfa as osfa
+    out = {"kind": "as-written", "unit": "us per query token", "cores": torch.get_num_threads(), "host_cpus": os.cpu_count()}
+    c1 = osfa.make_case(1, 16, 1, [4096], topk=256, seed=7, dist="bench", softmax_scale=scale)
+    args1 = (c1["q"], c1["kn"], c1["kr"], c1["kn_scales"], c1["topk_indices"], c1["block_table"], c1["act_seq"],
+             c1["block_size"], c1["softmax_scale"], c1["topk"])
+    osfa.attention_no_flash_token_loop(*args1)
+    t0 = time.perf_counter()
+    osfa.attention_no_flash_token_loop(*args1)
+    out["attention_tiny"] = round((time.perf_counter() - t0) * 1e6, 1)
+    n_seq, s1 = min(2, w["b"]), w["s1"]
+    t = n_seq * s1
+    s = w["sets"][0]
+    host = {k: v.cpu() for k, v in s.items() if k != "rows"}
+    table, act = w["table"][:n_seq].cpu(), w["act"][:n_seq].tolist()
+    q = torch.cat([w["q_nope"][:t * 128].cpu().reshape(n_seq, s1, 128, 512),
+                   w["q_rope"][:t * 128].cpu().reshape(n_seq, s1, 128, 64)], dim=-1)
+    t0 = time.perf_counter()
+    tk = oi.lightning_indexer(w["idx_q"][:t].cpu(), w["idx_qs"][:t].cpu(), host["idx_k"], host["idx_ks"],
+                              w["idx_w"][:t].cpu(), act, table, s1, 2048)
+    t1 = time.perf_counter()
+    osfa.attention_no_flash_token_loop(q, host["kn"], host["kr"], host["ks"], tk.reshape(t, 2048), table, act, 128, scale, 2048)
+    t2 = time.perf_counter()
+    out["indexer_first_2_sequences"] = round((t1 - t0) * 1e6 / t, 1)
+    out["attention_first_2_sequences"] = round((t2 - t1) * 1e6 / t, 1)
+    out["sample"] = ("one pass each: oracle.sfa.attention_no_flash_token_loop at batch 1 / 16 heads / top-256, then "
+                     "oracle.indexer.lightning_indexer (page loop) + the token loop on the first 2 sequences of this workload")
+    return out
 
 
 if __name__ == "__main__":

@@ -135,6 +135,28 @@ uint64_t pto_lightning_indexer_workspace(const PtoTensorDesc* tensors, uint32_t 
 int pto_lightning_indexer_launch(const PtoTensorDesc* tensors, uint32_t n_tensors, const PtoIndexerParams* params,
                                  void* workspace, uint64_t workspace_bytes, void* hip_stream, int sync);
 
+/* Scalar arguments of topk (python/pypto/op/comparison.py:302-344: k, largest; dim is the last one - the Python mirror
+ * moves any other dimension there). */
+typedef struct {
+    int32_t k;
+    int32_t largest; /* non-zero: the k largest; zero: the k smallest */
+} PtoTopkParams;
+
+/*
+ * topk (python/pypto/op/comparison.py:302-344; interpreter semantics
+ * framework/src/interface/interpreter/calculator/calc_torch.cpp:2481-2494,2734-2749; golden torch.topk(sorted=True),
+ * framework/tests/st/operation/python/vector_operator_golden.py:2247-2259): the k largest (smallest) elements of every
+ * row, best first, equal values by ascending index (-0 and +0 are equal).
+ * tensors[3], in order:
+ *   0 input    [rows, n] FP32 (finite values)
+ *   1 values   [rows, k] FP32  (output)
+ *   2 indices  [rows, k] INT32 (output)
+ * 1 <= k <= n; rows longer than 8192 elements need k <= 2048.  No workspace.
+ */
+uint64_t pto_topk_workspace(const PtoTensorDesc* tensors, uint32_t n_tensors, const PtoTopkParams* params);
+int pto_topk_launch(const PtoTensorDesc* tensors, uint32_t n_tensors, const PtoTopkParams* params, void* workspace,
+                    uint64_t workspace_bytes, void* hip_stream, int sync);
+
 /* Scalar arguments of select_experts (models/glm_v4_5/glm_select_experts.py:317-330: top_k, renormalize, topk_group,
  * num_expert_group).  routed_scaling_factor and fill_neg_inf come from the reference's generalised gating golden
  * (python/tests/ut/interpreter/_ops/moe_gating_topk.py:272,285): the weights are multiplied by the factor, and the experts

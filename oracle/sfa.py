@@ -101,6 +101,33 @@ def attention_no_flash(q, kn, kr, kn_scales, topk_indices, block_table, act_seq,
     return out
 
 
+def attention_no_flash_token_loop(q, kn, kr, kn_scales, topk_indices, block_table, act_seq, block_size, softmax_scale, topk):
+    """The single-pass golden the way the reference writes it: Python loops over batch, query token and selected
+    token, one cache row looked up, dequantised and copied at a time
+    (models/deepseek_v32_exp/deepseekv32_sparse_flash_attention_quant.py:203-257).  Same arithmetic as
+    attention_no_flash, which gathers with index tensors; kept for the pin that the two agree bit for bit and as the
+    "as written" CPU timing."""
+    b, s1, nq, _ = q.shape
+    out = torch.zeros((b, s1, nq, NOPE_DIM), dtype=torch.bfloat16)
+    for bi in range(b):
+        for si in range(s1):
+            n = cur_seq_of(act_seq[bi], s1, si, topk)
+            if n == 0:
+                continue
+            k_rows = torch.zeros((n, NOPE_DIM + ROPE_DIM), dtype=torch.bfloat16)
+            for j in range(n):
+                idx = int(topk_indices[bi * s1 + si, j])
+                off = int(block_table[bi, idx // block_size]) * block_size + idx % block_size
+                deq = (kn[off].reshape(4, SCALE_GROUP).float() * kn_scales[off].reshape(4, 1)).reshape(NOPE_DIM)
+                k_rows[j, :NOPE_DIM] = deq.to(torch.bfloat16)
+                k_rows[j, NOPE_DIM:] = kr[off]
+            s = torch.matmul(q[bi, si].float(), k_rows.float().t()) * softmax_scale
+            p = torch.exp(s - s.amax(dim=-1, keepdim=True))
+            p = (p / p.sum(dim=-1, keepdim=True)).to(torch.bfloat16)
+            out[bi, si] = torch.matmul(p.float(), k_rows[:, :NOPE_DIM].float()).to(torch.bfloat16)
+    return out
+
+
 def attention_flash(q, kn, kr, kn_scales, topk_indices, block_table, act_seq, block_size, softmax_scale, topk,
                     s2_tile=512):
     """Online-softmax golden: per s2_tile chunk, P~ = exp(s - m_tile) is rounded to

@@ -12,6 +12,7 @@ import functools
 import os
 import struct
 import threading
+import weakref
 
 import torch
 
@@ -67,6 +68,10 @@ class AttentionPreQuantParams(ctypes.Structure):
     _fields_ = [("eps", ctypes.c_float)]
 
 
+class TopkParams(ctypes.Structure):
+    _fields_ = [("k", ctypes.c_int32), ("largest", ctypes.c_int32)]
+
+
 class PagedGatherParams(ctypes.Structure):
     _fields_ = [("block_size", ctypes.c_int32), ("size", ctypes.c_int32)]
 
@@ -82,6 +87,7 @@ _OPS = {
     "mla_indexer_prolog_quant": MlaIndexerPrologParams,
     "attention_pre_quant": AttentionPreQuantParams,
     "paged_gather": PagedGatherParams,
+    "topk": TopkParams,
 }
 
 # C status -> Python exception type wrapped by FeError
@@ -176,7 +182,9 @@ def _check_and_describe(tensors):
         off += _DESC.size
     if dev.type != "cuda":
         raise FeError(RuntimeError(f"tensors must be on a HIP device (torch device type 'cuda'), got {dev}"))
-    return dev, (TensorDesc * n).from_buffer(buf)
+    descs = (TensorDesc * n).from_buffer(buf)
+    descs._buf = buf  # (the planned path rewrites addresses in place)
+    return dev, descs
 
 
 _fns = {}
@@ -190,25 +198,76 @@ def _entry_points(op):
     return fns
 
 
-def _launch_on_current_device(dev, ws_fn, launch_fn, descs, n, params):
-    p = ctypes.byref(params)
-    ws_bytes = ws_fn(descs, n, p)
+def _launch_on_current_device(dev, launch_fn, descs, n, params_ref, ws_bytes):
     ws = torch.empty(ws_bytes, dtype=torch.uint8, device=dev) if ws_bytes else None
-    return launch_fn(descs, n, p, ws.data_ptr() if ws is not None else None, ws_bytes,
+    return launch_fn(descs, n, params_ref, ws.data_ptr() if ws is not None else None, ws_bytes,
                      torch.cuda.current_stream(dev).cuda_stream, 0)
 
 
+class _Plan:
+    """What a call leaves behind for the next call of the same operator on the same thread: the checked descriptor
+    array and the workspace size.  The reference keeps a compiled kernel module per (operator, argument shapes) and
+    skips compilation on a hit (python/pypto/frontend/parser/entry.py:613-636, python/src/bindings/runtime.cpp:430-523);
+    what there is to skip here is the validation of the tensor list and the workspace query."""
+    __slots__ = ("refs", "shapes", "ptrs", "buf", "descs", "n", "params", "params_ref", "ws_bytes", "dev", "current")
+
+
+_tls = threading.local()
+_PTR = struct.Struct("P")
+
+
+def _plan_hit(plan, tensors, params):
+    """True when `tensors` are the very objects of the planned call, unchanged in shape and layout, and the scalar
+    parameters are the same bytes; refreshes the descriptors' addresses (the one thing that may differ: storage can be
+    reallocated under a live tensor)."""
+    if plan.n != len(tensors) or bytes(params) != plan.params:
+        return False
+    refs, shapes, ptrs = plan.refs, plan.shapes, plan.ptrs
+    i = 0
+    for t in tensors:
+        if refs[i]() is not t or t.shape != shapes[i] or not t.is_contiguous():
+            return False
+        p = t.data_ptr() if ptrs[i] else 0  # (an empty tensor's descriptor carries a null address)
+        if p != ptrs[i]:
+            _PTR.pack_into(plan.buf, i * _DESC.size, p)
+            ptrs[i] = p
+        i += 1
+    return True
+
+
 def launch(op, tensors, params):
-    """Validate, size the workspace, launch on the current stream of the tensors' device."""
-    ws_fn, launch_fn = _entry_points(op)
-    dev, descs = _check_and_describe(tensors)
-    n = len(tensors)
-    if dev.index is None or dev.index == torch.cuda.current_device():
-        rc = _launch_on_current_device(dev, ws_fn, launch_fn, descs, n, params)
+    """Validate, size the workspace, launch on the current stream of the tensors' device.  A repeated call with the
+    same tensor objects and parameters takes the planned path: only identities, shapes, layouts and addresses are
+    looked at."""
+    plans = getattr(_tls, "plans", None)
+    if plans is None:
+        plans = _tls.plans = {}
+    plan = plans.get(op)
+    if plan is None or not _plan_hit(plan, tensors, params):
+        ws_fn, launch_fn = _entry_points(op)
+        dev, descs = _check_and_describe(tensors)
+        plan = _Plan()
+        plan.n = len(tensors)
+        plan.refs = [weakref.ref(t) for t in tensors]
+        plan.shapes = [t.shape for t in tensors]
+        plan.ptrs = [t.data_ptr() if t.numel() else 0 for t in tensors]
+        plan.descs = descs
+        plan.buf = descs._buf
+        plan.params = bytes(params)
+        plan.params_ref = ctypes.byref(params.__class__.from_buffer_copy(plan.params))
+        plan.ws_bytes = ws_fn(descs, plan.n, plan.params_ref)
+        plan.dev = dev
+        plan.current = dev.index is None
+        plans[op] = plan
+    launch_fn = _entry_points(op)[1]
+    dev = plan.dev
+    if plan.current or dev.index == torch.cuda.current_device():
+        rc = _launch_on_current_device(dev, launch_fn, plan.descs, plan.n, plan.params_ref, plan.ws_bytes)
     else:
         with torch.cuda.device(dev):
-            rc = _launch_on_current_device(dev, ws_fn, launch_fn, descs, n, params)
+            rc = _launch_on_current_device(dev, launch_fn, plan.descs, plan.n, plan.params_ref, plan.ws_bytes)
     if rc != 0:
+        plans.pop(op, None)
         msg = _lib.pto_last_error().decode()
         raise _STATUS_EXC.get(rc, RuntimeError)(msg)
 

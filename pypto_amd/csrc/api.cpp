@@ -893,6 +893,31 @@ static int paged_gather_launch_async(const PtoTensorDesc* tensors, uint32_t n_te
     return PTO_OK;
 }
 
+uint64_t pto_topk_workspace(const PtoTensorDesc*, uint32_t, const PtoTopkParams*) { return 0; }
+
+static int topk_launch_async(const PtoTensorDesc* ts, uint32_t n, const PtoTopkParams* p, void*, uint64_t, void* hip_stream)
+{
+    const char* op = "topk";
+    if (ts == nullptr || n != 3) return fail(PTO_ERR_ARG_COUNT, "%s: expected 3 tensors, got %u", op, n);
+    if (p == nullptr) return fail(PTO_ERR_PARAM, "%s: params is null", op);
+    int rc;
+    if ((rc = check_tensor(op, ts[0], "input", PTO_DT_FP32, 2))) return rc;
+    if ((rc = check_tensor(op, ts[1], "values", PTO_DT_FP32, 2))) return rc;
+    if ((rc = check_tensor(op, ts[2], "indices", PTO_DT_INT32, 2))) return rc;
+    const int64_t rows = ts[0].shape[0], len = ts[0].shape[1];
+    if (ts[1].shape[0] != rows || ts[2].shape[0] != rows || ts[1].shape[1] != p->k || ts[2].shape[1] != p->k)
+        return fail(PTO_ERR_SHAPE, "%s: values and indices must be [%lld, %d]", op, (long long)rows, p->k);
+    if (rows > 0x7fffffff) return fail(PTO_ERR_SHAPE, "%s: too many rows", op);
+    if (!pto::topk_supported(len, p->k))
+        return fail(PTO_ERR_PARAM, "%s: need 1 <= k <= row length; rows longer than 8192 elements need k <= 2048; got row length %lld, k %d",
+                    op, (long long)len, p->k);
+    hipError_t e = pto::topk_launch(static_cast<const float*>(ts[0].addr), static_cast<float*>(ts[1].addr),
+                                    static_cast<int32_t*>(ts[2].addr), rows, (int)len, p->k, p->largest != 0,
+                                    static_cast<hipStream_t>(hip_stream));
+    if (e != hipSuccess) return fail(PTO_ERR_HIP, "%s: HIP launch failed: %s", op, hipGetErrorString(e));
+    return PTO_OK;
+}
+
 uint64_t pto_select_experts_workspace(const PtoTensorDesc*, uint32_t, const PtoSelectExpertsParams*) { return 0; }
 
 static int select_experts_launch_async(const PtoTensorDesc* tensors, uint32_t n_tensors, const PtoSelectExpertsParams* params,
@@ -991,6 +1016,7 @@ PTO_EXPORT_LAUNCH(attention_pre_quant, PtoAttentionPreQuantParams)
 PTO_EXPORT_LAUNCH(gqa_decode, PtoGqaParams)
 PTO_EXPORT_LAUNCH(paged_gather, PtoPagedGatherParams)
 PTO_EXPORT_LAUNCH(select_experts, PtoSelectExpertsParams)
+PTO_EXPORT_LAUNCH(topk, PtoTopkParams)
 PTO_EXPORT_LAUNCH(sfa_quant, PtoSfaParams)
 PTO_EXPORT_LAUNCH(sfa_antiquant, PtoSfaParams)
 PTO_EXPORT_LAUNCH(lightning_indexer, PtoIndexerParams)
@@ -1025,7 +1051,7 @@ const char* pto_kernel_name(int kernel_id)
                                   "sfa_combine_kernel", "indexer_select_kernel", "select_experts_kernel",
                                   "gqa_decode_kernel", "gqa_combine_kernel", "apq_norm_kernel", "prolog_qx_kernel", "apq_gemm_kernel",
                                   "prolog_k_kernel", "mla_xa_kernel", "mla_norm_kernel", "mla_qb_kernel",
-                                  "mla_wuk_kernel", "apq_head_kernel", "paged_gather_kernel"};
+                                  "mla_wuk_kernel", "apq_head_kernel", "paged_gather_kernel", "indexer_zero_kernel"};
     return kernel_id >= 0 && kernel_id < pto::KID_COUNT ? names[kernel_id] : "";
 }
 

@@ -749,7 +749,81 @@ __global__ __launch_bounds__(1024) void indexer_topk_kernel(IndexerArgs a)
                     a.topk_res + (int64_t)row * k, k);
 }
 
+// Standalone top-k of fp32 rows (pypto.topk: python/pypto/op/comparison.py:302-344; order of equal values - smaller
+// index first - framework/src/interface/interpreter/calculator/calc_torch.cpp:2481-2494,2734-2749): values and int32
+// indices of the k largest (or smallest) elements of every row, best first.  One workgroup of 1024 lanes per row.  Rows
+// of up to TOPK_SORT_CAP elements are sorted whole in LDS; longer rows (then k <= MAX_K) go through the radix select
+// first.  Words are (key << 32 | ~index) with the order-preserving key of the value (of its negation for the smallest),
+// so descending word order is the rule above; -0 and +0 count as equal.
+constexpr int TOPK_SORT_CAP = 8192;
+
+// bitonic sort of a[0 .. p), p a power of two <= TOPK_SORT_CAP, descending; 1024 lanes
+__device__ __forceinline__ void bitonic_desc(uint64_t* a, int p)
+{
+    const int tid = threadIdx.x;
+    for (int size = 2; size <= p; size <<= 1)
+        for (int stride = size >> 1; stride > 0; stride >>= 1) {
+            __syncthreads();
+            for (int i = tid; i < p / 2; i += 1024) {
+                const int pos = 2 * i - (i & (stride - 1)); // lower index of the pair
+                const bool desc = (pos & size) == 0;
+                const uint64_t lo = a[pos], hi = a[pos + stride];
+                if ((lo < hi) == desc) {
+                    a[pos] = hi;
+                    a[pos + stride] = lo;
+                }
+            }
+        }
+    __syncthreads();
+}
+
+__global__ __launch_bounds__(1024) void topk_rows_kernel(const float* __restrict__ x, float* __restrict__ values,
+                                                         int32_t* __restrict__ indices, int n, int k, int largest)
+{
+    __shared__ uint64_t buf[TOPK_SORT_CAP];
+    __shared__ uint32_t hist[NBINS];
+    __shared__ uint32_t tmp[16];
+    __shared__ uint32_t s_bin, s_krem, s_cnt, s_out;
+    const int tid = threadIdx.x;
+    const float* row = x + (int64_t)blockIdx.x * n;
+    auto word = [&](int i) { return make_cand(score_key(largest ? row[i] : -row[i]), i); };
+    int p;
+    if (n <= TOPK_SORT_CAP) {
+        p = 2;
+        while (p < n) p <<= 1;
+        for (int i = tid; i < p; i += 1024) buf[i] = i < n ? word(i) : 0ull; // (every real word is > 0: its index part is)
+    } else {
+        p = MAX_K;
+        for (int i = tid; i < MAX_K; i += 1024) buf[i] = 0ull;
+        if (tid == 0) s_out = 0;
+        __syncthreads();
+        auto each = [&](auto&& f) {
+            for (int i = tid; i < n; i += 1024) f(word(i));
+        };
+        auto emit = [&](uint64_t w) {
+            const uint32_t q = atomicAdd(&s_out, 1u);
+            if (q < MAX_K) buf[q] = w;
+        };
+        radix_select64(each, emit, (uint32_t)k, 64, hist, tmp, &s_bin, &s_krem, &s_cnt);
+    }
+    bitonic_desc(buf, p);
+    for (int j = tid; j < k; j += 1024) {
+        const int i = (int)(0xffffffffu - (uint32_t)(buf[j] & 0xffffffffull));
+        indices[(int64_t)blockIdx.x * k + j] = i;
+        values[(int64_t)blockIdx.x * k + j] = row[i];
+    }
+}
+
 } // namespace
+
+bool topk_supported(int64_t n, int64_t k) { return n >= 1 && k >= 1 && k <= n && n <= (1 << 24) && (n <= TOPK_SORT_CAP || k <= MAX_K); }
+
+hipError_t topk_launch(const float* x, float* values, int32_t* indices, int64_t rows, int n, int k, bool largest, hipStream_t stream)
+{
+    if (rows == 0) return hipSuccess;
+    hipLaunchKernelGGL(topk_rows_kernel, dim3((unsigned)rows), dim3(1024), 0, stream, x, values, indices, n, k, largest ? 1 : 0);
+    return hipGetLastError();
+}
 
 // workspace: scores [t, stride] f32 | hist [t, 2048] u32 | counters [t, 4] u32 | winners [t, 2048] u64 | ties [t, 8192] u64
 static uint64_t align256(uint64_t x) { return (x + 255) & ~(uint64_t)255; }
@@ -792,8 +866,11 @@ hipError_t indexer_launch(const IndexerArgs& a, hipStream_t stream)
     args.max_ctx = max_ctx;
     const bool paged = a.block_size % 128 == 0;
     if (!paged || (int64_t)a.b * pchunks > SPAN_LIST_CAP || pchunks > 1024) args.span_list = nullptr;
-    hipLaunchKernelGGL(indexer_zero_kernel, dim3((nzero + 255) / 256), dim3(256), 0, stream, a.hist, nzero, a.act_seq, a.b,
-                       pchunks, max_ctx, args.span_list);
+    {
+        ScopedKernelTimer tm(KID_INDEXER_ZERO, stream);
+        hipLaunchKernelGGL(indexer_zero_kernel, dim3((nzero + 255) / 256), dim3(256), 0, stream, a.hist, nzero, a.act_seq, a.b,
+                           pchunks, max_ctx, args.span_list);
+    }
     {
         ScopedKernelTimer tm(KID_INDEXER_SCORE, stream);
         const bool pow2 = (a.block_size & (a.block_size - 1)) == 0;

@@ -64,6 +64,11 @@ uint64_t indexer_workspace_bytes(int t, int score_stride);
 void indexer_bind_workspace(IndexerArgs& a, void* workspace);
 hipError_t indexer_launch(const IndexerArgs& a, hipStream_t stream);
 
+// ---------------------------------------------------------------- standalone top-k of fp32 rows
+bool topk_supported(int64_t n, int64_t k); // rows of up to 8192 elements with any k <= n; longer rows with k <= 2048
+hipError_t topk_launch(const float* x, float* values, int32_t* indices, int64_t rows, int n, int k, bool largest,
+                       hipStream_t stream);
+
 // ---------------------------------------------------------------- grouped expert selection
 struct SelectExpertsArgs {
     const void* logits; // [t, ne] fp32 or bf16

@@ -54,6 +54,18 @@ def test_every_declared_symbol_is_exported(lib):
     assert lib.pto_abi_version() == 2
 
 
+def test_topk_validation_codes(lib):
+    from pypto_amd._runtime import TopkParams
+    ok = [(FP32, (4, 100)), (FP32, (4, 10)), (INT32, (4, 10))]
+    p = TopkParams(10, 1)
+    assert launch_rc(lib, "topk", ok[:2], p)[0] == -1
+    assert launch_rc(lib, "topk", [(BF16, (4, 100))] + ok[1:], p)[0] == -2
+    assert launch_rc(lib, "topk", [ok[0], (FP32, (4, 9)), ok[2]], p)[0] == -3
+    rc, msg = launch_rc(lib, "topk", [(FP32, (4, 9000)), (FP32, (4, 3000)), (INT32, (4, 3000))], TopkParams(3000, 1))
+    assert rc == -4 and "k <= 2048" in msg
+    assert launch_rc(lib, "topk", [(FP32, (4, 5)), (FP32, (4, 6)), (INT32, (4, 6))], TopkParams(6, 0))[0] == -4
+
+
 def test_tensor_desc_layout_matches_the_reference_abi():
     # framework/include/tile_fwk_bundle/pypto_bundle_api.h:30-35: void* | int32 | int32 | int64[8]
     assert ctypes.sizeof(TensorDesc) == 8 + 4 + 4 + 64

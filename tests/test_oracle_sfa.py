@@ -178,20 +178,5 @@ def test_packed_entry_equals_three_tensor_entry():
 def test_naive_token_loop_restatement_matches():
     """The reference's golden walks the selected tokens one at a time (offset = page * bs + idx % bs, copy the
     row); doing exactly that on a small case must reproduce the vectorised oracle bit for bit."""
-    c = sfa.make_case(1, 3, 2, [150], topk=64, seed=12)
-    out = sfa.attention_no_flash(*_args(c))
-    q, kn, kr, ks = c["q"], c["kn"], c["kr"], c["kn_scales"]
-    for si in range(2):
-        n = min(max(150 - 2 + 1 + si, 0), 64)
-        k_rows = torch.zeros((n, 576), dtype=torch.bfloat16)
-        for j in range(n):
-            idx = int(c["topk_indices"][si, j])
-            off = int(c["block_table"][0, idx // 128]) * 128 + idx % 128
-            deq = (kn[off].reshape(4, 128).float() * ks[off].reshape(4, 1)).reshape(512).to(torch.bfloat16)
-            k_rows[j, :512] = deq
-            k_rows[j, 512:] = kr[off]
-        s = torch.matmul(q[0, si].float(), k_rows.float().t()) * c["softmax_scale"]
-        p = torch.exp(s - s.amax(dim=-1, keepdim=True))
-        p = (p / p.sum(dim=-1, keepdim=True)).to(torch.bfloat16)
-        want = torch.matmul(p.float(), k_rows[:, :512].float()).to(torch.bfloat16)
-        assert torch.equal(out[0, si], want)
+    for c in (sfa.make_case(1, 3, 2, [150], topk=64, seed=12), sfa.make_case(2, 4, 2, [300, 1], topk=128, seed=13)):
+        assert torch.equal(sfa.attention_no_flash_token_loop(*_args(c)), sfa.attention_no_flash(*_args(c)))
