@@ -216,35 +216,74 @@ _tls = threading.local()
 _PTR = struct.Struct("P")
 
 
-def _plan_hit(plan, tensors, params):
-    """True when `tensors` are the very objects of the planned call, unchanged in shape and layout, and the scalar
-    parameters are the same bytes; refreshes the descriptors' addresses (the one thing that may differ: storage can be
-    reallocated under a live tensor)."""
-    if plan.n != len(tensors) or bytes(params) != plan.params:
+def _check_one(idx, t, dev):
+    """The per-tensor checks of _check_and_describe for one operand of a planned call; returns its dtype code."""
+    if type(t) is not torch.Tensor:
+        if not isinstance(t, torch.Tensor):
+            raise FeError(RuntimeError(f"Input {idx + 1} (index {idx}) must be a torch.Tensor, got {t.__class__}"))
+        if type(t).__name__ == "DTensor":
+            raise FeError(RuntimeError(f"Input {idx + 1} (index {idx}) must not be a DTensor, got {t.__class__}"))
+    if not t.is_contiguous():
+        raise FeError(RuntimeError("not all tensors are contiguous"))
+    if t.device != dev:
+        raise FeError(RuntimeError(f"all tensors must be on the same device, got {dev} and {t.device}"))
+    code = _DTYPE_CODE.get(t.dtype)
+    if code is None:
+        raise ValueError(f"unsupported tensor dtype {t.dtype}")
+    if len(t.shape) > 8:
+        raise ValueError("tensors of more than 8 dimensions are not supported")
+    return code
+
+
+def _refresh(plan, tensors, params, ws_fn):
+    """Brings the plan up to date with this call, operand by operand: an operand that is the very object of the planned
+    call, unchanged in shape and layout, only has its address looked at (storage can be reallocated under a live
+    tensor); any other operand - another layer's weights, a new activation - is checked and described afresh.  The
+    workspace is sized again only if a shape or the scalar parameters changed.  False: plan from scratch."""
+    if plan.n != len(tensors):
         return False
-    refs, shapes, ptrs = plan.refs, plan.shapes, plan.ptrs
+    resize = False
+    pb = bytes(params)
+    if pb != plan.params:
+        plan.params = pb
+        plan.params_ref = ctypes.byref(params.__class__.from_buffer_copy(pb))
+        resize = True
+    refs, shapes, ptrs, buf, dev = plan.refs, plan.shapes, plan.ptrs, plan.buf, plan.dev
     i = 0
     for t in tensors:
-        if refs[i]() is not t or t.shape != shapes[i] or not t.is_contiguous():
-            return False
-        p = t.data_ptr() if ptrs[i] else 0  # (an empty tensor's descriptor carries a null address)
-        if p != ptrs[i]:
-            _PTR.pack_into(plan.buf, i * _DESC.size, p)
-            ptrs[i] = p
+        if refs[i]() is t and t.shape == shapes[i] and t.is_contiguous():
+            p = t.data_ptr() if ptrs[i] else 0  # (an empty tensor's descriptor carries a null address)
+            if p != ptrs[i]:
+                _PTR.pack_into(buf, i * _DESC.size, p)
+                ptrs[i] = p
+        else:
+            code = _check_one(i, t, dev)
+            shape = t.shape
+            r = len(shape)
+            p = t.data_ptr() if t.numel() else 0
+            _DESC.pack_into(buf, i * _DESC.size, p, code, r, *shape, *_PAD[r])
+            resize = resize or shape != shapes[i]
+            refs[i], shapes[i], ptrs[i] = weakref.ref(t), shape, p
         i += 1
+    if resize:
+        plan.ws_bytes = ws_fn(plan.descs, plan.n, plan.params_ref)
     return True
 
 
 def launch(op, tensors, params):
-    """Validate, size the workspace, launch on the current stream of the tensors' device.  A repeated call with the
-    same tensor objects and parameters takes the planned path: only identities, shapes, layouts and addresses are
-    looked at."""
+    """Validate, size the workspace, launch on the current stream of the tensors' device.  A repeated call of an
+    operator takes the planned path (_refresh)."""
     plans = getattr(_tls, "plans", None)
     if plans is None:
         plans = _tls.plans = {}
+    ws_fn, launch_fn = _entry_points(op)
     plan = plans.get(op)
-    if plan is None or not _plan_hit(plan, tensors, params):
-        ws_fn, launch_fn = _entry_points(op)
+    try:
+        hit = plan is not None and _refresh(plan, tensors, params, ws_fn)
+    except Exception:
+        plans.pop(op, None)  # the buffer may be half rewritten
+        raise
+    if not hit:
         dev, descs = _check_and_describe(tensors)
         plan = _Plan()
         plan.n = len(tensors)
@@ -259,7 +298,6 @@ def launch(op, tensors, params):
         plan.dev = dev
         plan.current = dev.index is None
         plans[op] = plan
-    launch_fn = _entry_points(op)[1]
     dev = plan.dev
     if plan.current or dev.index == torch.cuda.current_device():
         rc = _launch_on_current_device(dev, launch_fn, plan.descs, plan.n, plan.params_ref, plan.ws_bytes)

@@ -22,9 +22,6 @@ def recorder(monkeypatch):
                       ctypes.cast(p, ctypes.POINTER(rt.TopkParams)).contents.k))
         return 0
 
-    class Dev:
-        type, index = "cuda", None
-
     def describe_with_buf(tensors):
         n = len(tensors)
         buf = bytearray(rt._DESC.size * n)
@@ -42,7 +39,7 @@ def recorder(monkeypatch):
         for t in tensors:
             if not t.is_contiguous():
                 raise rt.FeError(RuntimeError("not all tensors are contiguous"))
-        return Dev(), describe_with_buf(tensors)
+        return tensors[0].device, describe_with_buf(tensors)
 
     monkeypatch.setattr(rt, "_check_and_describe", check2)
     monkeypatch.setattr(rt, "_entry_points", lambda op: (ws_fn, launch_fn))
@@ -73,15 +70,19 @@ def test_new_storage_under_the_same_tensor_is_picked_up(recorder):
     assert recorder[2][1][0] == x.data_ptr()
 
 
-def test_anything_else_that_changes_plans_again(recorder):
+def test_operands_that_change_are_described_afresh(recorder):
     x, v, i = torch.zeros(4, 100), torch.zeros(4, 10), torch.zeros(4, 10, dtype=torch.int32)
     rt.launch("topk", [x, v, i], rt.TopkParams(10, 1))
-    rt.launch("topk", [x.clone(), v, i], rt.TopkParams(10, 1))        # another object of the same shape
-    rt.launch("topk", [x, v, i], rt.TopkParams(10, 0))                # other scalar parameters
+    x2 = x.clone()
+    rt.launch("topk", [x2, v, i], rt.TopkParams(10, 1))               # another object of the same shape: no new sizing
+    assert [c[0] for c in recorder] == ["workspace", "launch", "launch"] and recorder[2][1][0] == x2.data_ptr()
+    rt.launch("topk", [x, v, i], rt.TopkParams(10, 0))                # other scalar parameters: sized again
     x.resize_(4, 50)
-    rt.launch("topk", [x, v, i], rt.TopkParams(10, 0))                # the same object with another shape
-    assert [c[0] for c in recorder] == ["workspace", "launch"] * 4
-    assert recorder[-1][2][0] == (4, 50) and recorder[5][3] == 10
+    rt.launch("topk", [x, v, i], rt.TopkParams(10, 0))                # the same object with another shape: sized again
+    assert [c[0] for c in recorder] == ["workspace", "launch", "launch", "workspace", "launch", "workspace", "launch"]
+    assert recorder[-1][2][0] == (4, 50) and recorder[4][3] == 10
+    with pytest.raises(rt.FeError, match="same device"):
+        rt.launch("topk", [x, v, torch.zeros(4, 10, dtype=torch.int32, device="meta")], rt.TopkParams(10, 0))
     y = torch.zeros(6, 4).t()
     with pytest.raises(rt.FeError, match="contiguous"):
         rt.launch("topk", [y, v, i], rt.TopkParams(10, 0))
@@ -95,6 +96,10 @@ def test_anything_else_that_changes_plans_again(recorder):
 def test_a_dead_tensor_never_matches(recorder):
     v, i = torch.zeros(4, 10), torch.zeros(4, 10, dtype=torch.int32)
     p = rt.TopkParams(10, 1)
+    ptrs = []
     for _ in range(3):
-        rt.launch("topk", [torch.zeros(4, 100), v, i], p)           # a fresh input every call
-    assert [c[0] for c in recorder] == ["workspace", "launch"] * 3
+        x = torch.zeros(4, 100)                                      # a fresh input every call
+        ptrs.append(x.data_ptr())
+        rt.launch("topk", [x, v, i], p)
+    assert [c[0] for c in recorder] == ["workspace", "launch", "launch", "launch"]
+    assert [c[1][0] for c in recorder if c[0] == "launch"] == ptrs
