@@ -49,6 +49,7 @@ constexpr int MQROW = 136;         // bytes per LDS row of a [k][128] int8 weigh
 constexpr int QB_GROUPS = 4;      // wavefront quads of mla_qb_kernel, each with its own stages in flight
 constexpr int QB_MAXS = MAX_R / QB_K / QB_GROUPS; // stages per group at the largest q_lora_rank
 constexpr int QB_QP = MTOK * (MAX_R / 16) / 1024; // 16-byte pieces of the q_norm tile per lane at the largest q_lora_rank
+constexpr int BIG_T = 128;        // token count from which the kernels that own an output tile take over
 
 
 // 32 outputs x 32 tokens += W[KSTEPS steps of 16 rows, outputs]^T . X[tokens, k]: A by transposing reads of the [k][n]
@@ -138,27 +139,114 @@ __device__ __forceinline__ void xa_body(const uint16_t* x, int ldx, int kdim, co
     }
 }
 
+// Output tile `tile` (64 columns) of x @ [w_dq | w_dkv_kr | w_k | w_proj]: its weight columns and their row stride.
+__device__ __forceinline__ const uint16_t* xa_source(const MlaPrologArgs& a, int tile, int& ld)
+{
+    const int qtiles = a.r / 64;
+    if (tile < qtiles) {
+        ld = a.r;
+        return a.w_dq + tile * 64;
+    }
+    if (tile < qtiles + MKV / 64) {
+        ld = MKV;
+        return a.w_dkv_kr + (tile - qtiles) * 64;
+    }
+    if (tile < qtiles + MKV / 64 + PD / 64) { // fused with the indexer prolog: its x @ [w_k | w_proj] rides along
+        ld = PD;
+        return a.w_k + (tile - qtiles - MKV / 64) * 64;
+    }
+    ld = a.n_idx;
+    return a.w_proj + (tile - qtiles - MKV / 64 - PD / 64) * 64;
+}
+
 __global__ __launch_bounds__(1024) void mla_xa_kernel(MlaPrologArgs a)
 {
     extern __shared__ __align__(16) uint8_t xa_lds[]; // [4 groups][256 k][64 n] bf16, rows of XROW2 bytes
-    const int tile = blockIdx.y;
-    const int qtiles = a.r / 64;
-    const uint16_t* src;
     int ld;
-    if (tile < qtiles) {
-        src = a.w_dq + tile * 64;
-        ld = a.r;
-    } else if (tile < qtiles + MKV / 64) {
-        src = a.w_dkv_kr + (tile - qtiles) * 64;
-        ld = MKV;
-    } else if (tile < qtiles + MKV / 64 + PD / 64) { // fused with the indexer prolog: its x @ [w_k | w_proj] rides along
-        src = a.w_k + (tile - qtiles - MKV / 64) * 64;
-        ld = PD;
-    } else {
-        src = a.w_proj + (tile - qtiles - MKV / 64 - PD / 64) * 64;
-        ld = a.n_idx;
+    const uint16_t* src = xa_source(a, blockIdx.y, ld);
+    xa_body(a.x, a.h, a.h, src, ld, a.xa_part, a.ncols, blockIdx.y * 64, blockIdx.x, blockIdx.z * MTOK, a.t, xa_lds);
+}
+
+// The same product at prefill sizes (128 tokens and more): a workgroup owns an output tile of 256 tokens x 64 columns
+// over one 1024-row split of the contraction and walks it in stages of 64 rows, both operands staged through LDS (the
+// next stage's global loads in flight while the current one is multiplied), so that the weights are read once per 256
+// tokens instead of once per 32 and a token row's piece is fetched by 8 neighbouring lanes as one 128-byte run.  Wave w
+// owns tokens [64 w, 64 w + 64) x the 64 columns: every operand fragment read from LDS feeds two MFMAs.  x is the A
+// operand here, so a result register holds one token's value for 32 consecutive columns across the lanes and the
+// partial sums leave as 128-byte runs.  grid (splits, output tiles of 64, token tiles of 256), 256 lanes.
+constexpr int BG_TOK = 256;             // tokens per workgroup
+constexpr int BG_KS = 64;               // contraction rows per stage
+constexpr int BG_XROW = BG_KS * 2 + 16; // bytes per LDS row of the [token][k] tile (padded against bank conflicts)
+__global__ __launch_bounds__(256, 2) void mla_xa_big_kernel(MlaPrologArgs a)
+{
+    __shared__ __align__(16) uint8_t wt[BG_KS * XROW2];
+    __shared__ __align__(16) uint8_t xt[BG_TOK * BG_XROW];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int l32 = lane & 31, hl = lane >> 5, jj = lane & 15, mh = (lane >> 4) & 1;
+    int ld;
+    const uint16_t* src = xa_source(a, blockIdx.y, ld);
+    const int split = blockIdx.x, tok0 = blockIdx.z * BG_TOK, col0 = blockIdx.y * 64;
+    const int kbeg = split * XA_SPLIT;
+    const int stages = (min(a.h, kbeg + XA_SPLIT) - kbeg) / BG_KS;
+    const int srow = tid >> 3, spc = tid & 7;
+    const uint16_t* xp[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) xp[i] = a.x + (int64_t)min(tok0 + srow + 32 * i, a.t - 1) * a.h + kbeg + 8 * spc;
+    const uint16_t* wp = src + (int64_t)(kbeg + srow) * ld + 8 * spc;
+    u32x4 xs[8], ws[2];
+    auto load = [&](int st) {
+#pragma unroll
+        for (int i = 0; i < 8; ++i) xs[i] = *reinterpret_cast<const u32x4*>(xp[i] + st * BG_KS);
+#pragma unroll
+        for (int i = 0; i < 2; ++i) ws[i] = *reinterpret_cast<const u32x4*>(wp + (int64_t)(st * BG_KS + 32 * i) * ld);
+    };
+    f32x16 acc[2][2];
+#pragma unroll
+    for (int tb = 0; tb < 2; ++tb)
+#pragma unroll
+        for (int nb = 0; nb < 2; ++nb)
+#pragma unroll
+            for (int e = 0; e < 16; ++e) acc[tb][nb][e] = 0.f;
+    const uint8_t* xr = xt + (64 * wave + l32) * BG_XROW + 16 * hl;
+    const uint8_t* hp = wt + (8 * hl + (jj >> 2)) * XROW2 + (16 * mh + 4 * (jj & 3)) * 2;
+    load(0);
+    for (int st = 0; st < stages; ++st) {
+        __syncthreads(); // everyone is done with the previous stage's tiles
+#pragma unroll
+        for (int i = 0; i < 8; ++i) *reinterpret_cast<u32x4*>(xt + (srow + 32 * i) * BG_XROW + 16 * spc) = xs[i];
+#pragma unroll
+        for (int i = 0; i < 2; ++i) *reinterpret_cast<u32x4*>(wt + (srow + 32 * i) * XROW2 + 16 * spc) = ws[i];
+        __syncthreads();
+        load(min(st + 1, stages - 1)); // (unconditional: past the end the last stage is fetched again and dropped)
+#pragma unroll
+        for (int ks = 0; ks < BG_KS / 16; ++ks) {
+            bf16x8 xf[2], wf[2];
+#pragma unroll
+            for (int tb = 0; tb < 2; ++tb) xf[tb] = *reinterpret_cast<const bf16x8*>(xr + 32 * tb * BG_XROW + ks * 32);
+#pragma unroll
+            for (int nb = 0; nb < 2; ++nb) {
+                const s16x4 lo = lds_read_tr(hp + 64 * nb + ks * 16 * XROW2);
+                const s16x4 hi = lds_read_tr(hp + 64 * nb + (ks * 16 + 4) * XROW2);
+                wf[nb] = __builtin_bit_cast(bf16x8, __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
+            }
+#pragma unroll
+            for (int tb = 0; tb < 2; ++tb)
+#pragma unroll
+                for (int nb = 0; nb < 2; ++nb)
+                    acc[tb][nb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(xf[tb], wf[nb], acc[tb][nb], 0, 0, 0);
+        }
     }
-    xa_body(a.x, a.h, a.h, src, ld, a.xa_part, a.ncols, tile * 64, blockIdx.x, blockIdx.z * MTOK, a.t, xa_lds);
+    // register e of acc[tb][nb]: token 64 w + 32 tb + 8 (e / 4) + 4 hl + e % 4, column 32 nb + lane % 32
+#pragma unroll
+    for (int tb = 0; tb < 2; ++tb)
+#pragma unroll
+        for (int e = 0; e < 16; ++e) {
+            const int gt = tok0 + 64 * wave + 32 * tb + 8 * (e >> 2) + 4 * hl + (e & 3);
+            if (gt >= a.t) continue;
+            float* out = a.xa_part + ((int64_t)split * a.t + gt) * a.ncols + col0 + l32;
+#pragma unroll
+            for (int nb = 0; nb < 2; ++nb) out[32 * nb] = acc[tb][nb][e];
+        }
 }
 
 // bf16 form of the operator: q_b = q_norm (bf16 [t, r]) @ w_uq_qr (bf16 [r, n * 192]) with the same kernel body;
@@ -514,6 +602,134 @@ __global__ __launch_bounds__(1024) void mla_qb_kernel(MlaPrologArgs a)
     mla_qb_body(a, blockIdx.x * 128, blockIdx.y * MTOK, qb_lds);
 }
 
+// The same product at prefill sizes (128 tokens and more): a workgroup owns 128 tokens x 128 outputs and walks the
+// contraction in stages of 128 rows, both operands staged through LDS with the next stage's global loads in flight.  Wave
+// (wr, wc) owns tokens [64 wr, +64) x outputs [64 wc, +64): every operand fragment read from LDS feeds four MFMAs.  The
+// int32 sums are exact, so the results are the bits of mla_qb_kernel's.  The outputs go through LDS (in place of the
+// operand tiles, which are no longer needed) so that they leave as the 128-byte runs they are in memory - a 128-column
+// tile holds two 64-column segments, each either half of a head's 128 first dims or a head's 64 rotary dims, rotated
+// into place on the way.  grid (n * 192 / 128, token tiles of 128), 256 lanes.
+constexpr int QG_TOK = 128, QG_K = 128;
+constexpr int QG_QROW = QG_K + 16;       // bytes per LDS row of the [token][k] int8 tile (padded against bank conflicts)
+constexpr int QG_OROW = 128 * 2 + 16;    // bytes per LDS row of the [token][128 outputs] bf16 tile
+constexpr int QG_STAGE_BYTES = QG_K * MQROW + QG_TOK * QG_QROW;
+static_assert(QG_TOK * QG_OROW <= QG_STAGE_BYTES, "the output tile takes the operand tiles' place");
+__global__ __launch_bounds__(256, 3) void mla_qb_big_kernel(MlaPrologArgs a)
+{
+#pragma clang fp contract(off)
+    __shared__ __align__(16) uint8_t stage_lds[QG_STAGE_BYTES]; // [128 k][MQROW] weights | [128 tokens][QG_QROW] q_norm
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int l16 = lane & 15, g = lane >> 4, wr = wave >> 1, wc = wave & 1;
+    const int r = a.r, col0 = blockIdx.x * 128, tok0 = blockIdx.y * QG_TOK;
+    const int64_t nq = (int64_t)a.n * MQH;
+    uint8_t* wl = stage_lds;
+    uint8_t* ql = stage_lds + QG_K * MQROW;
+    const int stages = r / QG_K;
+    // 128 rows x 128 bytes of either operand per stage = 4 pieces of 16 bytes per lane (rows tid / 8 + 32 i, piece tid % 8)
+    const int srow = tid >> 3, spc = tid & 7;
+    const int8_t* wp = static_cast<const int8_t*>(a.w_uq_qr) + (int64_t)srow * nq + col0 + 16 * spc;
+    const int8_t* qp[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) qp[i] = a.q_norm + (int64_t)min(tok0 + srow + 32 * i, a.t - 1) * r + 16 * spc;
+    u32x4 wst[4], qst[4];
+    auto load = [&](int st) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) qst[i] = *reinterpret_cast<const u32x4*>(qp[i] + st * QG_K);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) wst[i] = *reinterpret_cast<const u32x4*>(wp + ((int64_t)st * QG_K + 32 * i) * nq);
+    };
+    // the epilogue's scales, requested first
+    float qs_pre[4];
+    f32x4 ws_pre[4];
+#pragma unroll
+    for (int tb = 0; tb < 4; ++tb) qs_pre[tb] = a.q_norm_scale[min(tok0 + 64 * wr + 16 * tb + l16, a.t - 1)];
+#pragma unroll
+    for (int nb = 0; nb < 4; ++nb) ws_pre[nb] = *reinterpret_cast<const f32x4*>(a.w_qb_scale + col0 + 64 * wc + 16 * nb + 4 * g);
+    i32x4 acc[4][4]; // [nb][tb]
+#pragma unroll
+    for (int nb = 0; nb < 4; ++nb)
+#pragma unroll
+        for (int tb = 0; tb < 4; ++tb) acc[nb][tb] = i32x4{0, 0, 0, 0};
+    load(0);
+    for (int st = 0; st < stages; ++st) {
+        __syncthreads(); // everyone is done with the previous stage's tiles
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            u32x2* d = reinterpret_cast<u32x2*>(wl + (srow + 32 * i) * MQROW + 16 * spc);
+            d[0] = u32x2{wst[i][0], wst[i][1]};
+            d[1] = u32x2{wst[i][2], wst[i][3]};
+            *reinterpret_cast<u32x4*>(ql + (srow + 32 * i) * QG_QROW + 16 * spc) = qst[i];
+        }
+        __syncthreads();
+        load(min(st + 1, stages - 1)); // (unconditional: past the end the last stage is fetched again and dropped)
+#pragma unroll
+        for (int ks = 0; ks < QG_K / 64; ++ks) {
+            i32x4 qf[4], wf[4];
+#pragma unroll
+            for (int tb = 0; tb < 4; ++tb)
+                qf[tb] = *reinterpret_cast<const i32x4*>(ql + (64 * wr + 16 * tb + l16) * QG_QROW + ks * 64 + 16 * g);
+            // (the byte-transposing read: see mla_qb_body)
+#pragma unroll
+            for (int nb = 0; nb < 4; ++nb) {
+                const uint8_t* p = wl + (ks * 64 + 16 * g + (l16 >> 1)) * MQROW + 64 * wc + 16 * nb + 8 * (l16 & 1);
+                const v2i lo = lds_read_tr8(p), hi = lds_read_tr8(p + 8 * MQROW);
+                wf[nb] = i32x4{lo[0], lo[1], hi[0], hi[1]};
+            }
+#pragma unroll
+            for (int nb = 0; nb < 4; ++nb)
+#pragma unroll
+                for (int tb = 0; tb < 4; ++tb)
+                    acc[nb][tb] = __builtin_amdgcn_mfma_i32_16x16x64_i8(wf[nb], qf[tb], acc[nb][tb], 0, 0, 0);
+        }
+    }
+    __syncthreads(); // the operand tiles are free: the output tile takes their place
+    // register e of acc[nb][tb]: output col0 + 64 wc + 16 nb + 4 g + e, token 64 wr + 16 tb + l16
+    uint8_t* ot = stage_lds;
+#pragma unroll
+    for (int tb = 0; tb < 4; ++tb) {
+        const int tl = 64 * wr + 16 * tb + l16;
+        const float qs = qs_pre[tb];
+#pragma unroll
+        for (int nb = 0; nb < 4; ++nb) {
+            const int cl = 64 * wc + 16 * nb + 4 * g; // column inside the tile
+            const int d = (col0 + cl) % MQH;
+            const f32x4 ws = ws_pre[nb];
+            uint16_t vb[4];
+#pragma unroll
+            for (int e = 0; e < 4; ++e) vb[e] = f32_to_bf16(((float)acc[nb][tb][e] * qs) * ws[e]);
+            if (d < MNOPE) {
+                const u32x2 pk = {(uint32_t)vb[0] | ((uint32_t)vb[1] << 16), (uint32_t)vb[2] | ((uint32_t)vb[3] << 16)};
+                *reinterpret_cast<u32x2*>(ot + tl * QG_OROW + cl * 2) = pk;
+            } else {
+                const int64_t gtc = (int64_t)min(tok0 + tl, a.t - 1) * MROPE;
+                const uint16_t* cp = a.cos + gtc;
+                const uint16_t* snp = a.sin + gtc;
+                uint16_t* seg = reinterpret_cast<uint16_t*>(ot + tl * QG_OROW) + (cl - (d - MNOPE)); // the head's 64 rotary dims
+#pragma unroll
+                for (int pr = 0; pr < 2; ++pr) {
+                    const int i = (d - MNOPE) / 2 + pr;
+                    const float xe = bf16_to_f32(vb[2 * pr]), xo = bf16_to_f32(vb[2 * pr + 1]);
+                    const float o1 = xe * bf16_to_f32(cp[i]) + (-xo) * bf16_to_f32(snp[i]);
+                    const float o2 = xo * bf16_to_f32(cp[i + 32]) + xe * bf16_to_f32(snp[i + 32]);
+                    seg[i] = f32_to_bf16(o1);
+                    seg[i + 32] = f32_to_bf16(o2);
+                }
+            }
+        }
+    }
+    __syncthreads();
+    // 128 tokens x 2 segments x 128 bytes = 8 pieces of 16 bytes per lane
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+        const int pc = tid + 256 * i, tl = pc >> 4, sg = (pc >> 3) & 1, c = pc & 7;
+        const int gt = tok0 + tl;
+        if (gt >= a.t) continue;
+        const int col = col0 + 64 * sg, head = col / MQH, d0 = col % MQH;
+        uint16_t* dst = d0 < MNOPE ? a.qb_nope + ((int64_t)gt * a.n + head) * MNOPE + d0 : a.q_rope + ((int64_t)gt * a.n + head) * MROPE;
+        *reinterpret_cast<u32x4*>(dst + 8 * c) = *reinterpret_cast<const u32x4*>(ot + tl * QG_OROW + (64 * sg + 8 * c) * 2);
+    }
+}
+
 // ------------------------------------------------------------------------------------------------ fused with the indexer prolog
 // The fused operator runs the two prologs' per-token kernels side by side in one launch, and likewise the two int8
 // GEMMs on q_norm (192 + 64 workgroups at model sizes: one per compute unit); the indexer's x @ [w_k | w_proj] rides along
@@ -543,34 +759,37 @@ __global__ __launch_bounds__(1024) void fused_qb_kernel(MlaPrologArgs m, PrologA
 // ------------------------------------------------------------------------------------------------ q_b[:, head, :128] @ w_uk[head]
 // grid (heads, 512 / 128, z), 256 lanes: wave w owns outputs [32 w, 32 w + 32) of the tile.  The head's 128 x 128 weight
 // tile stays in LDS while the workgroup walks the token tiles z, z + gridDim.z, ... (one at decode sizes; at prefill
-// sizes the weights are then read once per workgroup instead of once per 32 tokens); the next tile's operand rows are
-// requested before the current tile's products.
+// sizes the weights are then read once per workgroup instead of once per token tile); the next tile's operand rows are
+// requested before the current tile's products.  TB blocks of 32 tokens per tile: 1 at decode sizes; 2 at prefill
+// sizes, where every weight fragment read from LDS then feeds two MFMAs.
+template <int TB>
 __global__ __launch_bounds__(256) void mla_wuk_kernel(MlaPrologArgs a)
 {
-    constexpr int OROW = 128 * 2 + 16; // bytes per LDS row of the 32 x 128 bf16 output tile (padded)
+    constexpr int WTOK = MTOK * TB;    // tokens per tile
+    constexpr int OROW = 128 * 2 + 16; // bytes per LDS row of the WTOK x 128 bf16 output tile (padded)
     __shared__ __align__(16) uint8_t wl[MNOPE * TROW];
-    __shared__ __align__(16) uint8_t bt[MTOK * OROW]; // the token tile's operand rows
-    __shared__ __align__(16) uint8_t ot[MTOK * OROW]; // its outputs
+    __shared__ __align__(16) uint8_t bt[WTOK * OROW]; // the token tile's operand rows
+    __shared__ __align__(16) uint8_t ot[WTOK * OROW]; // its outputs
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int l32 = lane & 31, hl = lane >> 5;
     const int head = blockIdx.x, ct = blockIdx.y;
-    const int ttiles = (a.t + MTOK - 1) / MTOK;
+    const int ttiles = (a.t + WTOK - 1) / WTOK;
     const uint16_t* src = a.w_uk + (int64_t)head * MNOPE * MC + ct * 128;
-    // a tile's operand rows: 32 tokens x 256 bytes, fetched once by the workgroup in 16-byte pieces (16 lanes per row) and
+    // a tile's operand rows: WTOK tokens x 256 bytes, fetched once by the workgroup in 16-byte pieces (16 lanes per row) and
     // handed to the waves through LDS - a wave loading its own operand would fetch a different row with every lane pair,
     // which costs the texture addresser a cycle per row and instruction, four times over for the four waves
     const int prow = tid >> 4, pcol = tid & 15;
-    auto fetch = [&](u32x4 (&q)[2], int tt) {
+    auto fetch = [&](u32x4 (&q)[2 * TB], int tt) {
 #pragma unroll
-        for (int i = 0; i < 2; ++i)
-            q[i] = *reinterpret_cast<const u32x4*>(a.qb_nope + ((int64_t)min(tt * MTOK + prow + 16 * i, a.t - 1) * a.n + head) * MNOPE +
+        for (int i = 0; i < 2 * TB; ++i)
+            q[i] = *reinterpret_cast<const u32x4*>(a.qb_nope + ((int64_t)min(tt * WTOK + prow + 16 * i, a.t - 1) * a.n + head) * MNOPE +
                                                    8 * pcol);
     };
-    auto park = [&](const u32x4 (&q)[2]) {
+    auto park = [&](const u32x4 (&q)[2 * TB]) {
 #pragma unroll
-        for (int i = 0; i < 2; ++i) *reinterpret_cast<u32x4*>(bt + (prow + 16 * i) * OROW + 16 * pcol) = q[i];
+        for (int i = 0; i < 2 * TB; ++i) *reinterpret_cast<u32x4*>(bt + (prow + 16 * i) * OROW + 16 * pcol) = q[i];
     };
-    u32x4 q0[2];
+    u32x4 q0[2 * TB];
     fetch(q0, blockIdx.z);
 #pragma unroll
     for (int i = tid; i < MNOPE * 16; i += 256) {
@@ -579,31 +798,45 @@ __global__ __launch_bounds__(256) void mla_wuk_kernel(MlaPrologArgs a)
     }
     park(q0);
     __syncthreads();
+    const int jj = lane & 15, mh = (lane >> 4) & 1;
+    const uint8_t* hp = wl + (8 * hl + (jj >> 2)) * TROW + (32 * wave + 16 * mh + 4 * (jj & 3)) * 2;
     for (int tt = blockIdx.z; tt < ttiles; tt += gridDim.z) {
         // the rows of the tile after this one, if there is one (uniform over the workgroup)
         const bool more = tt + (int)gridDim.z < ttiles;
-        u32x4 qn[2];
+        u32x4 qn[2 * TB];
         if (more) fetch(qn, tt + gridDim.z);
-        u32x4 bx[MNOPE / 16];
+        f32x16 acc[TB];
 #pragma unroll
-        for (int ks = 0; ks < MNOPE / 16; ++ks) bx[ks] = *reinterpret_cast<const u32x4*>(bt + l32 * OROW + (ks * 16 + 8 * hl) * 2);
-        f32x16 acc;
+        for (int tb = 0; tb < TB; ++tb)
 #pragma unroll
-        for (int e = 0; e < 16; ++e) acc[e] = 0.f;
-        gemm_tr_tile<MNOPE / 16, TROW>(acc, wl, 32 * wave, bx, lane);
+            for (int e = 0; e < 16; ++e) acc[tb][e] = 0.f;
+        // (the weight fragment by transposing reads: see gemm_tr_tile)
+#pragma unroll
+        for (int ks = 0; ks < MNOPE / 16; ++ks) {
+            const s16x4 lo = lds_read_tr(hp + ks * 16 * TROW);
+            const s16x4 hi = lds_read_tr(hp + (ks * 16 + 4) * TROW);
+            const bf16x8 av = __builtin_bit_cast(bf16x8, __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
+#pragma unroll
+            for (int tb = 0; tb < TB; ++tb) {
+                const bf16x8 bx = *reinterpret_cast<const bf16x8*>(bt + (32 * tb + l32) * OROW + (ks * 16 + 8 * hl) * 2);
+                acc[tb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(av, bx, acc[tb], 0, 0, 0);
+            }
+        }
         // through LDS, so that a token's 128 outputs leave as one 256-byte run (16 lanes x 16 bytes)
 #pragma unroll
-        for (int e4 = 0; e4 < 4; ++e4) {
-            const u32x2 pk = {(uint32_t)f32_to_bf16(acc[4 * e4]) | ((uint32_t)f32_to_bf16(acc[4 * e4 + 1]) << 16),
-                              (uint32_t)f32_to_bf16(acc[4 * e4 + 2]) | ((uint32_t)f32_to_bf16(acc[4 * e4 + 3]) << 16)};
-            *reinterpret_cast<u32x2*>(ot + l32 * OROW + (32 * wave + 8 * e4 + 4 * hl) * 2) = pk;
-        }
+        for (int tb = 0; tb < TB; ++tb)
+#pragma unroll
+            for (int e4 = 0; e4 < 4; ++e4) {
+                const u32x2 pk = {(uint32_t)f32_to_bf16(acc[tb][4 * e4]) | ((uint32_t)f32_to_bf16(acc[tb][4 * e4 + 1]) << 16),
+                                  (uint32_t)f32_to_bf16(acc[tb][4 * e4 + 2]) | ((uint32_t)f32_to_bf16(acc[tb][4 * e4 + 3]) << 16)};
+                *reinterpret_cast<u32x2*>(ot + (32 * tb + l32) * OROW + (32 * wave + 8 * e4 + 4 * hl) * 2) = pk;
+            }
         __syncthreads(); // outputs parked; every wave is done with the operand rows
 #pragma unroll
-        for (int i = 0; i < 2; ++i) {
+        for (int i = 0; i < 2 * TB; ++i) {
             const int tok = prow + 16 * i;
-            if (tt * MTOK + tok < a.t)
-                *reinterpret_cast<u32x4*>(a.q_nope + ((int64_t)(tt * MTOK + tok) * a.n + head) * MC + ct * 128 + 8 * pcol) =
+            if (tt * WTOK + tok < a.t)
+                *reinterpret_cast<u32x4*>(a.q_nope + ((int64_t)(tt * WTOK + tok) * a.n + head) * MC + ct * 128 + 8 * pcol) =
                     *reinterpret_cast<const u32x4*>(ot + tok * OROW + 16 * pcol);
         }
         if (more) park(qn);
@@ -684,9 +917,13 @@ static hipError_t launch_prologs(const MlaPrologArgs& a, const PrologArgs* p, hi
     const int ttiles = (a.t + MTOK - 1) / MTOK;
     hipError_t e = set_lds_limits();
     if (e != hipSuccess) return e;
+    const bool big = a.t >= BIG_T; // prefill sizes: the kernels that own an output tile
     {
         ScopedKernelTimer tm(KID_MLA_XA, stream);
-        hipLaunchKernelGGL(mla_xa_kernel, dim3(a.ksplits, a.ncols / 64, ttiles), dim3(1024), 4 * XA_K * XROW2, stream, a);
+        if (big)
+            hipLaunchKernelGGL(mla_xa_big_kernel, dim3(a.ksplits, a.ncols / 64, (a.t + BG_TOK - 1) / BG_TOK), dim3(256), 0, stream, a);
+        else
+            hipLaunchKernelGGL(mla_xa_kernel, dim3(a.ksplits, a.ncols / 64, ttiles), dim3(1024), 4 * XA_K * XROW2, stream, a);
     }
     if ((e = hipGetLastError()) != hipSuccess) return e;
     {
@@ -704,6 +941,8 @@ static hipError_t launch_prologs(const MlaPrologArgs& a, const PrologArgs* p, hi
             hipLaunchKernelGGL(mla_qb16_kernel, dim3((a.r + XA_SPLIT - 1) / XA_SPLIT, nq / 64, ttiles), dim3(1024),
                                4 * XA_K * XROW2, stream, a);
             hipLaunchKernelGGL(mla_qb16_epilogue_kernel, dim3(a.t, (nq / 4 + 255) / 256), dim3(256), 0, stream, a);
+        } else if (big && !p) {
+            hipLaunchKernelGGL(mla_qb_big_kernel, dim3(a.n * MQH / 128, (a.t + QG_TOK - 1) / QG_TOK), dim3(256), 0, stream, a);
         } else if (p) {
             const int smem = mla_qb_lds_bytes(a.r) > prolog_q_lds_bytes(a.r) ? mla_qb_lds_bytes(a.r) : prolog_q_lds_bytes(a.r);
             hipLaunchKernelGGL(fused_qb_kernel, dim3(a.n * MQH / 128 + p->n, ttiles), dim3(1024), smem, stream, a, *p);
@@ -715,8 +954,14 @@ static hipError_t launch_prologs(const MlaPrologArgs& a, const PrologArgs* p, hi
     {
         ScopedKernelTimer tm(KID_MLA_WUK, stream);
         // token tiles per workgroup: one while that leaves the grid at about a thousand workgroups or fewer, more beyond
-        const int zdim = std::min(ttiles, std::max(1, 1024 / (a.n * (MC / 128))));
-        hipLaunchKernelGGL(mla_wuk_kernel, dim3(a.n, MC / 128, zdim), dim3(256), 0, stream, a);
+        if (big) {
+            const int wtiles = (a.t + 2 * MTOK - 1) / (2 * MTOK);
+            const int zdim = std::min(wtiles, std::max(1, 1024 / (a.n * (MC / 128))));
+            hipLaunchKernelGGL(mla_wuk_kernel<2>, dim3(a.n, MC / 128, zdim), dim3(256), 0, stream, a);
+        } else {
+            const int zdim = std::min(ttiles, std::max(1, 1024 / (a.n * (MC / 128))));
+            hipLaunchKernelGGL(mla_wuk_kernel<1>, dim3(a.n, MC / 128, zdim), dim3(256), 0, stream, a);
+        }
     }
     return hipGetLastError();
 }

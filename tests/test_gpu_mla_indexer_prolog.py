@@ -130,6 +130,16 @@ def test_prefill_entry_ragged_tiles_small_sizes(cuda):
     check_against_oracle(mla_case, idx_case, fused)
 
 
+def test_prefill_sizes_fused_equals_separate_and_oracle(cuda):
+    # 128 tokens and more: the first product of both calls runs the kernel that owns an output tile, and so does the
+    # separate call's int8 product (exact, so still the fused call's bits)
+    mla_case, idx_case = op.make_fused_case(150, 1, 300, seed=24, n_idx=64, h=1280, q_lora_rank=256, n=4)
+    fused = run_fused(mla_case, idx_case, cuda, entry="mla_indexer_prolog_quant_p")
+    sep = run_separate(mla_case, idx_case, cuda)
+    same_as_separate(fused, sep)
+    check_against_oracle(mla_case, idx_case, fused)
+
+
 def test_index_head_counts_without_the_side_by_side_kernels(cuda):
     # 32 index heads: x @ w_proj is half an output tile wide, so the fused entry runs the two operators back to back
     mla_case, idx_case = op.make_fused_case(5, 1, 300, seed=23, n_idx=32, h=512, q_lora_rank=256, n=4)

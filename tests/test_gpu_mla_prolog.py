@@ -113,10 +113,23 @@ def test_reference_prefill_case_t128(cuda):
     check(case, run(case, cuda, entry="mla_prolog_quant_p"))
 
 
-def check_bf16_form(case, got, eps=EPS):
+def test_prefill_sizes_ragged_token_tiles(cuda):
+    # 128 tokens and more run the kernels that own an output tile (256 / 128 tokens per workgroup): token counts that
+    # end inside a tile, a contraction that is not a whole number of 1024-row splits, several heads per output tile
+    for b, s1, seed, kw in ((130, 1, 31, dict(h=512, q_lora_rank=256, n=4)), (100, 3, 32, dict(h=1280, q_lora_rank=384, n=6)),
+                            (257, 2, 33, dict(h=512, q_lora_rank=128, n=2))):
+        case = op.make_case(b, s1, 64 * s1 * 2 + 300, seed=seed, **kw)
+        check(case, run(case, cuda, entry="mla_prolog_quant_p"))
+    case = op.make_case(150, 1, 600, seed=34, h=1280, q_lora_rank=1280, n=6, quant_b=False)
+    check_bf16_form(case, run(case, cuda, entry="mla_prolog_quant_p"), outliers=1e-4)
+
+
+def check_bf16_form(case, got, eps=EPS, outliers=0.0):
     """bf16 form (the reference's tolerances, :686-694: q_norm, kv, kr rtol 2^-7 / atol 1e-4; q_nope, q_rope rtol 2^-7 /
     atol 5e-3): everything within those everywhere, and bit-equal in at least 98 % of the places - the difference is
-    the summation order of x @ w, which now and then moves a bf16 rounding."""
+    the summation order of x @ w, which now and then moves a bf16 rounding.  `outliers`: the fraction of values that may
+    sit up to 1.5 x outside (a flipped rounding of q_a that the norm's own rounding carries to a second bf16 step; the
+    reference's comparator lets 0.5 % of the values be anywhere)."""
     gold = op.mla_prolog(case, eps, eps)
     rows = case["cache_index"]
 
@@ -124,7 +137,8 @@ def check_bf16_form(case, got, eps=EPS):
         a, b = a.float(), b.float()
         assert torch.isfinite(a).all(), name
         ratio = (a - b).abs() / (atol + rtol * b.abs())
-        assert ratio.max() <= 1, f"{name}: worst {float(ratio.max())} x the tolerance"
+        assert (ratio > 1).float().mean() <= outliers and ratio.max() <= (1.5 if outliers else 1), \
+            f"{name}: worst {float(ratio.max())} x the tolerance, {int((ratio > 1).sum())} values outside"
         assert (a == b).float().mean() >= min_equal, f"{name}: only {(a == b).float().mean():.3f} bit-equal"
 
     floats(got["q_norm"], gold["q_norm"], "q_norm", 0.0078125, 1e-4)
