@@ -18,7 +18,8 @@ import torch
 
 from .error import FeError, PyptoError, PyptoRtError
 
-_LIB_PATH = os.path.join(os.path.dirname(os.path.abspath(__file__)), "libpypto_amd.so")
+# PYPTO_AMD_LIBRARY names another build of the library (e.g. the host-sanitizer build of pypto_amd.build)
+_LIB_PATH = os.environ.get("PYPTO_AMD_LIBRARY") or os.path.join(os.path.dirname(os.path.abspath(__file__)), "libpypto_amd.so")
 _lib = None
 _lib_lock = threading.Lock()
 

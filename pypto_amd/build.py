@@ -2,6 +2,9 @@
 
     python -m pypto_amd.build            # compile
     python -m pypto_amd.build --verbose  # also print register / LDS usage per kernel
+    python -m pypto_amd.build --sanitize # host code with AddressSanitizer and UndefinedBehaviorSanitizer, into
+                                         # libpypto_amd_san.so: for the boundary's validation paths on a machine
+                                         # without a GPU (tests/test_abi_host_sanitized.py runs tests/test_abi_host.py on it)
 """
 import os
 import subprocess
@@ -39,5 +42,32 @@ def build(verbose=False):
     return LIB_PATH
 
 
+SAN_LIB_PATH = os.path.join(HERE, "libpypto_amd_san.so")
+
+
+def build_sanitized():
+    """The library with its host side under ASan + UBSan (the device code is compiled as usual, without optimisation:
+    the host objects refer to it, but nothing this build is used for launches a kernel).  The sanitizer runtime is
+    linked shared, so a process that loads the library preloads sanitizer_runtime()."""
+    hipcc = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
+    cmd = [hipcc, "--offload-arch=gfx950", "-O1", "-g0", "-std=c++17", "-fPIC", "-shared", "-x", "hip",
+           "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+           "-Xarch_host", "-fsanitize=address", "-Xarch_host", "-fsanitize=undefined", "-Xarch_host",
+           "-fno-sanitize-recover=undefined", "-shared-libsan", "-Wno-unused-command-line-argument",
+           "-Wno-unknown-attributes", "-I", INCLUDE, "-I", CSRC]
+    cmd += [os.path.join(CSRC, s) for s in SOURCES] + ["-o", SAN_LIB_PATH]
+    res = subprocess.run(cmd, capture_output=True, text=True)
+    if res.returncode != 0:
+        raise RuntimeError("hipcc failed:\n" + res.stderr)
+    return SAN_LIB_PATH
+
+
+def sanitizer_runtime():
+    clang = os.path.join(os.path.dirname(os.path.realpath(os.environ.get("HIPCC", "/opt/rocm/bin/hipcc"))), "..", "llvm", "bin", "clang")
+    if not os.path.exists(clang):
+        clang = "/opt/rocm/llvm/bin/clang"
+    return subprocess.run([clang, "-print-file-name=libclang_rt.asan-x86_64.so"], capture_output=True, text=True, check=True).stdout.strip()
+
+
 if __name__ == "__main__":
-    print(build(verbose="--verbose" in sys.argv))
+    print(build_sanitized() if "--sanitize" in sys.argv else build(verbose="--verbose" in sys.argv))
