@@ -22,6 +22,8 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include <algorithm>
+
 #include "common.h"
 #include "kernels.h"
 #include "prolog_common.h"
@@ -192,6 +194,83 @@ __global__ __launch_bounds__(256) void apq_gemm_kernel(AttnPreArgs a)
     }
 }
 
+// The projection at prefill sizes (128 tokens and more): a workgroup owns 128 tokens x 128 outputs over one split of
+// the contraction and walks it in stages of 128 rows, both operands staged through LDS with the next stage's global
+// loads in flight while the current stage is multiplied.  Wave (wr, wc) owns tokens [64 wr, +64) x outputs [64 wc, +64):
+// every operand fragment read from LDS feeds four MFMAs, and the weights are read once per 128 tokens instead of once
+// per 32.  Same int32 partial sums as apq_gemm_kernel (exact, so neither the tiling nor the split shows).
+// grid (n_out / 128, splits, token tiles of 128), 256 lanes.
+constexpr int BTOK = 128, BK = 128;
+constexpr int BQROW = BK + 16; // bytes per LDS row of the [token][k] int8 tile (padded against bank conflicts)
+__global__ __launch_bounds__(256, 3) void apq_gemm_big_kernel(AttnPreArgs a, int per)
+{
+    __shared__ __align__(16) uint8_t wl[BK * AROW];
+    __shared__ __align__(16) uint8_t ql[BTOK * BQROW];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int l16 = lane & 15, g = lane >> 4, wr = wave >> 1, wc = wave & 1;
+    const int col0 = blockIdx.x * AD, split = blockIdx.y, tok0 = blockIdx.z * BTOK;
+    const int st0 = split * per, stages = min(a.h / BK, st0 + per) - st0; // this split's stages of 128 rows
+    // 128 rows x 128 bytes of either operand per stage = 4 pieces of 16 bytes per lane (rows tid / 8 + 32 i, piece tid % 8)
+    const int srow = tid >> 3, spc = tid & 7;
+    const int8_t* wp = a.w + ((int64_t)st0 * BK + srow) * a.n_out + col0 + 16 * spc;
+    const int8_t* qp[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) qp[i] = a.x_q + (int64_t)min(tok0 + srow + 32 * i, a.t - 1) * a.h + (int64_t)st0 * BK + 16 * spc;
+    u32x4 wst[4], qst[4];
+    auto load = [&](int st) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) qst[i] = *reinterpret_cast<const u32x4*>(qp[i] + st * BK);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) wst[i] = *reinterpret_cast<const u32x4*>(wp + ((int64_t)st * BK + 32 * i) * a.n_out);
+    };
+    i32x4 acc[4][4]; // [db][tb]
+#pragma unroll
+    for (int db = 0; db < 4; ++db)
+#pragma unroll
+        for (int tb = 0; tb < 4; ++tb) acc[db][tb] = i32x4{0, 0, 0, 0};
+    load(0);
+    for (int st = 0; st < stages; ++st) {
+        __syncthreads(); // everyone is done with the previous stage's tiles
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            u32x2* d = reinterpret_cast<u32x2*>(wl + (srow + 32 * i) * AROW + 16 * spc);
+            d[0] = u32x2{wst[i][0], wst[i][1]};
+            d[1] = u32x2{wst[i][2], wst[i][3]};
+            *reinterpret_cast<u32x4*>(ql + (srow + 32 * i) * BQROW + 16 * spc) = qst[i];
+        }
+        __syncthreads();
+        load(min(st + 1, stages - 1)); // (unconditional: past the end the last stage is fetched again and dropped)
+#pragma unroll
+        for (int ks = 0; ks < BK / 64; ++ks) {
+            i32x4 qf[4], wf[4];
+#pragma unroll
+            for (int tb = 0; tb < 4; ++tb)
+                qf[tb] = *reinterpret_cast<const i32x4*>(ql + (64 * wr + 16 * tb + l16) * BQROW + ks * 64 + 16 * g);
+            // (the byte-transposing read: see apq_gemm_kernel)
+#pragma unroll
+            for (int db = 0; db < 4; ++db) {
+                const uint8_t* p = wl + (ks * 64 + 16 * g + (l16 >> 1)) * AROW + 64 * wc + 16 * db + 8 * (l16 & 1);
+                const v2i lo = lds_read_tr8(p), hi = lds_read_tr8(p + 8 * AROW);
+                wf[db] = i32x4{lo[0], lo[1], hi[0], hi[1]};
+            }
+#pragma unroll
+            for (int db = 0; db < 4; ++db)
+#pragma unroll
+                for (int tb = 0; tb < 4; ++tb)
+                    acc[db][tb] = __builtin_amdgcn_mfma_i32_16x16x64_i8(wf[db], qf[tb], acc[db][tb], 0, 0, 0);
+        }
+    }
+    // register e of acc[db][tb]: output 64 wc + 16 db + 4 g + e, token 64 wr + 16 tb + l16
+#pragma unroll
+    for (int tb = 0; tb < 4; ++tb) {
+        const int tok = tok0 + 64 * wr + 16 * tb + l16;
+        if (tok >= a.t) continue;
+        int32_t* dst = a.part + ((int64_t)split * a.t + tok) * a.n_out + col0 + 64 * wc + 4 * g;
+#pragma unroll
+        for (int db = 0; db < 4; ++db) *reinterpret_cast<i32x4*>(dst + 16 * db) = acc[db][tb];
+    }
+}
+
 // ------------------------------------------------------------------------------------------------ heads
 // grid (q_heads + 2 kv_heads, tokens), 128 lanes: lane = dim of the head
 __global__ __launch_bounds__(128) void apq_head_kernel(AttnPreArgs a)
@@ -256,8 +335,22 @@ static int stages_per_split(int64_t t, int64_t h, int64_t n_out)
     return wgs >= 8 * 448 ? 4 : wgs >= 2 * 448 ? 2 : 1;
 }
 
+// prefill sizes: stages of 128 rows per workgroup of apq_gemm_big_kernel - all of them while that still leaves
+// 256 workgroups, otherwise as many as do
+constexpr int BIG_T = 128;
+static int big_stages_per_split(int64_t t, int64_t h, int64_t n_out)
+{
+    const int64_t tiles = (n_out / AD) * ((t + BTOK - 1) / BTOK), stages = h / BK;
+    const int64_t splits = std::min<int64_t>(stages, std::max<int64_t>(1, (256 + tiles - 1) / tiles));
+    return (int)((stages + splits - 1) / splits);
+}
+
 int attention_pre_ksplits(int64_t t, int64_t h, int64_t n_out)
 {
+    if (t >= BIG_T) {
+        const int per = big_stages_per_split(t, h, n_out);
+        return (int)((h / BK + per - 1) / per);
+    }
     const int per = stages_per_split(t, h, n_out);
     return (int)((h / AK + per - 1) / per);
 }
@@ -290,7 +383,10 @@ hipError_t attention_pre_launch(const AttnPreArgs& a, hipStream_t stream)
         const dim3 grid(a.n_out / AD, a.ksplits, (a.t + ATOK - 1) / ATOK);
         const int per = stages_per_split(a.t, a.h, a.n_out);
         if (a.ksplits != attention_pre_ksplits(a.t, a.h, a.n_out)) return hipErrorInvalidValue;
-        if (per == 4)
+        if (a.t >= BIG_T)
+            hipLaunchKernelGGL(apq_gemm_big_kernel, dim3(a.n_out / AD, a.ksplits, (a.t + BTOK - 1) / BTOK), dim3(256), 0, stream, a,
+                               big_stages_per_split(a.t, a.h, a.n_out));
+        else if (per == 4)
             hipLaunchKernelGGL(apq_gemm_kernel<4>, grid, dim3(256), 0, stream, a);
         else if (per == 2)
             hipLaunchKernelGGL(apq_gemm_kernel<2>, grid, dim3(256), 0, stream, a);

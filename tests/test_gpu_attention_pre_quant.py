@@ -139,6 +139,15 @@ def test_token_counts(cuda, t):
     check(case, run(case, cuda))
 
 
+@pytest.mark.parametrize("t,h,q_heads,kv_heads", [(128, 1024, 4, 2), (200, 5120, 12, 1), (300, 6400, 30, 3), (513, 256, 2, 1)])
+def test_prefill_token_counts(cuda, t, h, q_heads, kv_heads):
+    """128 tokens and more run the projection kernel that owns a 128 x 128 output tile: token counts that end inside a
+    tile, a contraction split into several workgroups with a short last split (6400 = 50 stages of 128), a contraction
+    of two stages taken whole."""
+    case = op.make_case(t, h=h, q_heads=q_heads, kv_heads=kv_heads, seed=t + h)
+    check(case, run(case, cuda))
+
+
 def test_whole_model_heads(cuda):
     """All 96 query and 8 key / value heads of GLM-4.5 on one device."""
     case = op.make_case(16, q_heads=96, kv_heads=8, seed=13)
