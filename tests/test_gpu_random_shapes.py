@@ -69,13 +69,14 @@ def test_attention_random_shapes(cuda, seed):
 def test_attention_pre_quant_random_shapes(cuda, seed):
     """GLM-4.5 attention_pre_quant: token counts around the 32-token tile, hidden sizes on both sides of the two norm
     kernels and with short last splits of the contraction, head counts that put the projection kernel at one, two and
-    four stages per workgroup, every rotary width, both input distributions."""
+    four stages per workgroup, token counts on both sides of the switch to the prefill-size projection kernel, every
+    rotary width, both input distributions."""
     from oracle import attention_pre_quant as oapq
     from test_gpu_attention_pre_quant import check as check_apq
     from test_gpu_attention_pre_quant import run as run_apq
     rng = random.Random(seed)
     for i in range(12):
-        t = rng.choice([1, 2, 7, 8, 31, 32, 33, 63, 64, 65, rng.randint(1, 130)])
+        t = rng.choice([1, 2, 7, 8, 31, 32, 33, 63, 64, 65, 127, 128, 129, 257, rng.randint(1, 130), rng.randint(128, 400)])
         h = 256 * rng.choice([1, 2, 3, 7, 20, 24, 25, 28, 33, 64])
         kv = rng.choice([1, 1, 2, 4])
         qh = kv * rng.choice([1, 2, 6, 12])
@@ -83,3 +84,24 @@ def test_attention_pre_quant_random_shapes(cuda, seed):
         case = oapq.make_case(t, h=h, q_heads=qh, kv_heads=kv, half=half, seed=seed + i, realistic=rng.random() < 0.8)
         print(f"attention_pre_quant case {i}: t {t} h {h} heads {qh}+{kv}+{kv} half {half}", flush=True)
         check_apq(case, run_apq(case, cuda))
+
+
+@pytest.mark.parametrize("seed", [606])
+def test_mla_prolog_prefill_random_shapes(cuda, seed):
+    """MLA prolog at 128 tokens and more (the kernels that own an output tile): token counts that end inside a 128- or
+    256-token tile, contractions of one to several 1024-row splits with a short last one, one to three stages of the
+    int8 product, several heads per 128-column output tile."""
+    from oracle import mla_prolog as omla
+    from test_gpu_mla_prolog import check as check_mla
+    from test_gpu_mla_prolog import run as run_mla
+    rng = random.Random(seed)
+    for i in range(5):
+        t = rng.choice([128, 129, 191, 256, 257, rng.randint(128, 330)])
+        h = 256 * rng.choice([1, 2, 5, 8, 9])
+        r = 128 * rng.choice([1, 2, 3])
+        n = rng.choice([2, 4, 6])
+        s1 = rng.choice([1, 1, 2])
+        b = (t + s1 - 1) // s1
+        print(f"mla_prolog case {i}: b {b} s1 {s1} h {h} r {r} n {n}", flush=True)
+        case = omla.make_case(b, s1, 300, seed=seed + i, h=h, q_lora_rank=r, n=n)
+        check_mla(case, run_mla(case, cuda, entry="mla_prolog_quant_p"))
