@@ -779,6 +779,13 @@ def main():
     sfa_row = next((r for r in per_kernel if r["kernel"] == "sfa_decode_kernel"), None)
     if sfa_row:
         sfa_row["hbm_gbs"] = round(sfa_bytes / sfa_row["us"] / 1e3, 1)
+    score_row = next((r for r in per_kernel if r["kernel"] == "indexer_score_kernel"), None)
+    if score_row:
+        # the score kernel is bound by the cache stream; its int8 MFMA rate (2 x 64 heads x 128 dims per key and query
+        # token) is reported beside it
+        int8_ops = s1 * sum(lengths) * 2 * 64 * 128
+        score_row["int8_mfma_tops"] = round(int8_ops / score_row["us"] / 1e6, 1)
+        score_row["int8_mfma_frac"] = round(int8_ops / score_row["us"] / 1e6 / 5000.0, 4)
 
     # the two stages of the step against their rooflines: the indexer (all of its kernels) streams the index cache
     # once; attention (decode + split merge) is the bf16 contraction.  The reference labels four sub-stages of its
