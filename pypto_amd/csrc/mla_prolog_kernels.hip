@@ -50,6 +50,10 @@ constexpr int QB_GROUPS = 4;      // wavefront quads of mla_qb_kernel, each with
 constexpr int QB_MAXS = MAX_R / QB_K / QB_GROUPS; // stages per group at the largest q_lora_rank
 constexpr int QB_QP = MTOK * (MAX_R / 16) / 1024; // 16-byte pieces of the q_norm tile per lane at the largest q_lora_rank
 constexpr int BIG_T = 128;        // token count from which the kernels that own an output tile take over
+constexpr int BIG_T2 = 256;       // token count above which their tiles are 256 tokens tall
+#ifndef XA_BIG2_DEPTH
+#define XA_BIG2_DEPTH 2
+#endif
 
 
 // 32 outputs x 32 tokens += W[KSTEPS steps of 16 rows, outputs]^T . X[tokens, k]: A by transposing reads of the [k][n]
@@ -167,81 +171,93 @@ __global__ __launch_bounds__(1024) void mla_xa_kernel(MlaPrologArgs a)
     xa_body(a.x, a.h, a.h, src, ld, a.xa_part, a.ncols, blockIdx.y * 64, blockIdx.x, blockIdx.z * MTOK, a.t, xa_lds);
 }
 
-// The same product at prefill sizes (128 tokens and more): a workgroup owns an output tile of 256 tokens x 64 columns
-// over one 1024-row split of the contraction and walks it in stages of 64 rows, both operands staged through LDS (the
-// next stage's global loads in flight while the current one is multiplied), so that the weights are read once per 256
-// tokens instead of once per 32 and a token row's piece is fetched by 8 neighbouring lanes as one 128-byte run.  Wave w
-// owns tokens [64 w, 64 w + 64) x the 64 columns: every operand fragment read from LDS feeds two MFMAs.  x is the A
-// operand here, so a result register holds one token's value for 32 consecutive columns across the lanes and the
-// partial sums leave as 128-byte runs.  grid (splits, output tiles of 64, token tiles of 256), 256 lanes.
-constexpr int BG_TOK = 256;             // tokens per workgroup
+// The same product at prefill sizes (128 tokens and more): a workgroup owns an output tile of 128 tokens x 64 columns
+// over one 1024-row split of the contraction and walks it in stages of 64 rows, both operands staged through LDS, so
+// that the weights are read once per 128 tokens instead of once per 32 and a token row's piece is fetched by 8
+// neighbouring lanes as one 128-byte run.  The global loads of BG_DEPTH stages are in flight at any time (register
+// sets used round-robin): a stage's multiplication takes a few hundred nanoseconds and a load comes back after one to
+// two microseconds, so with one stage ahead the sixteen stages of a split were sixteen memory latencies in a row
+// (29 us at 512 tokens with 256 x 64 tiles; a 256 x 128 tile that halves the operand traffic but leaves one
+// workgroup per CU was slower still: 33 us).  Wave w owns tokens [32 w, +32) x the 64 columns.  x is the A operand here,
+// so a result register holds one token's value for 32 consecutive columns across the lanes and the partial sums leave
+// as 128-byte runs.  grid (splits, output tiles of 64, token tiles), 256 lanes.
 constexpr int BG_KS = 64;               // contraction rows per stage
 constexpr int BG_XROW = BG_KS * 2 + 16; // bytes per LDS row of the [token][k] tile (padded against bank conflicts)
-__global__ __launch_bounds__(256, 2) void mla_xa_big_kernel(MlaPrologArgs a)
+// TB: blocks of 32 tokens per wave (the workgroup's tile is 128 TB tokens x 64 columns; with TB = 2 a weight fragment read
+// from LDS feeds two MFMAs and the weights are read half as often, which is what counts once the token count is large
+// enough for the kernel to be bound by what the CUs draw from the L2); DEPTH: stages whose loads are in flight.
+template <int TB, int DEPTH>
+__global__ __launch_bounds__(256, TB == 1 ? 3 : 2) void mla_xa_big_kernel(MlaPrologArgs a)
 {
+    constexpr int TOK = 128 * TB;
+    static_assert((XA_SPLIT / BG_KS) % DEPTH == 0 && XA_K % (BG_KS * DEPTH) == 0, "whole rounds of stages in every split");
     __shared__ __align__(16) uint8_t wt[BG_KS * XROW2];
-    __shared__ __align__(16) uint8_t xt[BG_TOK * BG_XROW];
+    __shared__ __align__(16) uint8_t xt[TOK * BG_XROW];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int l32 = lane & 31, hl = lane >> 5, jj = lane & 15, mh = (lane >> 4) & 1;
     int ld;
     const uint16_t* src = xa_source(a, blockIdx.y, ld);
-    const int split = blockIdx.x, tok0 = blockIdx.z * BG_TOK, col0 = blockIdx.y * 64;
+    const int split = blockIdx.x, tok0 = blockIdx.z * TOK, col0 = blockIdx.y * 64;
     const int kbeg = split * XA_SPLIT;
-    const int stages = (min(a.h, kbeg + XA_SPLIT) - kbeg) / BG_KS;
+    const int stages = (min(a.h, kbeg + XA_SPLIT) - kbeg) / BG_KS; // a multiple of DEPTH (h is one of 256)
     const int srow = tid >> 3, spc = tid & 7;
-    const uint16_t* xp[8];
+    const uint16_t* xp[4 * TB];
 #pragma unroll
-    for (int i = 0; i < 8; ++i) xp[i] = a.x + (int64_t)min(tok0 + srow + 32 * i, a.t - 1) * a.h + kbeg + 8 * spc;
+    for (int i = 0; i < 4 * TB; ++i) xp[i] = a.x + (int64_t)min(tok0 + srow + 32 * i, a.t - 1) * a.h + kbeg + 8 * spc;
     const uint16_t* wp = src + (int64_t)(kbeg + srow) * ld + 8 * spc;
-    u32x4 xs[8], ws[2];
-    auto load = [&](int st) {
+    u32x4 xs[DEPTH][4 * TB], ws[DEPTH][2];
+    auto load = [&](int st, int u) {
 #pragma unroll
-        for (int i = 0; i < 8; ++i) xs[i] = *reinterpret_cast<const u32x4*>(xp[i] + st * BG_KS);
+        for (int i = 0; i < 4 * TB; ++i) xs[u][i] = *reinterpret_cast<const u32x4*>(xp[i] + st * BG_KS);
 #pragma unroll
-        for (int i = 0; i < 2; ++i) ws[i] = *reinterpret_cast<const u32x4*>(wp + (int64_t)(st * BG_KS + 32 * i) * ld);
+        for (int i = 0; i < 2; ++i) ws[u][i] = *reinterpret_cast<const u32x4*>(wp + (int64_t)(st * BG_KS + 32 * i) * ld);
     };
-    f32x16 acc[2][2];
+    f32x16 acc[TB][2];
 #pragma unroll
-    for (int tb = 0; tb < 2; ++tb)
+    for (int tb = 0; tb < TB; ++tb)
 #pragma unroll
         for (int nb = 0; nb < 2; ++nb)
 #pragma unroll
             for (int e = 0; e < 16; ++e) acc[tb][nb][e] = 0.f;
-    const uint8_t* xr = xt + (64 * wave + l32) * BG_XROW + 16 * hl;
+    const uint8_t* xr = xt + (32 * TB * wave + l32) * BG_XROW + 16 * hl;
     const uint8_t* hp = wt + (8 * hl + (jj >> 2)) * XROW2 + (16 * mh + 4 * (jj & 3)) * 2;
-    load(0);
-    for (int st = 0; st < stages; ++st) {
-        __syncthreads(); // everyone is done with the previous stage's tiles
 #pragma unroll
-        for (int i = 0; i < 8; ++i) *reinterpret_cast<u32x4*>(xt + (srow + 32 * i) * BG_XROW + 16 * spc) = xs[i];
+    for (int u = 0; u < DEPTH; ++u) load(u, u);
+    for (int st0 = 0; st0 < stages; st0 += DEPTH) {
 #pragma unroll
-        for (int i = 0; i < 2; ++i) *reinterpret_cast<u32x4*>(wt + (srow + 32 * i) * XROW2 + 16 * spc) = ws[i];
-        __syncthreads();
-        load(min(st + 1, stages - 1)); // (unconditional: past the end the last stage is fetched again and dropped)
+        for (int u = 0; u < DEPTH; ++u) {
+            __syncthreads(); // everyone is done with the previous stage's tiles
 #pragma unroll
-        for (int ks = 0; ks < BG_KS / 16; ++ks) {
-            bf16x8 xf[2], wf[2];
+            for (int i = 0; i < 4 * TB; ++i) *reinterpret_cast<u32x4*>(xt + (srow + 32 * i) * BG_XROW + 16 * spc) = xs[u][i];
 #pragma unroll
-            for (int tb = 0; tb < 2; ++tb) xf[tb] = *reinterpret_cast<const bf16x8*>(xr + 32 * tb * BG_XROW + ks * 32);
+            for (int i = 0; i < 2; ++i) *reinterpret_cast<u32x4*>(wt + (srow + 32 * i) * XROW2 + 16 * spc) = ws[u][i];
+            __syncthreads();
+            load(min(st0 + u + DEPTH, stages - 1), u); // (unconditional: past the end the last stage is fetched again and dropped)
 #pragma unroll
-            for (int nb = 0; nb < 2; ++nb) {
-                const s16x4 lo = lds_read_tr(hp + 64 * nb + ks * 16 * XROW2);
-                const s16x4 hi = lds_read_tr(hp + 64 * nb + (ks * 16 + 4) * XROW2);
-                wf[nb] = __builtin_bit_cast(bf16x8, __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
+            for (int ks = 0; ks < BG_KS / 16; ++ks) {
+                bf16x8 xf[TB], wf[2];
+#pragma unroll
+                for (int tb = 0; tb < TB; ++tb) xf[tb] = *reinterpret_cast<const bf16x8*>(xr + 32 * tb * BG_XROW + ks * 32);
+#pragma unroll
+                for (int nb = 0; nb < 2; ++nb) {
+                    const s16x4 lo = lds_read_tr(hp + 64 * nb + ks * 16 * XROW2);
+                    const s16x4 hi = lds_read_tr(hp + 64 * nb + (ks * 16 + 4) * XROW2);
+                    wf[nb] = __builtin_bit_cast(bf16x8, __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
+                }
+#pragma unroll
+                for (int tb = 0; tb < TB; ++tb)
+#pragma unroll
+                    for (int nb = 0; nb < 2; ++nb)
+                        acc[tb][nb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(xf[tb], wf[nb], acc[tb][nb], 0, 0, 0);
             }
-#pragma unroll
-            for (int tb = 0; tb < 2; ++tb)
-#pragma unroll
-                for (int nb = 0; nb < 2; ++nb)
-                    acc[tb][nb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(xf[tb], wf[nb], acc[tb][nb], 0, 0, 0);
         }
     }
-    // register e of acc[tb][nb]: token 64 w + 32 tb + 8 (e / 4) + 4 hl + e % 4, column 32 nb + lane % 32
+    // register e of acc[tb][nb]: token 32 TB w + 32 tb + 8 (e / 4) + 4 hl + e % 4, column 32 nb + lane % 32
 #pragma unroll
-    for (int tb = 0; tb < 2; ++tb)
+    for (int tb = 0; tb < TB; ++tb)
 #pragma unroll
         for (int e = 0; e < 16; ++e) {
-            const int gt = tok0 + 64 * wave + 32 * tb + 8 * (e >> 2) + 4 * hl + (e & 3);
+            const int gt = tok0 + 32 * TB * wave + 32 * tb + 8 * (e >> 2) + 4 * hl + (e & 3);
             if (gt >= a.t) continue;
             float* out = a.xa_part + ((int64_t)split * a.t + gt) * a.ncols + col0 + l32;
 #pragma unroll
@@ -932,7 +948,10 @@ static hipError_t launch_prologs(const MlaPrologArgs& a, const PrologArgs* p, hi
     {
         ScopedKernelTimer tm(KID_MLA_XA, stream);
         if (big)
-            hipLaunchKernelGGL(mla_xa_big_kernel, dim3(a.ksplits, a.ncols / 64, (a.t + BG_TOK - 1) / BG_TOK), dim3(256), 0, stream, a);
+            if (a.t <= BIG_T2)
+                hipLaunchKernelGGL((mla_xa_big_kernel<1, 4>), dim3(a.ksplits, a.ncols / 64, (a.t + 127) / 128), dim3(256), 0, stream, a);
+            else
+                hipLaunchKernelGGL((mla_xa_big_kernel<2, XA_BIG2_DEPTH>), dim3(a.ksplits, a.ncols / 64, (a.t + 255) / 256), dim3(256), 0, stream, a);
         else
             hipLaunchKernelGGL(mla_xa_kernel, dim3(a.ksplits, a.ncols / 64, ttiles), dim3(1024), 4 * XA_K * XROW2, stream, a);
     }
