@@ -630,7 +630,11 @@ constexpr int QG_QROW = QG_K + 16;       // bytes per LDS row of the [token][k] 
 constexpr int QG_OROW = 128 * 2 + 16;    // bytes per LDS row of the [token][128 outputs] bf16 tile
 constexpr int QG_STAGE_BYTES = QG_K * MQROW + QG_TOK * QG_QROW;
 static_assert(QG_TOK * QG_OROW <= QG_STAGE_BYTES, "the output tile takes the operand tiles' place");
-__global__ __launch_bounds__(256, 3) void mla_qb_big_kernel(MlaPrologArgs a)
+// DEPTH: stages whose loads are in flight (register sets used round-robin).  One keeps the kernel at 158 registers, three
+// workgroups to a CU - what the 768 workgroups of 512 tokens want; at 256 tokens and fewer the grid leaves at most two
+// workgroups to a CU anyway, and the twelve stages of a tile are otherwise twelve memory latencies in a row.
+template <int DEPTH>
+__global__ __launch_bounds__(256, DEPTH == 1 ? 3 : 2) void mla_qb_big_kernel(MlaPrologArgs a)
 {
 #pragma clang fp contract(off)
     __shared__ __align__(16) uint8_t stage_lds[QG_STAGE_BYTES]; // [128 k][MQROW] weights | [128 tokens][QG_QROW] q_norm
@@ -647,12 +651,12 @@ __global__ __launch_bounds__(256, 3) void mla_qb_big_kernel(MlaPrologArgs a)
     const int8_t* qp[4];
 #pragma unroll
     for (int i = 0; i < 4; ++i) qp[i] = a.q_norm + (int64_t)min(tok0 + srow + 32 * i, a.t - 1) * r + 16 * spc;
-    u32x4 wst[4], qst[4];
-    auto load = [&](int st) {
+    u32x4 wst[DEPTH][4], qst[DEPTH][4];
+    auto load = [&](int st, int u) {
 #pragma unroll
-        for (int i = 0; i < 4; ++i) qst[i] = *reinterpret_cast<const u32x4*>(qp[i] + st * QG_K);
+        for (int i = 0; i < 4; ++i) qst[u][i] = *reinterpret_cast<const u32x4*>(qp[i] + st * QG_K);
 #pragma unroll
-        for (int i = 0; i < 4; ++i) wst[i] = *reinterpret_cast<const u32x4*>(wp + ((int64_t)st * QG_K + 32 * i) * nq);
+        for (int i = 0; i < 4; ++i) wst[u][i] = *reinterpret_cast<const u32x4*>(wp + ((int64_t)st * QG_K + 32 * i) * nq);
     };
     // the epilogue's scales, requested first
     float qs_pre[4];
@@ -666,36 +670,42 @@ __global__ __launch_bounds__(256, 3) void mla_qb_big_kernel(MlaPrologArgs a)
     for (int nb = 0; nb < 4; ++nb)
 #pragma unroll
         for (int tb = 0; tb < 4; ++tb) acc[nb][tb] = i32x4{0, 0, 0, 0};
-    load(0);
-    for (int st = 0; st < stages; ++st) {
-        __syncthreads(); // everyone is done with the previous stage's tiles
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            u32x2* d = reinterpret_cast<u32x2*>(wl + (srow + 32 * i) * MQROW + 16 * spc);
-            d[0] = u32x2{wst[i][0], wst[i][1]};
-            d[1] = u32x2{wst[i][2], wst[i][3]};
-            *reinterpret_cast<u32x4*>(ql + (srow + 32 * i) * QG_QROW + 16 * spc) = qst[i];
-        }
-        __syncthreads();
-        load(min(st + 1, stages - 1)); // (unconditional: past the end the last stage is fetched again and dropped)
+    for (int u = 0; u < DEPTH; ++u) load(min(u, stages - 1), u);
+    for (int st0 = 0; st0 < stages; st0 += DEPTH) {
 #pragma unroll
-        for (int ks = 0; ks < QG_K / 64; ++ks) {
-            i32x4 qf[4], wf[4];
-#pragma unroll
-            for (int tb = 0; tb < 4; ++tb)
-                qf[tb] = *reinterpret_cast<const i32x4*>(ql + (64 * wr + 16 * tb + l16) * QG_QROW + ks * 64 + 16 * g);
-            // (the byte-transposing read: see mla_qb_body)
-#pragma unroll
-            for (int nb = 0; nb < 4; ++nb) {
-                const uint8_t* p = wl + (ks * 64 + 16 * g + (l16 >> 1)) * MQROW + 64 * wc + 16 * nb + 8 * (l16 & 1);
-                const v2i lo = lds_read_tr8(p), hi = lds_read_tr8(p + 8 * MQROW);
-                wf[nb] = i32x4{lo[0], lo[1], hi[0], hi[1]};
+        for (int u = 0; u < DEPTH; ++u) {
+            if (st0 + u < stages) { // (uniform over the workgroup)
+                __syncthreads(); // everyone is done with the previous stage's tiles
+    #pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    u32x2* d = reinterpret_cast<u32x2*>(wl + (srow + 32 * i) * MQROW + 16 * spc);
+                    d[0] = u32x2{wst[u][i][0], wst[u][i][1]};
+                    d[1] = u32x2{wst[u][i][2], wst[u][i][3]};
+                    *reinterpret_cast<u32x4*>(ql + (srow + 32 * i) * QG_QROW + 16 * spc) = qst[u][i];
+                }
+                __syncthreads();
+                load(min(st0 + u + DEPTH, stages - 1), u); // (unconditional: past the end the last stage is fetched again and dropped)
+    #pragma unroll
+                for (int ks = 0; ks < QG_K / 64; ++ks) {
+                    i32x4 qf[4], wf[4];
+    #pragma unroll
+                    for (int tb = 0; tb < 4; ++tb)
+                        qf[tb] = *reinterpret_cast<const i32x4*>(ql + (64 * wr + 16 * tb + l16) * QG_QROW + ks * 64 + 16 * g);
+                    // (the byte-transposing read: see mla_qb_body)
+    #pragma unroll
+                    for (int nb = 0; nb < 4; ++nb) {
+                        const uint8_t* p = wl + (ks * 64 + 16 * g + (l16 >> 1)) * MQROW + 64 * wc + 16 * nb + 8 * (l16 & 1);
+                        const v2i lo = lds_read_tr8(p), hi = lds_read_tr8(p + 8 * MQROW);
+                        wf[nb] = i32x4{lo[0], lo[1], hi[0], hi[1]};
+                    }
+    #pragma unroll
+                    for (int nb = 0; nb < 4; ++nb)
+    #pragma unroll
+                        for (int tb = 0; tb < 4; ++tb)
+                            acc[nb][tb] = __builtin_amdgcn_mfma_i32_16x16x64_i8(wf[nb], qf[tb], acc[nb][tb], 0, 0, 0);
+                }
             }
-#pragma unroll
-            for (int nb = 0; nb < 4; ++nb)
-#pragma unroll
-                for (int tb = 0; tb < 4; ++tb)
-                    acc[nb][tb] = __builtin_amdgcn_mfma_i32_16x16x64_i8(wf[nb], qf[tb], acc[nb][tb], 0, 0, 0);
         }
     }
     __syncthreads(); // the operand tiles are free: the output tile takes their place
@@ -972,7 +982,11 @@ static hipError_t launch_prologs(const MlaPrologArgs& a, const PrologArgs* p, hi
                                4 * XA_K * XROW2, stream, a);
             hipLaunchKernelGGL(mla_qb16_epilogue_kernel, dim3(a.t, (nq / 4 + 255) / 256), dim3(256), 0, stream, a);
         } else if (big) {
-            hipLaunchKernelGGL(mla_qb_big_kernel, dim3(a.n * MQH / 128, (a.t + QG_TOK - 1) / QG_TOK), dim3(256), 0, stream, a);
+            const dim3 qgrid(a.n * MQH / 128, (a.t + QG_TOK - 1) / QG_TOK);
+            if (a.t <= BIG_T2)
+                hipLaunchKernelGGL(mla_qb_big_kernel<3>, qgrid, dim3(256), 0, stream, a);
+            else
+                hipLaunchKernelGGL(mla_qb_big_kernel<1>, qgrid, dim3(256), 0, stream, a);
             if (p) hipLaunchKernelGGL(fused_q_only_kernel, dim3(p->n, ttiles), dim3(1024), prolog_q_lds_bytes(a.r), stream, *p);
         } else if (p) {
             const int smem = mla_qb_lds_bytes(a.r) > prolog_q_lds_bytes(a.r) ? mla_qb_lds_bytes(a.r) : prolog_q_lds_bytes(a.r);
