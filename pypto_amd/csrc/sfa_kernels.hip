@@ -32,6 +32,7 @@
 #include "common.h"
 #include "kernels.h"
 #include "timing.h"
+#include <type_traits>
 
 namespace pto {
 namespace {
@@ -55,23 +56,22 @@ constexpr int NR_PR = 4;
 constexpr int S_AHEAD = 2, PV_AHEAD = 1;
 constexpr int NPARK_SM = KSTEPS / 2 - NREG_SM, NPARK_PR = KSTEPS / 2 - NREG_PR;
 // LDS layout: two tile stages | partial S, 4 KB per head group | P~, 2 KB per head group | rescale factors [4][32],
-// row sums [128], flags [4] | parked Q | per-split arrays sized by SfaArgs::split_cap (validity words, rows) |
+// flags [4] | parked Q | per-split arrays sized by SfaArgs::split_cap (validity words, rows) |
 // this sequence's page table (when it fits)
 constexpr int XBUF_OFF = 2 * STAGE;
 constexpr int PBUF_OFF = XBUF_OFF + 4 * 4096;
 constexpr int ALPHA_OFF = PBUF_OFF + 4 * 2048;
-constexpr int LSUM_OFF = ALPHA_OFF + 4 * 32 * 4;
-constexpr int FLAG_OFF = LSUM_OFF + HEADS_PER_WG * 4;
+constexpr int FLAG_OFF = ALPHA_OFF + 4 * 32 * 4;
 constexpr int QPARK_OFF = FLAG_OFF + 16;
 constexpr int SPLIT_OFF = QPARK_OFF + 4 * (NPARK_SM + NPARK_PR) * 1024;
 constexpr int LDS_LIMIT = 160 * 1024;
-constexpr int OUT_ROW = DN * 4;  // epilogue staging: 64 heads x 512 fp32 per pass, reusing the front of LDS
-constexpr int OUT_HEADS = 64;
+constexpr int OUT_ROW = DN * 2;  // epilogue staging: 128 heads x 512 values of 16 bits, reusing the front of LDS
+constexpr int OUT_LSUM_OFF = HEADS_PER_WG * OUT_ROW; // the epilogue's row sums, behind the staging area (in the parked Q, dead by then)
 constexpr int QPITCH = 272;      // start-up staging of Q: 128 heads x 256 bytes per round, padded against bank conflicts
 static_assert(HEADS_PER_WG * QPITCH <= STAGE, "a round of Q fits one tile stage");
 __host__ __device__ constexpr int tmask_bytes(int cap) { return (cap / T + 2) * 4; }
 __host__ __device__ constexpr int split_bytes(int cap) { return tmask_bytes(cap) + cap * 4; }
-static_assert(OUT_HEADS * OUT_ROW <= LDS_LIMIT, "epilogue staging must fit");
+static_assert(OUT_LSUM_OFF >= QPARK_OFF && OUT_LSUM_OFF + HEADS_PER_WG * 4 <= SPLIT_OFF, "the epilogue's row sums lie in the parked Q, which nothing reads after the last tile's scores");
 static_assert(QPARK_OFF % 16 == 0 && SPLIT_OFF % 16 == 0, "16-byte LDS accesses");
 static_assert(SPLIT_OFF + split_bytes(MAX_SPLIT_TOKENS) <= LDS_LIMIT, "a whole top-k list must fit one workgroup");
 
@@ -615,11 +615,15 @@ __device__ __forceinline__ void sfa_wave(const SfaArgs& a, uint8_t* smem, uint32
         }
     }
 
-    // Epilogue.  The softmax waves publish the row sums; then, 64 heads at a time, the O^T blocks go to LDS as
-    // [head][512] fp32 rows (everything but the split arrays is free now), 16-byte chunks XOR-swizzled with the
-    // head so that the 8 lanes of a b128 write hit distinct banks, and all 512 lanes copy the rows out.  Register r of
-    // o[i][hb] holds dim 32*(4*dq + i) + 8*(r/4) + 4*hl + r%4 of head 64*hh + 32*hb + l32.
-    float* lsum = reinterpret_cast<float*>(smem + LSUM_OFF);
+    // Epilogue.  The softmax waves publish the row sums (in a part of LDS the staging area below does not reach); then
+    // every wave normalises its O^T blocks, rounds them to the output's 16-bit type and stages them in LDS as
+    // [head][512] rows of 1024 bytes (everything below OUT_LSUM_OFF is free now), and all 512 lanes copy the rows out,
+    // a wavefront writing one whole row per instruction.  Register r of o[i][hb] holds dim
+    // 32*(4*dq + i) + 8*(r/4) + 4*hl + r%4 of head 64*hh + 32*hb + l32: four consecutive dims, and the other half-wave
+    // holds the four next to them.  v_permlane32_swap pairs them up - the lower half-wave ends up with the 8 dims of
+    // block g = 2 gp, the upper one with those of block 2 gp + 1 - so that a lane stores 16 bytes; the 16-byte chunks
+    // of a row are XOR-swizzled with the head so that the 8 lanes of a b128 access hit distinct banks.
+    float* lsum = reinterpret_cast<float*>(smem + OUT_LSUM_OFF);
     if (KH == 0) {
         const float l_tot = l_run + __shfl_xor(l_run, 32);
         if (hl == 0) lsum[hg * 32 + l32] = s_active ? l_tot : 0.f;
@@ -629,55 +633,66 @@ __device__ __forceinline__ void sfa_wave(const SfaArgs& a, uint8_t* smem, uint32
             a.part_ml[prow * 2 + 1] = l_tot;
         }
     }
-    __syncthreads();
-    float mul[2]; // splits hand over their normalised output as well
+    __syncthreads(); // row sums published; nobody reads a tile, P~ or parked Q any more
+    const bool final_out = a.nsplit == 1; // bf16 output; otherwise the split's share, normalised by its own sum, in fp16:
+                                          // |value| <= max |V| and 2^-11 relative rounding, a quarter of the final bf16
+                                          // rounding, half the bytes of fp32 for this kernel to write and the merge to read
+    // (one copy of the staging code per output type: a test of the type inside it ends up as a branch per value pair)
+    auto stage_out = [&](auto as_final) {
+        constexpr bool FINAL = decltype(as_final)::value;
 #pragma unroll
-    for (int hb = 0; hb < 2; ++hb) {
-        const float l = lsum[(2 * hh + hb) * 32 + l32];
-        mul[hb] = l > 0.f ? 1.f / l : 0.f;
+        for (int hb = 0; hb < 2; ++hb) {
+            const int hrow = 64 * hh + 32 * hb + l32;
+            const float l = lsum[hrow];
+            const float mul = l > 0.f ? 1.f / l : 0.f;
+            uint8_t* orow = smem + hrow * OUT_ROW;
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+#pragma unroll
+                for (int gp = 0; gp < 2; ++gp) {
+                    uint32_t w[2][2]; // [block 2 gp, 2 gp + 1][pair of dims]
+#pragma unroll
+                    for (int g = 0; g < 2; ++g)
+#pragma unroll
+                        for (int k = 0; k < 2; ++k) {
+                            const float x = o[i][hb][4 * (2 * gp + g) + 2 * k] * mul, y = o[i][hb][4 * (2 * gp + g) + 2 * k + 1] * mul;
+                            if constexpr (FINAL) {
+                                w[g][k] = pack_bf16x2(x, y);
+                            } else {
+                                typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
+                                w[g][k] = __builtin_bit_cast(uint32_t, f16x2{(_Float16)x, (_Float16)y});
+                            }
+                        }
+                    // the swap exchanges the upper half-wave of its first operand with the lower half-wave of its second
+                    const auto s0 = __builtin_amdgcn_permlane32_swap(w[0][0], w[1][0], false, false);
+                    const auto s1 = __builtin_amdgcn_permlane32_swap(w[0][1], w[1][1], false, false);
+                    const int c = 4 * (4 * dq + i) + 2 * gp + hl;
+                    *reinterpret_cast<u32x4*>(orow + ((c ^ (hrow & 7)) << 4)) = u32x4{(uint32_t)s0[0], (uint32_t)s1[0], (uint32_t)s0[1], (uint32_t)s1[1]};
+                }
+        }
+    };
+    if (pv_active) {
+        if (final_out)
+            stage_out(std::true_type{});
+        else
+            stage_out(std::false_type{});
     }
-    __syncthreads(); // the staging area covers the row sums
-#pragma unroll
-    for (int pass = 0; pass < 2; ++pass) {
-        if (hh == pass) {
-#pragma unroll
-            for (int hb = 0; hb < 2; ++hb) {
-                const int hrow = hb * 32 + l32;
-                uint8_t* orow = smem + hrow * OUT_ROW;
-#pragma unroll
-                for (int i = 0; i < 4; ++i)
-#pragma unroll
-                    for (int g = 0; g < 4; ++g) {
-                        const int c = 8 * (4 * dq + i) + 2 * g + hl;
-                        const f32x4 v = {o[i][hb][4 * g] * mul[hb], o[i][hb][4 * g + 1] * mul[hb], o[i][hb][4 * g + 2] * mul[hb],
-                                         o[i][hb][4 * g + 3] * mul[hb]};
-                        *reinterpret_cast<f32x4*>(orow + ((c ^ (hrow & 7)) << 4)) = v;
-                    }
-            }
-        }
-        __syncthreads();
-        // a wavefront writes 512 B (bf16 output or fp16 partial) of one row per instruction
+    __syncthreads();
 #pragma unroll 4
-        for (int id = tid; id < OUT_HEADS * (DN / 4); id += 512) {
-            const int hrow = id / (DN / 4), c = id % (DN / 4);
-            const int oh = head0 + pass * OUT_HEADS + hrow;
-            if (oh >= a.nq) continue;
-            const f32x4 v = *reinterpret_cast<const f32x4*>(smem + hrow * OUT_ROW + ((c ^ (hrow & 7)) << 4));
-            if (a.nsplit == 1) {
-                const u32x2 w = {pack_bf16x2(v[0], v[1]), pack_bf16x2(v[2], v[3])};
-                *reinterpret_cast<u32x2*>(reinterpret_cast<uint8_t*>(a.out) + (((int64_t)tq * a.nq + oh) * DN + c * 4) * 2) = w;
-            } else {
-                // a split's share, normalised by its own sum, in fp16: |value| <= max |V| and 2^-11 relative rounding, a
-                // quarter of the final bf16 rounding; half the bytes of fp32 for this kernel to write and the merge to read
-                const int64_t prow = ((int64_t)tq * a.nsplit + sp) * a.nq + oh;
-                const f16x4 hv = {(_Float16)v[0], (_Float16)v[1], (_Float16)v[2], (_Float16)v[3]};
-                // (streaming stores: 34 MB leave the chip's 256 workgroups at once and are read back once by the merge;
-                // kept out of the caches they cost this kernel 1.5 us less, and the next step's index cache stream finds
-                // the caches free of them)
-                __builtin_nontemporal_store(hv, reinterpret_cast<f16x4*>(a.part_o + prow * DN + c * 4));
-            }
+    for (int id = tid; id < HEADS_PER_WG * (DN / 8); id += 512) {
+        const int hrow = id / (DN / 8), c = id % (DN / 8);
+        const int oh = head0 + hrow;
+        if (oh >= a.nq) break; // (wave-uniform: a wavefront copies one row)
+        const u32x4 v = *reinterpret_cast<const u32x4*>(smem + hrow * OUT_ROW + ((c ^ (hrow & 7)) << 4));
+        if (final_out) {
+            *reinterpret_cast<u32x4*>(reinterpret_cast<uint8_t*>(a.out) + (((int64_t)tq * a.nq + oh) * DN + c * 8) * 2) = v;
+        } else {
+            // (streaming stores: 34 MB leave the chip's 256 workgroups at once and are read back once by the merge;
+            // kept out of the caches they cost this kernel 1.5 us less, and the next step's index cache stream finds
+            // the caches free of them)
+            const int64_t prow = ((int64_t)tq * a.nsplit + sp) * a.nq + oh;
+            __builtin_nontemporal_store(v, reinterpret_cast<u32x4*>(a.part_o + prow * DN + c * 8));
         }
-        if (pass == 0) __syncthreads();
     }
 }
 
@@ -829,7 +844,6 @@ hipError_t sfa_launch(const SfaArgs& a, hipStream_t stream)
     int smem_bytes = SPLIT_OFF + split_bytes(args.split_cap);
     args.bt_cached = smem_bytes + a.bt_stride * 4 <= LDS_LIMIT ? 1 : 0;
     if (args.bt_cached) smem_bytes += a.bt_stride * 4;
-    if (smem_bytes < OUT_HEADS * OUT_ROW) smem_bytes = OUT_HEADS * OUT_ROW; // epilogue staging
     static DeviceOnce attr_done[2];
     auto kern = a.quant ? sfa_decode_kernel<true> : sfa_decode_kernel<false>;
     {
