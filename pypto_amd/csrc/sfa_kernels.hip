@@ -120,29 +120,53 @@ __device__ __forceinline__ uint64_t row_offset(uint32_t row, uint32_t stride)
 // rows[] holds valid cache rows only (absent entries point at row 0); the tile's validity word says which rows are
 // absent, and their data is zeroed when it is consumed, so that no load depends on it.  All loads are unconditional.
 // The share is rows pair0 + E0 .. pair0 + E0 + NR - 1 of the tile, pair0 a multiple of 8.
+template <int NR>
+struct RowRefs {
+    uint64_t off[NR];  // byte offsets of the share's rows in the nope cache (scalar registers)
+    uint32_t rope_row; // this lane's row for the rope columns
+    uint32_t sc_row;   // this lane's row for the scales
+};
 template <bool QUANT, int NR, int E0>
-__device__ __forceinline__ void load_raw(RawTile<QUANT, NR>& r, const SfaArgs& a, const int* rows, int tile, int pair0,
-                                         int lane, int tid)
+__device__ __forceinline__ void prepare_rows(RowRefs<NR>& f, const SfaArgs& a, const int* rows, int tile, int pair0, int lane, int tid)
 {
     // the pair's eight rows are the same for every lane: two 16-byte LDS reads, then scalar address arithmetic
     const u32x4 ra = *reinterpret_cast<const u32x4*>(rows + tile * T + pair0);
     const u32x4 rb = *reinterpret_cast<const u32x4*>(rows + tile * T + pair0 + 4);
+    f.rope_row = (uint32_t)rows[tile * T + (tid >> 4)];
+    if constexpr (QUANT) {
+        const int l = lane < 4 * NR ? lane : 0;
+        f.sc_row = (uint32_t)rows[tile * T + pair0 + E0 + (l >> 2)];
+    }
 #pragma unroll
     for (int e = 0; e < NR; ++e) {
         const uint32_t row = __builtin_amdgcn_readfirstlane(E0 + e < 4 ? ra[(E0 + e) & 3] : rb[(E0 + e) & 3]);
-        const uint8_t* rp = a.kn + row_offset(row, a.kn_stride);
+        f.off[e] = row_offset(row, a.kn_stride);
+    }
+}
+template <bool QUANT, int NR>
+__device__ __forceinline__ void issue_raw(RawTile<QUANT, NR>& r, const RowRefs<NR>& f, const SfaArgs& a, int lane, int tid)
+{
+#pragma unroll
+    for (int e = 0; e < NR; ++e) {
+        const uint8_t* rp = a.kn + f.off[e];
         if constexpr (QUANT)
             r.nope[e] = *reinterpret_cast<const u32x2*>(rp + lane * 8);
         else
             r.nope[e] = *reinterpret_cast<const u32x4*>(rp + lane * 16);
     }
-    const uint32_t row = (uint32_t)rows[tile * T + (tid >> 4)];
-    r.rope = *reinterpret_cast<const u32x2*>(a.kr + (uint64_t)row * a.kr_stride + (tid & 15) * 8);
+    r.rope = *reinterpret_cast<const u32x2*>(a.kr + (uint64_t)f.rope_row * a.kr_stride + (tid & 15) * 8);
     if constexpr (QUANT) {
         const int l = lane < 4 * NR ? lane : 0;
-        const uint32_t srow = (uint32_t)rows[tile * T + pair0 + E0 + (l >> 2)];
-        r.sc = *reinterpret_cast<const float*>(a.ks + (uint64_t)srow * a.ks_stride + (l & 3) * 4);
+        r.sc = *reinterpret_cast<const float*>(a.ks + (uint64_t)f.sc_row * a.ks_stride + (l & 3) * 4);
     }
+}
+template <bool QUANT, int NR, int E0>
+__device__ __forceinline__ void load_raw(RawTile<QUANT, NR>& r, const SfaArgs& a, const int* rows, int tile, int pair0,
+                                         int lane, int tid)
+{
+    RowRefs<NR> f;
+    prepare_rows<QUANT, NR, E0>(f, a, rows, tile, pair0, lane, tid);
+    issue_raw<QUANT, NR>(r, f, a, lane, tid);
 }
 
 // int8 -> fp32 -> * scale with one conversion and one fma per element: byte k of w holds x + 128 (the caller
@@ -504,6 +528,8 @@ __device__ __forceinline__ void sfa_wave(const SfaArgs& a, uint8_t* smem, uint32
     for (int it = 0; it < ntiles; ++it) {
         uint8_t* stage = smem + (it & 1) * STAGE;
         const uint32_t valid = __builtin_amdgcn_readfirstlane(tmask[it]);
+        RowRefs<NR> next_rows; // of the tile after next, looked up under the score MFMAs
+        prepare_rows<QUANT, NR, E0>(next_rows, a, rows, min(it + 2, last), pair0, lane, tid);
         f32x16 s;
         if (s_active) s_partial<NREG, KH>(s, stage, s_off, q, qpark);
         if (KH == 1 && s_active) {
@@ -569,7 +595,7 @@ __device__ __forceinline__ void sfa_wave(const SfaArgs& a, uint8_t* smem, uint32
             // the next tile: out of the registers into the other stage, then the gather of the tile after
             const int nx = min(it + 1, last);
             dequant_store<QUANT, NR>(raw, smem + ((it + 1) & 1) * STAGE, __builtin_amdgcn_readfirstlane(tmask[nx]), row0, lane, tid);
-            load_raw<QUANT, NR, E0>(raw, a, rows, min(it + 2, last), pair0, lane, tid);
+            issue_raw<QUANT, NR>(raw, next_rows, a, lane, tid);
         }
         __syncthreads(); // P~ and the next tile are in LDS
         if (pv_active && valid != 0u) {
