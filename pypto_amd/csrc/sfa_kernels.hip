@@ -67,8 +67,8 @@ constexpr int SPLIT_OFF = QPARK_OFF + 4 * (NPARK_SM + NPARK_PR) * 1024;
 constexpr int LDS_LIMIT = 160 * 1024;
 constexpr int OUT_ROW = DN * 2;  // epilogue staging: 128 heads x 512 values of 16 bits, reusing the front of LDS
 constexpr int OUT_LSUM_OFF = HEADS_PER_WG * OUT_ROW; // the epilogue's row sums, behind the staging area (in the parked Q, dead by then)
-constexpr int QPITCH = 272;      // start-up staging of Q: 128 heads x 256 bytes per round, padded against bank conflicts
-static_assert(HEADS_PER_WG * QPITCH <= STAGE, "a round of Q fits one tile stage");
+constexpr int QROW = KROW;       // start-up staging of Q: 128 heads x 1152 bytes
+static_assert(HEADS_PER_WG * QROW <= SPLIT_OFF, "the query of 128 heads fits below the per-split arrays");
 __host__ __device__ constexpr int tmask_bytes(int cap) { return (cap / T + 2) * 4; }
 __host__ __device__ constexpr int split_bytes(int cap) { return tmask_bytes(cap) + cap * 4; }
 static_assert(OUT_LSUM_OFF >= QPARK_OFF && OUT_LSUM_OFF + HEADS_PER_WG * 4 <= SPLIT_OFF, "the epilogue's row sums lie in the parked Q, which nothing reads after the last tile's scores");
@@ -426,8 +426,7 @@ __device__ __forceinline__ void sfa_wave(const SfaArgs& a, uint8_t* smem, uint32
 
     // Q into operand layout: this lane's head (hg, l32) and its slice - the 16 k-steps of nope columns
     // [256 KH, 256 KH + 256) and the 2 of rope columns [32 KH, 32 KH + 32); B operand layout: head = column, 8
-    // consecutive k per half-wave.  Five rounds through the two (still unused) tile stages, alternately: a round's
-    // 128 columns of all heads are written row-major (pitch QPITCH) while the round before is read.
+    // consecutive k per half-wave.  One trip through LDS (all of it below the per-split arrays is still unused).
     bf16x8 q[NREG];
     uint8_t* qpark = smem + QPARK_OFF + (KH ? 4 * NPARK_SM * 1024 + hg * (NPARK_PR * 1024) : hg * (NPARK_SM * 1024)) + lane * 16;
     {
@@ -435,49 +434,41 @@ __device__ __forceinline__ void sfa_wave(const SfaArgs& a, uint8_t* smem, uint32
         // taken on the raw scores, which needs a factor that commutes with max)
         const uint32_t f = a.softmax_scale < 0.f ? 0x80008000u : 0u;
         const u32x4 qflip = {f, f, f, f};
-        auto keep = [&](int i, u32x4 w) { // k-step i of this wave's 18
-            const bf16x8 v = __builtin_bit_cast(bf16x8, w ^ qflip);
+        // all 128 heads' rows at once: row h at h * QROW, its 72 16-byte chunks (64 nope, 8 rope) XOR-swizzled with h
+        // so that the 8 lanes of a b128 access hit distinct banks although a row is a multiple of 128 bytes
+#pragma unroll
+        for (int r = 0; r < 4; ++r)
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const int pp = tid + 512 * j, h = pp >> 4, c = 16 * r + (pp & 15);
+                *reinterpret_cast<u32x4*>(smem + h * QROW + ((c ^ (h & 7)) << 4)) = qraw[r][j];
+            }
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+            const int pp = tid + 512 * j, h = pp >> 3, c = 64 + (pp & 7);
+            *reinterpret_cast<u32x4*>(smem + h * QROW + ((c ^ (h & 7)) << 4)) = qraw_rope[j];
+        }
+        __syncthreads();
+        // k-step i of this wave's 18: nope chunks 2 (16 KH + i) + hl, rope chunks 64 + 2 (2 KH + i - 16) + hl
+        u32x4 qa[KSTEPS / 2];
+        {
+            const int h = hg * 32 + l32;
+            const uint8_t* row = smem + h * QROW;
+#pragma unroll
+            for (int i = 0; i < KSTEPS / 2; ++i) {
+                const int c = (i < 16 ? 2 * (16 * KH + i) : 64 + 2 * (2 * KH + i - 16)) + hl;
+                qa[i] = *reinterpret_cast<const u32x4*>(row + ((c ^ (h & 7)) << 4)) ^ qflip;
+            }
+        }
+        __syncthreads(); // every wave has its fragments: the rows' space is free for the parked fragments and the tiles
+#pragma unroll
+        for (int i = 0; i < KSTEPS / 2; ++i) {
+            const bf16x8 v = __builtin_bit_cast(bf16x8, qa[i]);
             if (i < NREG)
                 q[i < NREG ? i : 0] = v;
             else
                 *reinterpret_cast<bf16x8*>(qpark + (i - NREG) * 1024) = v;
-        };
-        auto put = [&](int r) {
-            uint8_t* buf = smem + (r & 1) * STAGE;
-            if (r < 4) {
-#pragma unroll
-                for (int j = 0; j < 4; ++j) {
-                    const int p = tid + 512 * j;
-                    *reinterpret_cast<u32x4*>(buf + (p >> 4) * QPITCH + (p & 15) * 16) = qraw[r < 4 ? r : 0][j];
-                }
-            } else {
-#pragma unroll
-                for (int j = 0; j < 2; ++j) {
-                    const int p = tid + 512 * j;
-                    *reinterpret_cast<u32x4*>(buf + (p >> 3) * QPITCH + (p & 7) * 16) = qraw_rope[j];
-                }
-            }
-        };
-        auto take = [&](int r) {
-            const uint8_t* row = smem + (r & 1) * STAGE + (hg * 32 + l32) * QPITCH + hl * 16;
-            if (r < 4) {
-                if ((r >> 1) == KH) {
-#pragma unroll
-                    for (int kk = 0; kk < 8; ++kk) keep(8 * (r & 1) + kk, *reinterpret_cast<const u32x4*>(row + kk * 32));
-                }
-            } else {
-#pragma unroll
-                for (int j = 0; j < 2; ++j) keep(16 + j, *reinterpret_cast<const u32x4*>(row + (2 * KH + j) * 32));
-            }
-        };
-        put(0);
-#pragma unroll
-        for (int r = 0; r < 5; ++r) {
-            __syncthreads();
-            take(r);
-            if (r + 1 < 5) put(r + 1);
         }
-        __syncthreads(); // the stages are free for the tiles
     }
     if (ntiles > 0) {
         dequant_store<QUANT, NR>(raw, smem, __builtin_amdgcn_readfirstlane(tmask[0]), row0, lane, tid);
