@@ -782,14 +782,6 @@ __global__ __launch_bounds__(1024) void fused_qb_kernel(MlaPrologArgs m, PrologA
         prolog_q_body(p, blockIdx.x - nqb, blockIdx.y * PTOK, fq_lds);
 }
 
-// At prefill sizes the MLA side of that launch is mla_qb_big_kernel; this is the indexer side on its own.
-// grid (index heads, token tiles of 32), 1024 lanes
-__global__ __launch_bounds__(1024) void fused_q_only_kernel(PrologArgs p)
-{
-    extern __shared__ __align__(16) uint8_t fq_lds[];
-    prolog_q_body(p, blockIdx.x, blockIdx.y * PTOK, fq_lds);
-}
-
 // ------------------------------------------------------------------------------------------------ q_b[:, head, :128] @ w_uk[head]
 // grid (heads, 512 / 128, z), 256 lanes: wave w owns outputs [32 w, 32 w + 32) of the tile.  The head's 128 x 128 weight
 // tile stays in LDS while the workgroup walks the token tiles z, z + gridDim.z, ... (one at decode sizes; at prefill
@@ -940,9 +932,6 @@ static hipError_t set_lds_limits()
         if (e != hipSuccess) return e;
         e = hipFuncSetAttribute(reinterpret_cast<const void*>(fused_qb_kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
                                 mla_qb_lds_bytes(MAX_R) > prolog_q_lds_bytes(QMAX_R) ? mla_qb_lds_bytes(MAX_R) : prolog_q_lds_bytes(QMAX_R));
-        if (e != hipSuccess) return e;
-        e = hipFuncSetAttribute(reinterpret_cast<const void*>(fused_q_only_kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
-                                prolog_q_lds_bytes(QMAX_R));
         return e;
     });
 }
@@ -987,7 +976,13 @@ static hipError_t launch_prologs(const MlaPrologArgs& a, const PrologArgs* p, hi
                 hipLaunchKernelGGL(mla_qb_big_kernel<3>, qgrid, dim3(256), 0, stream, a);
             else
                 hipLaunchKernelGGL(mla_qb_big_kernel<1>, qgrid, dim3(256), 0, stream, a);
-            if (p) hipLaunchKernelGGL(fused_q_only_kernel, dim3(p->n, ttiles), dim3(1024), prolog_q_lds_bytes(a.r), stream, *p);
+            if (p) {
+                const dim3 pgrid(p->n, (a.t + QB_TOK - 1) / QB_TOK);
+                if (a.t <= PROLOG_DEEP_T)
+                    hipLaunchKernelGGL(prolog_q_big_kernel<3>, pgrid, dim3(256), 0, stream, *p);
+                else
+                    hipLaunchKernelGGL(prolog_q_big_kernel<1>, pgrid, dim3(256), 0, stream, *p);
+            }
         } else if (p) {
             const int smem = mla_qb_lds_bytes(a.r) > prolog_q_lds_bytes(a.r) ? mla_qb_lds_bytes(a.r) : prolog_q_lds_bytes(a.r);
             hipLaunchKernelGGL(fused_qb_kernel, dim3(a.n * MQH / 128 + p->n, ttiles), dim3(1024), smem, stream, a, *p);

@@ -246,6 +246,197 @@ __device__ __forceinline__ void prolog_q_body(const PrologArgs& a, int head, int
     }
 }
 
+// ------------------------------------------------------------------------------------------------ query path, prefill sizes
+// The same product for 128 tokens and more: a workgroup of 256 lanes owns (head, 128 tokens) and walks the contraction
+// in stages of 128 rows, both operands staged through LDS with the loads of the next DEPTH stages in flight.  Wave
+// (wr, wc) owns tokens [64 wr, +64) x dims [64 wc, +64): every operand fragment read from LDS feeds four MFMAs, and the
+// head's weight slice is fetched once per 128 tokens instead of once per 32.  Then, in LDS, for all 128 tokens: scale
+// and round to bf16, rotary, hadamard (wave w: outputs [32 w, +32) of all tokens, every hadamard fragment feeding four
+// MFMAs), quantisation.  The int32 sums are exact and the rest is the same operations in the same order, so the
+// results are the bits of prolog_q_body's.
+constexpr int QB_TOK = 128;
+constexpr int QB_QROW = QK + 16; // bytes per LDS row of the [token][k] int8 tile (padded against bank conflicts)
+constexpr int QB_STAGE_BYTES = QK * QROW + QB_TOK * QB_QROW;
+constexpr int QB_EPI_BYTES = PD * PD * 2 + QB_TOK * XROW + 4 * QB_TOK * 4; // hadamard_q | bf16 tile | per-wave maxima
+constexpr int QB_LDS_BYTES = QB_EPI_BYTES > QB_STAGE_BYTES ? QB_EPI_BYTES : QB_STAGE_BYTES;
+
+template <int DEPTH>
+__global__ __launch_bounds__(256, 2) void prolog_q_big_kernel(PrologArgs a)
+{
+#pragma clang fp contract(off)
+    __shared__ __align__(16) uint8_t lds[QB_LDS_BYTES];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int l16 = lane & 15, g = lane >> 4, l32 = lane & 31, hl = lane >> 5, wr = wave >> 1, wc = wave & 1;
+    const int r = a.r, head = blockIdx.x, tok0 = blockIdx.y * QB_TOK;
+    const int64_t nd = (int64_t)a.n * PD;
+    uint8_t* wl = lds;
+    uint8_t* ql = lds + QK * QROW;
+    const int stages = r / QK;
+    // 128 rows x 128 bytes of either operand per stage = 4 pieces of 16 bytes per lane (rows tid / 8 + 32 i, piece tid % 8)
+    const int srow = tid >> 3, spc = tid & 7;
+    const int8_t* wp = a.w_qb + (int64_t)srow * nd + head * PD + 16 * spc;
+    const int8_t* qp[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) qp[i] = a.q_norm + (int64_t)min(tok0 + srow + 32 * i, a.t - 1) * r + 16 * spc;
+    u32x4 wst[DEPTH][4], qst[DEPTH][4];
+    auto load = [&](int st, int u) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) qst[u][i] = *reinterpret_cast<const u32x4*>(qp[i] + st * QK);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) wst[u][i] = *reinterpret_cast<const u32x4*>(wp + ((int64_t)st * QK + 32 * i) * nd);
+    };
+    // the epilogue's scales, requested first
+    float qs_pre[4];
+    f32x4 ws_pre[4];
+#pragma unroll
+    for (int tb = 0; tb < 4; ++tb) qs_pre[tb] = a.q_norm_scale[min(tok0 + 64 * wr + 16 * tb + l16, a.t - 1)];
+#pragma unroll
+    for (int nb = 0; nb < 4; ++nb) ws_pre[nb] = *reinterpret_cast<const f32x4*>(a.w_qb_scale + (int64_t)head * PD + 64 * wc + 16 * nb + 4 * g);
+    i32x4 acc[4][4]; // [nb][tb]
+#pragma unroll
+    for (int nb = 0; nb < 4; ++nb)
+#pragma unroll
+        for (int tb = 0; tb < 4; ++tb) acc[nb][tb] = i32x4{0, 0, 0, 0};
+#pragma unroll
+    for (int u = 0; u < DEPTH; ++u) load(min(u, stages - 1), u);
+    for (int st0 = 0; st0 < stages; st0 += DEPTH) {
+#pragma unroll
+        for (int u = 0; u < DEPTH; ++u) {
+            if (st0 + u < stages) { // (uniform over the workgroup)
+                __syncthreads();    // everyone is done with the previous stage's tiles
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    u32x2* d = reinterpret_cast<u32x2*>(wl + (srow + 32 * i) * QROW + 16 * spc);
+                    d[0] = u32x2{wst[u][i][0], wst[u][i][1]};
+                    d[1] = u32x2{wst[u][i][2], wst[u][i][3]};
+                    *reinterpret_cast<u32x4*>(ql + (srow + 32 * i) * QB_QROW + 16 * spc) = qst[u][i];
+                }
+                __syncthreads();
+                load(min(st0 + u + DEPTH, stages - 1), u); // (unconditional: past the end the last stage is fetched again and dropped)
+#pragma unroll
+                for (int ks = 0; ks < QK / 64; ++ks) {
+                    i32x4 qf[4], wf[4];
+#pragma unroll
+                    for (int tb = 0; tb < 4; ++tb)
+                        qf[tb] = *reinterpret_cast<const i32x4*>(ql + (64 * wr + 16 * tb + l16) * QB_QROW + ks * 64 + 16 * g);
+                    // (the byte-transposing read: see prolog_q_body)
+#pragma unroll
+                    for (int nb = 0; nb < 4; ++nb) {
+                        const uint8_t* p = wl + (ks * 64 + 16 * g + (l16 >> 1)) * QROW + 64 * wc + 16 * nb + 8 * (l16 & 1);
+                        const v2i lo = lds_read_tr8(p), hi = lds_read_tr8(p + 8 * QROW);
+                        wf[nb] = i32x4{lo[0], lo[1], hi[0], hi[1]};
+                    }
+#pragma unroll
+                    for (int nb = 0; nb < 4; ++nb)
+#pragma unroll
+                        for (int tb = 0; tb < 4; ++tb)
+                            acc[nb][tb] = __builtin_amdgcn_mfma_i32_16x16x64_i8(wf[nb], qf[tb], acc[nb][tb], 0, 0, 0);
+                }
+            }
+        }
+    }
+    __syncthreads(); // the operand tiles are free: hadamard_q and the bf16 tile take their place
+    uint8_t* had = lds;
+    uint8_t* xt = lds + PD * PD * 2;
+    float(*smax)[QB_TOK] = reinterpret_cast<float(*)[QB_TOK]>(lds + PD * PD * 2 + QB_TOK * XROW);
+#pragma unroll
+    for (int i = 0; i < PD * PD * 2 / 16 / 256; ++i) reinterpret_cast<u32x4*>(had)[tid + 256 * i] = reinterpret_cast<const u32x4*>(a.had_q)[tid + 256 * i];
+    // register e of acc[nb][tb]: dim 64 wc + 16 nb + 4 g + e, token 64 wr + 16 tb + l16
+#pragma unroll
+    for (int tb = 0; tb < 4; ++tb) {
+        const int tl = 64 * wr + 16 * tb + l16;
+        const float qs = qs_pre[tb];
+#pragma unroll
+        for (int nb = 0; nb < 4; ++nb) {
+            const int dim = 64 * wc + 16 * nb + 4 * g;
+            const f32x4 ws = ws_pre[nb];
+            uint16_t vb[4];
+#pragma unroll
+            for (int e = 0; e < 4; ++e) vb[e] = f32_to_bf16(((float)acc[nb][tb][e] * qs) * ws[e]);
+            *reinterpret_cast<u32x2*>(xt + tl * XROW + dim * 2) = u32x2{(uint32_t)vb[0] | ((uint32_t)vb[1] << 16), (uint32_t)vb[2] | ((uint32_t)vb[3] << 16)};
+        }
+    }
+    __syncthreads();
+    // rotary on the first 64 dims: 128 tokens x 32 pairs, 16 items per lane (the arithmetic of rope_tile)
+#pragma unroll 4
+    for (int it = 0; it < QB_TOK * 32 / 256; ++it) {
+        const int item = tid + 256 * it;
+        const int tok = item >> 5, i = item & 31;
+        uint16_t* row = reinterpret_cast<uint16_t*>(xt + tok * XROW);
+        const int64_t gtc = (int64_t)min(tok0 + tok, a.t - 1) * PROPE;
+        const uint16_t* cosp = a.cos + gtc;
+        const uint16_t* sinp = a.sin + gtc;
+        const float x1 = bf16_to_f32(row[i]), x2 = bf16_to_f32(row[i + 32]);
+        const float c1 = bf16_to_f32(cosp[i]), c2 = bf16_to_f32(cosp[i + 32]);
+        const float s1 = bf16_to_f32(sinp[i]), s2 = bf16_to_f32(sinp[i + 32]);
+        const float o1 = x1 * c1 + (-x2) * s1;
+        const float o2 = x2 * c2 + x1 * s2;
+        row[i] = f32_to_bf16(o1);
+        row[i + 32] = f32_to_bf16(o2);
+    }
+    __syncthreads();
+    // Y^T[n, token] = H^T[n, k] . X^T[k, token]: wave w owns n in [32 w, 32 w + 32) for the four blocks of 32 tokens
+    // (operand addressing as in prolog_q_body)
+    f32x16 y[4];
+#pragma unroll
+    for (int tb = 0; tb < 4; ++tb)
+#pragma unroll
+        for (int e = 0; e < 16; ++e) y[tb][e] = 0.f;
+    {
+        const int jj = lane & 15, mh = (lane >> 4) & 1;
+        const uint8_t* hp = had + (4 * hl + (jj >> 2)) * (PD * 2) + (32 * wave + 16 * mh + 4 * (jj & 3)) * 2;
+        const uint8_t* xp = xt + l32 * XROW + hl * 8;
+#pragma unroll
+        for (int ks = 0; ks < PD / 16; ++ks) {
+            const s16x4 lo = lds_read_tr(hp + ks * 16 * (PD * 2));
+            const s16x4 hi = lds_read_tr(hp + (ks * 16 + 8) * (PD * 2));
+            const bf16x8 av = __builtin_bit_cast(bf16x8, __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
+#pragma unroll
+            for (int tb = 0; tb < 4; ++tb) {
+                const u32x2 b0 = *reinterpret_cast<const u32x2*>(xp + 32 * tb * XROW + ks * 32);
+                const u32x2 b1 = *reinterpret_cast<const u32x2*>(xp + 32 * tb * XROW + ks * 32 + 16);
+                const bf16x8 bv = __builtin_bit_cast(bf16x8, u32x4{b0[0], b0[1], b1[0], b1[1]});
+                y[tb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(av, bv, y[tb], 0, 0, 0);
+            }
+        }
+    }
+    // register e of y[tb]: n = 32 w + 8 (e/4) + 4 hl + e%4, token 32 tb + l32.  Round to bf16, per-token absmax over the 128 n
+    float mx[4];
+#pragma unroll
+    for (int tb = 0; tb < 4; ++tb) {
+        mx[tb] = 0.f;
+#pragma unroll
+        for (int e = 0; e < 16; ++e) {
+            y[tb][e] = bf16_to_f32(f32_to_bf16(y[tb][e]));
+            mx[tb] = fmaxf(mx[tb], fabsf(y[tb][e]));
+        }
+        mx[tb] = fmaxf(mx[tb], __shfl_xor(mx[tb], 32));
+        if (hl == 0) smax[wave][32 * tb + l32] = mx[tb];
+    }
+    __syncthreads();
+#pragma unroll
+    for (int tb = 0; tb < 4; ++tb) {
+        const int tl = 32 * tb + l32;
+        const float m = fmaxf(fmaxf(smax[0][tl], smax[1][tl]), fmaxf(smax[2][tl], smax[3][tl]));
+        const float sq = quant_scale(m);
+        const int gt = tok0 + tl;
+        if (gt < a.t) {
+            int8_t* qo = a.q_int8 + ((int64_t)gt * a.n + head) * PD + 32 * wave + 4 * hl;
+#pragma unroll
+            for (int e4 = 0; e4 < 4; ++e4) {
+                uint32_t pk = 0;
+#pragma unroll
+                for (int e = 0; e < 4; ++e) pk |= ((uint32_t)(int)__builtin_rintf(y[tb][4 * e4 + e] * sq) & 0xffu) << (8 * e);
+                *reinterpret_cast<uint32_t*>(qo + 8 * e4) = pk;
+            }
+            if (wave == 0 && hl == 0) a.q_scale[(int64_t)gt * a.n + head] = __builtin_bit_cast(uint16_t, (_Float16)(1.0f / sq));
+        }
+    }
+}
+constexpr int PROLOG_BIG_T = 256;   // token count from which the query product runs per 128 tokens (below, its 64 x t / 128
+                                    // workgroups leave most of the chip idle and the kernel per 32 tokens is faster)
+constexpr int PROLOG_DEEP_T = 1024; // up to here at most two of its workgroups share a CU: three stages of loads in flight each
+
 // ------------------------------------------------------------------------------------------------ key path, weights
 __device__ __forceinline__ float block_sum128(float v, float* red)
 {

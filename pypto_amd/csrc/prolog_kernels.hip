@@ -38,8 +38,10 @@ namespace {
 __global__ __launch_bounds__(128) void prolog_k_kernel(PrologArgs a) { prolog_k_body(a, blockIdx.x); }
 
 // ------------------------------------------------------------------------------------------------ x @ [w_k | w_proj]
-// 256 lanes per (256 rows of the weights, token tile of 32): partial sums over those rows; wl is [256 k][nw] bf16,
-// nw = 128 + n
+// 256 lanes per (256 rows of the weights, token tile of 32 TB): partial sums over those rows; wl is [256 k][nw] bf16,
+// nw = 128 + n.  TB blocks of 32 tokens per workgroup: 1 at decode sizes; 4 at prefill sizes, where the weight rows are
+// then staged once per 128 tokens and every weight fragment read from LDS feeds four MFMAs.
+template <int TB>
 __device__ __forceinline__ void prolog_xw_body(const PrologArgs& a, int split, int tok0, uint8_t* wl)
 {
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -63,15 +65,31 @@ __device__ __forceinline__ void prolog_xw_body(const PrologArgs& a, int split, i
     const int nblocks = nw / 32; // 32-wide output blocks; wave w takes blocks w, w + 4
     const int jj = lane & 15, mh = (lane >> 4) & 1;
     // B operand: the transposing reads below hand lane half hl the contraction rows 8 hl .. 8 hl + 7 of every 16-row step,
-    // so B is one 16-byte load per step (32 bytes contiguous per token row and instruction)
-    const uint16_t* xp = a.x + (int64_t)min(tok0 + l32, a.t - 1) * a.h + kbase + hl * 8;
-    f32x16 acc[2];
+    // so B is one 16-byte load per step (32 bytes contiguous per token row and instruction), requested one step ahead
+    const uint16_t* xp[TB];
 #pragma unroll
-    for (int j = 0; j < 2; ++j)
+    for (int tb = 0; tb < TB; ++tb) xp[tb] = a.x + (int64_t)min(tok0 + 32 * tb + l32, a.t - 1) * a.h + kbase + hl * 8;
+    f32x16 acc[TB][2];
 #pragma unroll
-        for (int e = 0; e < 16; ++e) acc[j][e] = 0.f;
+    for (int tb = 0; tb < TB; ++tb)
+#pragma unroll
+        for (int j = 0; j < 2; ++j)
+#pragma unroll
+            for (int e = 0; e < 16; ++e) acc[tb][j][e] = 0.f;
+    u32x4 xv[TB];
+#pragma unroll
+    for (int tb = 0; tb < TB; ++tb) xv[tb] = *reinterpret_cast<const u32x4*>(xp[tb]);
     for (int ks = 0; ks < XW_K / 16; ++ks) {
-        const bf16x8 bv = __builtin_bit_cast(bf16x8, *reinterpret_cast<const u32x4*>(xp + ks * 16));
+        bf16x8 bv[TB];
+#pragma unroll
+        for (int tb = 0; tb < TB; ++tb) bv[tb] = __builtin_bit_cast(bf16x8, xv[tb]);
+        // (TB = 1 runs beside the query product in a 1024-lane launch, at 128 registers: no room for the step ahead,
+        // the load sits at the end of the step instead)
+        const int kn = min(ks + 1, XW_K / 16 - 1); // (past the end: the last step again, dropped)
+        if constexpr (TB > 1) {
+#pragma unroll
+            for (int tb = 0; tb < TB; ++tb) xv[tb] = *reinterpret_cast<const u32x4*>(xp[tb] + kn * 16);
+        }
 #pragma unroll
         for (int j = 0; j < 2; ++j) {
             const int nb = wave + 4 * j;
@@ -80,22 +98,27 @@ __device__ __forceinline__ void prolog_xw_body(const PrologArgs& a, int split, i
                 const s16x4 lo = lds_read_tr(hp);
                 const s16x4 hi = lds_read_tr(hp + 4 * rowb);
                 const bf16x8 av = __builtin_bit_cast(bf16x8, __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
-                acc[j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(av, bv, acc[j], 0, 0, 0);
+#pragma unroll
+                for (int tb = 0; tb < TB; ++tb) acc[tb][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(av, bv[tb], acc[tb][j], 0, 0, 0);
             }
         }
+        if constexpr (TB == 1) xv[0] = *reinterpret_cast<const u32x4*>(xp[0] + kn * 16);
     }
-    // register e of block nb: output 32 nb + 8 (e/4) + 4 hl + e%4, token l32
-    const int gt = tok0 + l32;
-    if (gt < a.t) {
-        float* out = a.xw_part + ((int64_t)split * a.t + gt) * nw;
+    // register e of block nb: output 32 nb + 8 (e/4) + 4 hl + e%4, token 32 tb + l32
 #pragma unroll
-        for (int j = 0; j < 2; ++j) {
-            const int nb = wave + 4 * j;
-            if (nb < nblocks)
+    for (int tb = 0; tb < TB; ++tb) {
+        const int gt = tok0 + 32 * tb + l32;
+        if (gt < a.t) {
+            float* out = a.xw_part + ((int64_t)split * a.t + gt) * nw;
 #pragma unroll
-                for (int e4 = 0; e4 < 4; ++e4)
-                    *reinterpret_cast<f32x4*>(out + 32 * nb + 8 * e4 + 4 * hl) =
-                        f32x4{acc[j][4 * e4], acc[j][4 * e4 + 1], acc[j][4 * e4 + 2], acc[j][4 * e4 + 3]};
+            for (int j = 0; j < 2; ++j) {
+                const int nb = wave + 4 * j;
+                if (nb < nblocks)
+#pragma unroll
+                    for (int e4 = 0; e4 < 4; ++e4)
+                        *reinterpret_cast<f32x4*>(out + 32 * nb + 8 * e4 + 4 * hl) =
+                            f32x4{acc[tb][j][4 * e4], acc[tb][j][4 * e4 + 1], acc[tb][j][4 * e4 + 2], acc[tb][j][4 * e4 + 3]};
+            }
         }
     }
 }
@@ -109,8 +132,16 @@ __global__ __launch_bounds__(1024) void prolog_qx_kernel(PrologArgs a)
         prolog_q_body(a, blockIdx.x, blockIdx.y * PTOK, plds);
     } else {
         if (threadIdx.x >= 256) return; // the barrier inside is among the remaining four waves
-        prolog_xw_body(a, blockIdx.x - a.n, blockIdx.y * PTOK, plds);
+        prolog_xw_body<1>(a, blockIdx.x - a.n, blockIdx.y * PTOK, plds);
     }
+}
+
+// x @ [w_k | w_proj] on its own, for the launches whose query product runs in prolog_q_big_kernel.
+// grid (h / 256, token tiles of 128), 256 lanes
+__global__ __launch_bounds__(256) void prolog_xw_kernel(PrologArgs a)
+{
+    extern __shared__ __align__(16) uint8_t plds[];
+    prolog_xw_body<4>(a, blockIdx.x, blockIdx.y * (4 * PTOK), plds);
 }
 
 } // namespace
@@ -146,8 +177,22 @@ hipError_t prolog_launch(const PrologArgs& a, hipStream_t stream)
                                    prolog_q_lds_bytes(QMAX_R) > xw_lds_max ? prolog_q_lds_bytes(QMAX_R) : xw_lds_max);
     });
     if (e != hipSuccess) return e;
-    {
-        const int xw_lds = XW_K * (PD + a.n) * 2;
+    const int xw_lds = XW_K * (PD + a.n) * 2;
+    if (a.t >= PROLOG_BIG_T) {
+        static DeviceOnce xw_attr_done;
+        e = xw_attr_done.run([] {
+            return hipFuncSetAttribute(reinterpret_cast<const void*>(prolog_xw_kernel), hipFuncAttributeMaxDynamicSharedMemorySize, xw_lds_max);
+        });
+        if (e != hipSuccess) return e;
+        ScopedKernelTimer tm(KID_PROLOG_Q, stream);
+        const dim3 qgrid(a.n, (a.t + QB_TOK - 1) / QB_TOK);
+        if (a.t <= PROLOG_DEEP_T)
+            hipLaunchKernelGGL(prolog_q_big_kernel<3>, qgrid, dim3(256), 0, stream, a);
+        else
+            hipLaunchKernelGGL(prolog_q_big_kernel<1>, qgrid, dim3(256), 0, stream, a);
+        if ((e = hipGetLastError()) != hipSuccess) return e;
+        hipLaunchKernelGGL(prolog_xw_kernel, dim3(a.ksplits, qgrid.y), dim3(256), xw_lds, stream, a);
+    } else {
         const int smem = prolog_q_lds_bytes(a.r) > xw_lds ? prolog_q_lds_bytes(a.r) : xw_lds;
         ScopedKernelTimer tm(KID_PROLOG_Q, stream);
         hipLaunchKernelGGL(prolog_qx_kernel, dim3(a.n + a.ksplits, ttiles), dim3(1024), smem, stream, a);

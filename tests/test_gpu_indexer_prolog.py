@@ -76,6 +76,23 @@ def test_decode_batch_and_ragged_token_tiles(cuda):
         check(case, run(case, cuda))
 
 
+def test_prefill_sizes_same_bits_as_the_decode_kernels(cuda):
+    """From 128 tokens on the query product runs per (head, 128 tokens) instead of per (head, 32 tokens).  Its integer
+    sums are exact and the rest is the same arithmetic, so the query outputs must be the bits the decode-size kernels
+    give for the same tokens (run here in slices of fewer than 128 tokens) - on token counts that leave ragged tiles."""
+    for b, s1, seed in ((64, 2, 20), (75, 4, 21), (257, 1, 22), (199, 1, 23)):
+        case = op.make_case(b, s1, 1024, seed=seed)
+        got = run(case, cuda)
+        check(case, got)
+        t = b * s1
+        per_token = ("x", "q_norm", "q_norm_scale", "cos", "sin", "k_cache_index")
+        for t0 in range(0, t, 100):
+            part = {k: (v[t0:t0 + 100] if k in per_token else v) for k, v in case.items()}
+            small = run(part, cuda)
+            assert torch.equal(small["q_int8"], got["q_int8"][t0:t0 + 100]), (t, t0)
+            assert torch.equal(small["q_scale"], got["q_scale"][t0:t0 + 100]), (t, t0)
+
+
 def test_walsh_hadamard_and_other_sizes(cuda):
     case = op.make_case(3, 2, 512, seed=12, hadamard="walsh")
     check(case, run(case, cuda))
