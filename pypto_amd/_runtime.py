@@ -93,7 +93,7 @@ _OPS = {
 
 # C status -> Python exception type wrapped by FeError
 _STATUS_EXC = {-1: RuntimeError, -2: ValueError, -3: ValueError, -4: ValueError, -5: RuntimeError, -6: RuntimeError,
-               -7: RuntimeError}
+               -7: RuntimeError, -8: ValueError}
 
 
 def library_path():

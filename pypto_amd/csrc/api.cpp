@@ -6,6 +6,7 @@
 #include "pypto_amd.h"
 
 #include <cstdarg>
+#include <cstdint>
 #include <cstdio>
 #include <string>
 
@@ -40,7 +41,9 @@ const char* dtype_name(int dt)
     }
 }
 
-int check_tensor(const char* op, const PtoTensorDesc& t, const char* name, int dtype, int rank, bool allow_empty = false)
+// `align`: the alignment the kernels' vector accesses assume of the tensor's address (16 bytes: what any torch allocation
+// and any view of whole rows has).  A misaligned address is refused here rather than left to the memory system.
+int check_tensor(const char* op, const PtoTensorDesc& t, const char* name, int dtype, int rank, int align = 16)
 {
     if (t.dataType != dtype)
         return fail(PTO_ERR_DTYPE, "%s: %s must be %s, got %s", op, name, dtype_name(dtype), dtype_name(t.dataType));
@@ -51,7 +54,8 @@ int check_tensor(const char* op, const PtoTensorDesc& t, const char* name, int d
         numel *= t.shape[i];
     }
     if (numel > 0 && t.addr == nullptr) return fail(PTO_ERR_NULL, "%s: %s has a null address", op, name);
-    (void)allow_empty;
+    if (numel > 0 && reinterpret_cast<uintptr_t>(t.addr) % (uintptr_t)align != 0)
+        return fail(PTO_ERR_ALIGN, "%s: the address of %s must be a multiple of %d bytes", op, name, align);
     return PTO_OK;
 }
 
@@ -358,12 +362,13 @@ int plan_paged_gather(const PtoTensorDesc* ts, uint32_t n, const PtoPagedGatherP
             return fail(PTO_ERR_DTYPE, "%s: %s must be int32 or int64, got %s", op, i == 1 ? "indices" : "block_table",
                         dtype_name(ts[i].dataType));
     int rc;
-    if ((rc = check_tensor(op, ts[0], "src", ts[0].dataType, 2))) return rc;
-    if ((rc = check_tensor(op, ts[1], "indices", ts[1].dataType, 2))) return rc;
-    if ((rc = check_tensor(op, ts[2], "block_table", ts[2].dataType, 2))) return rc;
-    if ((rc = check_tensor(op, ts[3], "out", ts[0].dataType, 2))) return rc; // out and src share a dtype
+    // (this operator moves rows in pieces as wide as the addresses allow: element alignment is all it asks for)
+    if ((rc = check_tensor(op, ts[0], "src", ts[0].dataType, 2, (int)esize))) return rc;
+    if ((rc = check_tensor(op, ts[1], "indices", ts[1].dataType, 2, ts[1].dataType == PTO_DT_INT64 ? 8 : 4))) return rc;
+    if ((rc = check_tensor(op, ts[2], "block_table", ts[2].dataType, 2, ts[2].dataType == PTO_DT_INT64 ? 8 : 4))) return rc;
+    if ((rc = check_tensor(op, ts[3], "out", ts[0].dataType, 2, (int)esize))) return rc; // out and src share a dtype
     if (n == 5) {
-        if ((rc = check_tensor(op, ts[4], "status", PTO_DT_INT32, 1))) return rc;
+        if ((rc = check_tensor(op, ts[4], "status", PTO_DT_INT32, 1, 4))) return rc;
         if (ts[4].shape[0] != 1) return fail(PTO_ERR_SHAPE, "%s: status must hold one word", op);
     }
     const int64_t hidden = ts[0].shape[1], b = ts[1].shape[0], k = ts[1].shape[1];

@@ -91,6 +91,26 @@ def launch_rc(lib, op, specs, params, ws=None, ws_bytes=0):
     return rc, lib.pto_last_error().decode()
 
 
+def test_misaligned_addresses_are_refused(lib):
+    """The kernels read and write 16 bytes per lane: an address that is not a multiple of 16 is refused with its own
+    code (-8) before anything is launched; the paged gather asks only for element alignment."""
+    from pypto_amd._runtime import PagedGatherParams
+    p = SfaParams(128, 1, 0.1, 2048, 128, 8, 4)
+    d = descs(sfa_specs())
+    d[0].addr = FAKE + 8
+    fn = lib.pto_sfa_quant_launch
+    assert fn(d, 9, ctypes.byref(p), None, 0, None, 0) == -8
+    assert "query_nope" in lib.pto_last_error().decode() and "16 bytes" in lib.pto_last_error().decode()
+    assert lib.pto_sfa_quant_workspace(d, 9, ctypes.byref(p)) == 0
+    # (the page table has one row too many, so that the call is refused after the address checks and launches nothing)
+    g = descs([(BF16, (64, 24)), (INT32, (2, 8)), (INT32, (3, 4)), (BF16, (16, 24))])
+    gp = PagedGatherParams(16, 0)
+    g[0].addr, g[3].addr = FAKE + 2, FAKE + 6     # views that start inside a row: fine for the gather
+    assert lib.pto_paged_gather_launch(g, 4, ctypes.byref(gp), None, 0, None, 0) == -3, lib.pto_last_error().decode()
+    g[0].addr = FAKE + 1                          # not even an element boundary
+    assert lib.pto_paged_gather_launch(g, 4, ctypes.byref(gp), None, 0, None, 0) == -8
+
+
 def test_sfa_validation_codes(lib):
     p = SfaParams(128, 1, 0.1, 2048, 128, 8, 4)
     rc, msg = launch_rc(lib, "sfa_quant", sfa_specs()[:8], p)
