@@ -634,13 +634,13 @@ static_assert(QG_TOK * QG_OROW <= QG_STAGE_BYTES, "the output tile takes the ope
 // workgroups to a CU - what the 768 workgroups of 512 tokens want; at 256 tokens and fewer the grid leaves at most two
 // workgroups to a CU anyway, and the twelve stages of a tile are otherwise twelve memory latencies in a row.
 template <int DEPTH>
-__global__ __launch_bounds__(256, DEPTH == 1 ? 3 : 2) void mla_qb_big_kernel(MlaPrologArgs a)
+__device__ __forceinline__ void mla_qb_big_body(const MlaPrologArgs& a, int col0, int tok0, uint8_t* stage_lds)
 {
 #pragma clang fp contract(off)
-    __shared__ __align__(16) uint8_t stage_lds[QG_STAGE_BYTES]; // [128 k][MQROW] weights | [128 tokens][QG_QROW] q_norm
+    // stage_lds: QG_STAGE_BYTES, [128 k][MQROW] weights | [128 tokens][QG_QROW] q_norm
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int l16 = lane & 15, g = lane >> 4, wr = wave >> 1, wc = wave & 1;
-    const int r = a.r, col0 = blockIdx.x * 128, tok0 = blockIdx.y * QG_TOK;
+    const int r = a.r;
     const int64_t nq = (int64_t)a.n * MQH;
     uint8_t* wl = stage_lds;
     uint8_t* ql = stage_lds + QG_K * MQROW;
@@ -756,6 +756,13 @@ __global__ __launch_bounds__(256, DEPTH == 1 ? 3 : 2) void mla_qb_big_kernel(Mla
     }
 }
 
+template <int DEPTH>
+__global__ __launch_bounds__(256, DEPTH == 1 ? 3 : 2) void mla_qb_big_kernel(MlaPrologArgs a)
+{
+    __shared__ __align__(16) uint8_t stage_lds[QG_STAGE_BYTES];
+    mla_qb_big_body<DEPTH>(a, blockIdx.x * 128, blockIdx.y * QG_TOK, stage_lds);
+}
+
 // ------------------------------------------------------------------------------------------------ fused with the indexer prolog
 // The fused operator runs the two prologs' per-token kernels side by side in one launch, and likewise the two int8
 // GEMMs on q_norm (192 + 64 workgroups at model sizes: one per compute unit); the indexer's x @ [w_k | w_proj] rides along
@@ -780,6 +787,29 @@ __global__ __launch_bounds__(1024) void fused_qb_kernel(MlaPrologArgs m, PrologA
         mla_qb_body(m, blockIdx.x * 128, blockIdx.y * MTOK, fq_lds);
     else
         prolog_q_body(p, blockIdx.x - nqb, blockIdx.y * PTOK, fq_lds);
+}
+
+// The same pair at prefill sizes: both products per 128 tokens, side by side.  The indexer's epilogue sets the LDS (68 KB:
+// two workgroups to a CU), so both run with three stages of loads in flight.
+// grid (n * 192 / 128 + index heads, token tiles of 128), 256 lanes
+__global__ __launch_bounds__(256, 2) void fused_qb_big_kernel(MlaPrologArgs m, PrologArgs p)
+{
+    static_assert(QB_LDS_BYTES >= QG_STAGE_BYTES && QB_TOK == QG_TOK, "one LDS block and one token tiling serve both bodies");
+    __shared__ __align__(16) uint8_t lds[QB_LDS_BYTES];
+    const int nqb = m.n * MQH / 128;
+    if ((int)blockIdx.x < nqb)
+        mla_qb_big_body<QB_DEPTH>(m, blockIdx.x * 128, blockIdx.y * QG_TOK, lds);
+    else
+        prolog_q_big_body<QB_DEPTH>(p, blockIdx.x - nqb, blockIdx.y * QB_TOK, lds);
+}
+
+// Above 256 tokens the two products are launches of their own again: the MLA product then fills the chip at three
+// workgroups to a CU (one stage of loads in flight, 36 KB of LDS), which the shared launch's 68 KB would not allow.
+// grid (index heads, token tiles of 128), 256 lanes
+__global__ __launch_bounds__(256, 2) void fused_q_big_kernel(PrologArgs p)
+{
+    __shared__ __align__(16) uint8_t lds[QB_LDS_BYTES];
+    prolog_q_big_body<QB_DEPTH>(p, blockIdx.x, blockIdx.y * QB_TOK, lds);
 }
 
 // ------------------------------------------------------------------------------------------------ q_b[:, head, :128] @ w_uk[head]
@@ -972,16 +1002,14 @@ static hipError_t launch_prologs(const MlaPrologArgs& a, const PrologArgs* p, hi
             hipLaunchKernelGGL(mla_qb16_epilogue_kernel, dim3(a.t, (nq / 4 + 255) / 256), dim3(256), 0, stream, a);
         } else if (big) {
             const dim3 qgrid(a.n * MQH / 128, (a.t + QG_TOK - 1) / QG_TOK);
-            if (a.t <= BIG_T2)
-                hipLaunchKernelGGL(mla_qb_big_kernel<3>, qgrid, dim3(256), 0, stream, a);
-            else
-                hipLaunchKernelGGL(mla_qb_big_kernel<1>, qgrid, dim3(256), 0, stream, a);
-            if (p) {
-                const dim3 pgrid(p->n, (a.t + QB_TOK - 1) / QB_TOK);
-                if (a.t <= PROLOG_DEEP_T)
-                    hipLaunchKernelGGL(prolog_q_big_kernel<3>, pgrid, dim3(256), 0, stream, *p);
+            if (p && a.t <= BIG_T2) {
+                hipLaunchKernelGGL(fused_qb_big_kernel, dim3(qgrid.x + p->n, qgrid.y), dim3(256), 0, stream, a, *p);
+            } else {
+                if (a.t <= BIG_T2)
+                    hipLaunchKernelGGL(mla_qb_big_kernel<3>, qgrid, dim3(256), 0, stream, a);
                 else
-                    hipLaunchKernelGGL(prolog_q_big_kernel<1>, pgrid, dim3(256), 0, stream, *p);
+                    hipLaunchKernelGGL(mla_qb_big_kernel<1>, qgrid, dim3(256), 0, stream, a);
+                if (p) hipLaunchKernelGGL(fused_q_big_kernel, dim3(p->n, qgrid.y), dim3(256), 0, stream, *p);
             }
         } else if (p) {
             const int smem = mla_qb_lds_bytes(a.r) > prolog_q_lds_bytes(a.r) ? mla_qb_lds_bytes(a.r) : prolog_q_lds_bytes(a.r);

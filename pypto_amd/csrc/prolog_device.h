@@ -11,7 +11,7 @@ namespace {
 constexpr int PD = 128;      // index head dim
 constexpr int PROPE = 64;    // rotary dims
 constexpr int PTOK = 32;     // tokens per workgroup tile
-constexpr int XW_K = 256;    // contraction rows per workgroup of prolog_xw_kernel
+constexpr int XW_K = 256;    // contraction rows per workgroup of the x @ [w_k | w_proj] product
 constexpr int XROW = PD * 2 + 16; // bytes per LDS row of the 32 x 128 bf16 tile (padded)
 constexpr int QK = 128;      // contraction rows per stage of prolog_q_kernel
 constexpr int QROW = 136;    // bytes per LDS row of a [k][128] int8 weight stage (padded, 8-byte aligned)
@@ -259,15 +259,16 @@ constexpr int QB_QROW = QK + 16; // bytes per LDS row of the [token][k] int8 til
 constexpr int QB_STAGE_BYTES = QK * QROW + QB_TOK * QB_QROW;
 constexpr int QB_EPI_BYTES = PD * PD * 2 + QB_TOK * XROW + 4 * QB_TOK * 4; // hadamard_q | bf16 tile | per-wave maxima
 constexpr int QB_LDS_BYTES = QB_EPI_BYTES > QB_STAGE_BYTES ? QB_EPI_BYTES : QB_STAGE_BYTES;
+constexpr int QB_DEPTH = 3; // stages of loads in flight (the epilogue's 68 KB of LDS leave two workgroups to a CU whatever the
+                            // register count, so the depth costs no occupancy)
 
 template <int DEPTH>
-__global__ __launch_bounds__(256, 2) void prolog_q_big_kernel(PrologArgs a)
+__device__ __forceinline__ void prolog_q_big_body(const PrologArgs& a, int head, int tok0, uint8_t* lds)
 {
 #pragma clang fp contract(off)
-    __shared__ __align__(16) uint8_t lds[QB_LDS_BYTES];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int l16 = lane & 15, g = lane >> 4, l32 = lane & 31, hl = lane >> 5, wr = wave >> 1, wc = wave & 1;
-    const int r = a.r, head = blockIdx.x, tok0 = blockIdx.y * QB_TOK;
+    const int r = a.r;
     const int64_t nd = (int64_t)a.n * PD;
     uint8_t* wl = lds;
     uint8_t* ql = lds + QK * QROW;
@@ -433,9 +434,7 @@ __global__ __launch_bounds__(256, 2) void prolog_q_big_kernel(PrologArgs a)
         }
     }
 }
-constexpr int PROLOG_BIG_T = 256;   // token count from which the query product runs per 128 tokens (below, its 64 x t / 128
-                                    // workgroups leave most of the chip idle and the kernel per 32 tokens is faster)
-constexpr int PROLOG_DEEP_T = 1024; // up to here at most two of its workgroups share a CU: three stages of loads in flight each
+constexpr int PROLOG_BIG_T = 128;   // token count from which the query product runs per 128 tokens
 
 // ------------------------------------------------------------------------------------------------ key path, weights
 __device__ __forceinline__ float block_sum128(float v, float* red)

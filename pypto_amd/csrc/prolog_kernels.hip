@@ -41,27 +41,16 @@ __global__ __launch_bounds__(128) void prolog_k_kernel(PrologArgs a) { prolog_k_
 // 256 lanes per (256 rows of the weights, token tile of 32 TB): partial sums over those rows; wl is [256 k][nw] bf16,
 // nw = 128 + n.  TB blocks of 32 tokens per workgroup: 1 at decode sizes; 4 at prefill sizes, where the weight rows are
 // then staged once per 128 tokens and every weight fragment read from LDS feeds four MFMAs.
-template <int TB>
+template <int TB, int PARTS = 1>
 __device__ __forceinline__ void prolog_xw_body(const PrologArgs& a, int split, int tok0, uint8_t* wl)
 {
+    // PARTS: the workgroup's 256 weight rows are staged in that many pieces, one after the other in the same LDS space
+    // (two at prefill sizes: 49 KB instead of 98, so that two workgroups share a CU next to the query product's)
+    constexpr int ROWS = XW_K / PARTS;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int l32 = lane & 31, hl = lane >> 5;
     const int nw = PD + a.n, rowb = nw * 2;
     const int64_t kbase = (int64_t)split * XW_K;
-    // stage the weights: w_k rows then w_proj rows, 16-byte pieces
-#pragma unroll 8
-    for (int i = tid; i < XW_K * (PD / 8); i += 256) {
-        const int k = i / (PD / 8), c = i % (PD / 8);
-        *reinterpret_cast<u32x4*>(wl + k * rowb + c * 16) =
-            *reinterpret_cast<const u32x4*>(a.w_k + (kbase + k) * PD + c * 8);
-    }
-#pragma unroll 8
-    for (int i = tid; i < XW_K * (a.n / 8); i += 256) {
-        const int k = i / (a.n / 8), c = i % (a.n / 8);
-        *reinterpret_cast<u32x4*>(wl + k * rowb + PD * 2 + c * 16) =
-            *reinterpret_cast<const u32x4*>(a.w_proj + (kbase + k) * a.n + c * 8);
-    }
-    __syncthreads();
     const int nblocks = nw / 32; // 32-wide output blocks; wave w takes blocks w, w + 4
     const int jj = lane & 15, mh = (lane >> 4) & 1;
     // B operand: the transposing reads below hand lane half hl the contraction rows 8 hl .. 8 hl + 7 of every 16-row step,
@@ -79,30 +68,47 @@ __device__ __forceinline__ void prolog_xw_body(const PrologArgs& a, int split, i
     u32x4 xv[TB];
 #pragma unroll
     for (int tb = 0; tb < TB; ++tb) xv[tb] = *reinterpret_cast<const u32x4*>(xp[tb]);
-    for (int ks = 0; ks < XW_K / 16; ++ks) {
-        bf16x8 bv[TB];
 #pragma unroll
-        for (int tb = 0; tb < TB; ++tb) bv[tb] = __builtin_bit_cast(bf16x8, xv[tb]);
-        // (TB = 1 runs beside the query product in a 1024-lane launch, at 128 registers: no room for the step ahead,
-        // the load sits at the end of the step instead)
-        const int kn = min(ks + 1, XW_K / 16 - 1); // (past the end: the last step again, dropped)
-        if constexpr (TB > 1) {
-#pragma unroll
-            for (int tb = 0; tb < TB; ++tb) xv[tb] = *reinterpret_cast<const u32x4*>(xp[tb] + kn * 16);
+    for (int part = 0; part < PARTS; ++part) {
+        if (part > 0) __syncthreads(); // everyone is done with the previous piece
+        // stage the weights: w_k rows then w_proj rows, 16-byte pieces
+        const int64_t k0 = kbase + part * ROWS;
+#pragma unroll 8
+        for (int i = tid; i < ROWS * (PD / 8); i += 256) {
+            const int k = i / (PD / 8), c = i % (PD / 8);
+            *reinterpret_cast<u32x4*>(wl + k * rowb + c * 16) = *reinterpret_cast<const u32x4*>(a.w_k + (k0 + k) * PD + c * 8);
         }
+#pragma unroll 8
+        for (int i = tid; i < ROWS * (a.n / 8); i += 256) {
+            const int k = i / (a.n / 8), c = i % (a.n / 8);
+            *reinterpret_cast<u32x4*>(wl + k * rowb + PD * 2 + c * 16) = *reinterpret_cast<const u32x4*>(a.w_proj + (k0 + k) * a.n + c * 8);
+        }
+        __syncthreads();
+        for (int ks = part * (ROWS / 16); ks < (part + 1) * (ROWS / 16); ++ks) {
+            bf16x8 bv[TB];
 #pragma unroll
-        for (int j = 0; j < 2; ++j) {
-            const int nb = wave + 4 * j;
-            if (nb < nblocks) {
-                const uint8_t* hp = wl + (ks * 16 + 8 * hl + (jj >> 2)) * rowb + (32 * nb + 16 * mh + 4 * (jj & 3)) * 2;
-                const s16x4 lo = lds_read_tr(hp);
-                const s16x4 hi = lds_read_tr(hp + 4 * rowb);
-                const bf16x8 av = __builtin_bit_cast(bf16x8, __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
+            for (int tb = 0; tb < TB; ++tb) bv[tb] = __builtin_bit_cast(bf16x8, xv[tb]);
+            // (TB = 1 runs beside the query product in a 1024-lane launch, at 128 registers: no room for the step ahead,
+            // the load sits at the end of the step instead)
+            const int kn = min(ks + 1, XW_K / 16 - 1); // (past the end: the last step again, dropped)
+            if constexpr (TB > 1) {
 #pragma unroll
-                for (int tb = 0; tb < TB; ++tb) acc[tb][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(av, bv[tb], acc[tb][j], 0, 0, 0);
+                for (int tb = 0; tb < TB; ++tb) xv[tb] = *reinterpret_cast<const u32x4*>(xp[tb] + kn * 16);
             }
+#pragma unroll
+            for (int j = 0; j < 2; ++j) {
+                const int nb = wave + 4 * j;
+                if (nb < nblocks) {
+                    const uint8_t* hp = wl + ((ks - part * (ROWS / 16)) * 16 + 8 * hl + (jj >> 2)) * rowb + (32 * nb + 16 * mh + 4 * (jj & 3)) * 2;
+                    const s16x4 lo = lds_read_tr(hp);
+                    const s16x4 hi = lds_read_tr(hp + 4 * rowb);
+                    const bf16x8 av = __builtin_bit_cast(bf16x8, __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
+#pragma unroll
+                    for (int tb = 0; tb < TB; ++tb) acc[tb][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(av, bv[tb], acc[tb][j], 0, 0, 0);
+                }
+            }
+            if constexpr (TB == 1) xv[0] = *reinterpret_cast<const u32x4*>(xp[0] + kn * 16);
         }
-        if constexpr (TB == 1) xv[0] = *reinterpret_cast<const u32x4*>(xp[0] + kn * 16);
     }
     // register e of block nb: output 32 nb + 8 (e/4) + 4 hl + e%4, token 32 tb + l32
 #pragma unroll
@@ -136,12 +142,17 @@ __global__ __launch_bounds__(1024) void prolog_qx_kernel(PrologArgs a)
     }
 }
 
-// x @ [w_k | w_proj] on its own, for the launches whose query product runs in prolog_q_big_kernel.
-// grid (h / 256, token tiles of 128), 256 lanes
-__global__ __launch_bounds__(256) void prolog_xw_kernel(PrologArgs a)
+// Prefill sizes: the query product per (head, 128 tokens) and x @ [w_k | w_proj] per (256 weight rows, 128 tokens) side
+// by side in one launch, as at decode sizes.  grid (heads + h / 256, token tiles of 128), 256 lanes; the dynamic LDS is
+// the larger of the two bodies' needs.
+template <int DEPTH>
+__global__ __launch_bounds__(256, 2) void prolog_qx_big_kernel(PrologArgs a)
 {
     extern __shared__ __align__(16) uint8_t plds[];
-    prolog_xw_body<4>(a, blockIdx.x, blockIdx.y * (4 * PTOK), plds);
+    if ((int)blockIdx.x < a.n)
+        prolog_q_big_body<DEPTH>(a, blockIdx.x, blockIdx.y * QB_TOK, plds);
+    else
+        prolog_xw_body<4, 2>(a, blockIdx.x - a.n, blockIdx.y * (4 * PTOK), plds);
 }
 
 } // namespace
@@ -179,19 +190,16 @@ hipError_t prolog_launch(const PrologArgs& a, hipStream_t stream)
     if (e != hipSuccess) return e;
     const int xw_lds = XW_K * (PD + a.n) * 2;
     if (a.t >= PROLOG_BIG_T) {
-        static DeviceOnce xw_attr_done;
-        e = xw_attr_done.run([] {
-            return hipFuncSetAttribute(reinterpret_cast<const void*>(prolog_xw_kernel), hipFuncAttributeMaxDynamicSharedMemorySize, xw_lds_max);
+        static DeviceOnce big_attr_done;
+        constexpr int big_lds_max = xw_lds_max / 2 > QB_LDS_BYTES ? xw_lds_max / 2 : QB_LDS_BYTES;
+        e = big_attr_done.run([] {
+            return hipFuncSetAttribute(reinterpret_cast<const void*>(prolog_qx_big_kernel<QB_DEPTH>), hipFuncAttributeMaxDynamicSharedMemorySize, big_lds_max);
         });
         if (e != hipSuccess) return e;
         ScopedKernelTimer tm(KID_PROLOG_Q, stream);
-        const dim3 qgrid(a.n, (a.t + QB_TOK - 1) / QB_TOK);
-        if (a.t <= PROLOG_DEEP_T)
-            hipLaunchKernelGGL(prolog_q_big_kernel<3>, qgrid, dim3(256), 0, stream, a);
-        else
-            hipLaunchKernelGGL(prolog_q_big_kernel<1>, qgrid, dim3(256), 0, stream, a);
-        if ((e = hipGetLastError()) != hipSuccess) return e;
-        hipLaunchKernelGGL(prolog_xw_kernel, dim3(a.ksplits, qgrid.y), dim3(256), xw_lds, stream, a);
+        const dim3 grid(a.n + a.ksplits, (a.t + QB_TOK - 1) / QB_TOK);
+        const int smem = xw_lds / 2 > QB_LDS_BYTES ? xw_lds / 2 : QB_LDS_BYTES; // (the x product stages its rows in two halves here)
+        hipLaunchKernelGGL(prolog_qx_big_kernel<QB_DEPTH>, grid, dim3(256), smem, stream, a);
     } else {
         const int smem = prolog_q_lds_bytes(a.r) > xw_lds ? prolog_q_lds_bytes(a.r) : xw_lds;
         ScopedKernelTimer tm(KID_PROLOG_Q, stream);

@@ -77,7 +77,8 @@ def test_decode_batch_and_ragged_token_tiles(cuda):
 
 
 def test_prefill_sizes_same_bits_as_the_decode_kernels(cuda):
-    """From 128 tokens on the query product runs per (head, 128 tokens) instead of per (head, 32 tokens).  Its integer
+    """From 128 tokens on the query product runs per (head, 128 tokens) instead of per (head, 32 tokens), beside the x
+    product per 128 tokens.  Its integer
     sums are exact and the rest is the same arithmetic, so the query outputs must be the bits the decode-size kernels
     give for the same tokens (run here in slices of fewer than 128 tokens) - on token counts that leave ragged tiles."""
     for b, s1, seed in ((64, 2, 20), (75, 4, 21), (257, 1, 22), (199, 1, 23)):
