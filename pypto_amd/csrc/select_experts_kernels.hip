@@ -25,23 +25,56 @@ __device__ __forceinline__ float load_as_f32(const uint16_t* p, int64_t i) { ret
 // true when (v2, e2) comes before (v, e)
 __device__ __forceinline__ int before(float v2, int e2, float v, int e) { return (v2 > v) || (v2 == v && e2 < e); }
 
+// Wavefront-wide maximum of a u32, the same value in every lane, in the vector unit's own lane network (DPP row_shr
+// steps inside the rows of 16 lanes, row_bcast15 / row_bcast31 across them).
+template <int CTRL, int ROW_MASK>
+__device__ __forceinline__ uint32_t se_dpp_from(uint32_t v)
+{
+    return (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, CTRL, ROW_MASK, 0xf, false);
+}
+__device__ __forceinline__ uint32_t se_wave_max(uint32_t v)
+{
+    v = max(v, se_dpp_from<0x111, 0xf>(v));
+    v = max(v, se_dpp_from<0x112, 0xf>(v));
+    v = max(v, se_dpp_from<0x114, 0xf>(v));
+    v = max(v, se_dpp_from<0x118, 0xf>(v));
+    v = max(v, se_dpp_from<0x142, 0xa>(v));
+    v = max(v, se_dpp_from<0x143, 0xc>(v));
+    return (uint32_t)__builtin_amdgcn_readlane((int)v, 63);
+}
+__device__ __forceinline__ float ordered_to_f32(uint32_t k)
+{
+    return __builtin_bit_cast(float, (k & 0x80000000u) ? (k & 0x7fffffffu) : ~k);
+}
+
+// One wavefront per token, everything but the group maxima in registers: lane l holds experts l, l + 64, l + 128,
+// l + 192.  Group maxima by LDS atomic maxima on order-preserving keys; group ranks by counting against the other groups'
+// maxima read lane by lane (v_readlane); experts by top_k rounds of a wave-wide arg-max in two steps - the largest
+// ordered score, then the smallest expert id among the lanes that hold it - both in the lane network (DPP), no trip
+// through LDS.  The selected experts' sigmoid values are picked out of their owners' registers with v_readlane.
 template <typename LT, typename BT>
 __global__ __launch_bounds__(64) void select_experts_kernel(SelectExpertsArgs a)
 {
-    __shared__ __align__(16) float s_sig[SE_MAX_NE];
-    __shared__ __align__(16) float s_x[SE_MAX_NE];
-    __shared__ float s_g[SE_MAX_GROUPS];
-    __shared__ int s_keep[SE_MAX_GROUPS];
-    __shared__ float s_w[SE_MAX_K];
+    __shared__ uint32_t s_gkey[SE_MAX_GROUPS];
 
     const int lane = threadIdx.x;
     const int ne = a.ne, ng = a.n_group, gs = ne / ng;
     const LT* logits = static_cast<const LT*>(a.logits);
     const BT* bias = static_cast<const BT*>(a.bias);
     const float fill = a.fill_neg_inf ? -__builtin_inff() : 0.0f;
+    // what does not depend on the token: this lane's experts' groups and bias
+    int grp[4];
+    float bs[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        const int e = lane + 64 * j;
+        grp[j] = e < ne ? e / gs : 0;
+        bs[j] = e < ne ? load_as_f32(bias, e) : 0.f;
+    }
 
     for (int64_t tok = blockIdx.x; tok < a.t; tok += gridDim.x) {
         float own_x[4], own_s[4];
+        if (lane < ng) s_gkey[lane] = 0u;
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
             const int e = lane + 64 * j;
@@ -52,70 +85,59 @@ __global__ __launch_bounds__(64) void select_experts_kernel(SelectExpertsArgs a)
                 // sigmoid in double, rounded once: the correctly rounded fp32 value whatever the libm
                 const float sg = (float)(1.0 / (1.0 + exp(-(double)x)));
                 own_s[j] = sg;
-                own_x[j] = sg + load_as_f32(bias, e);
-                s_sig[e] = sg;
-                s_x[e] = own_x[j];
+                own_x[j] = sg + bs[j];
             }
         }
         __syncthreads();
-        if (lane < ng) {
-            float m = s_x[lane * gs];
-            for (int i = 1; i < gs; ++i) m = fmaxf(m, s_x[lane * gs + i]);
-            s_g[lane] = m;
-        }
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+            if (lane + 64 * j < ne) atomicMax(&s_gkey[grp[j]], f32_to_ordered(own_x[j]));
         __syncthreads();
-        if (lane < ng) {
-            const float m = s_g[lane];
-            int rank = 0;
-            for (int g2 = 0; g2 < ng; ++g2) rank += before(s_g[g2], g2, m, lane);
-            s_keep[lane] = rank < a.topk_group;
+        // lane g < ng: the maximum of group g, its rank among the groups (value descending, index ascending)
+        const float m = ordered_to_f32(s_gkey[lane < ng ? lane : 0]);
+        int rank = 0;
+        for (int g2 = 0; g2 < ng; ++g2) {
+            const float m2 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, m), g2));
+            rank += before(m2, g2, m, lane);
         }
-        __syncthreads();
+        const uint64_t keep = __ballot(lane < ng && rank < a.topk_group);
+        // ordered score and inverted id of this lane's experts (0 / 0 for the slots past the last expert and for the
+        // experts already taken): the largest (score, ~id) is the largest score and, among equal scores, the smallest id
+        uint32_t hi[4], lo[4];
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
             const int e = lane + 64 * j;
-            if (e < ne && !s_keep[e / gs]) {
-                own_x[j] = fill;
-                s_x[e] = fill;
-            }
+            if (!((keep >> grp[j]) & 1ull)) own_x[j] = fill;
+            hi[j] = e < ne ? f32_to_ordered(own_x[j] + 0.0f) : 0u;
+            lo[j] = e < ne ? (uint32_t)(~e) : 0u;
         }
-        __syncthreads();
-        // top_k rounds of a wave-wide arg-max over 64-bit keys (ordered score << 32 | ~expert): the largest key is the
-        // largest score and, among equal scores, the smallest expert id
-        unsigned long long key[4];
-#pragma unroll
-        for (int j = 0; j < 4; ++j) {
-            const int e = lane + 64 * j;
-            key[j] = e < ne ? ((unsigned long long)f32_to_ordered(own_x[j] + 0.0f) << 32) | (uint32_t)(~e) : 0ull;
-        }
+        int my_id = 0;
+        float my_w = 0.f, sum = 0.f;
         for (int r = 0; r < a.top_k; ++r) {
-            unsigned long long best = key[0] > key[1] ? key[0] : key[1];
-            const unsigned long long b2 = key[2] > key[3] ? key[2] : key[3];
-            best = best > b2 ? best : b2;
+            const uint32_t hmax = se_wave_max(max(max(hi[0], hi[1]), max(hi[2], hi[3])));
+            uint32_t cand = 0u;
 #pragma unroll
-            for (int sh = 1; sh < 64; sh <<= 1) {
-                const unsigned long long o = __shfl_xor(best, sh);
-                best = best > o ? best : o;
-            }
-            const int e = (int)~(uint32_t)best;
-            if (lane == 0) {
-                a.topk_ids[tok * a.top_k + r] = e;
-                s_w[r] = s_sig[e];
+            for (int j = 0; j < 4; ++j) cand = max(cand, hi[j] == hmax ? lo[j] : 0u);
+            const uint32_t lmax = se_wave_max(cand);
+            const int e = (int)~lmax;
+            // the expert's sigmoid value sits in register e / 64 of lane e % 64
+            const int ej = e >> 6;
+            const float src = ej == 0 ? own_s[0] : ej == 1 ? own_s[1] : ej == 2 ? own_s[2] : own_s[3];
+            const float w = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, src), e & 63));
+            sum += w;
+            if (lane == r) {
+                my_id = e;
+                my_w = w;
             }
 #pragma unroll
-            for (int j = 0; j < 4; ++j) key[j] = key[j] == best ? 0ull : key[j];
+            for (int j = 0; j < 4; ++j) hi[j] = (hi[j] == hmax && lo[j] == lmax) ? 0u : hi[j];
         }
-        __syncthreads();
         if (lane < a.top_k) {
-            float w = s_w[lane];
-            if (a.renormalize) {
-                float sum = 0.f;
-                for (int i = 0; i < a.top_k; ++i) sum += s_w[i];
-                w = w / sum;
-            }
+            a.topk_ids[tok * a.top_k + lane] = my_id;
+            const float w = a.renormalize ? my_w / sum : my_w;
             a.topk_weights[tok * a.top_k + lane] = w * a.routed_scaling_factor;
         }
-        __syncthreads();
+        __syncthreads(); // the group maxima are cleared for the next token only after every lane has read them
     }
 }
 
