@@ -58,7 +58,10 @@ def test_config2_grouped(cuda):
 
 def test_dtypes_sizes_and_flags(cuda):
     for seed, (t, ne, ng, tg, k, renorm) in enumerate([(5, 256, 64, 7, 32, False), (1, 1, 1, 1, 1, True),
-                                                        (300, 96, 3, 2, 6, True), (17, 64, 4, 4, 5, False)]):
+                                                        (300, 96, 3, 2, 6, True), (17, 64, 4, 4, 5, False),
+                                                        # (more than 160 experts with at most 16 groups and 16 selected: the widest
+                                                        # form of the four-tokens-per-wavefront kernel; 13 groups of 16)
+                                                        (33, 256, 16, 5, 16, True), (9, 208, 13, 6, 9, False)]):
         for ld, bd in ((torch.float32, torch.bfloat16), (torch.bfloat16, torch.bfloat16), (torch.float32, torch.float32)):
             logits, bias = ose.make_case(t, ne, 40 + seed, logits_dtype=ld, bias_dtype=bd)
             check(logits, bias, k, renorm, tg, ng, cuda, scale=1.5, neg=bool(seed % 2))
