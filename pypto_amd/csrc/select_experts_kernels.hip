@@ -2,9 +2,11 @@
 // weights.  Reference: models/glm_v4_5/glm_select_experts.py:60-228 (kernel) and :274-313 (golden);
 // python/tests/ut/interpreter/_ops/moe_gating_topk.py:223-287 (groups, -inf fill, scaling factor).
 //
-// The whole problem is a few MB (8192 x 160 logits), so the kernel is bound by launch and memory latency, not by a
-// roofline: one wavefront per token; groups are ranked by counting (rank of g = number of groups that come before g in
-// the order "value descending, index ascending"), experts by top_k rounds of a wave-wide arg-max on 64-bit keys.
+// The whole problem is a few MB (8192 x 160 logits): what bounds the kernels is vector instruction issue, more than half
+// of it the double-precision sigmoid.  Groups are ranked by counting (rank of g = number of groups that come before g
+// in the order "value descending, index ascending"), experts by top_k rounds of an arg-max on (ordered score, ~id).
+// select_experts_rows_kernel puts four tokens in a wavefront (the router's shapes); select_experts_kernel, one token per
+// wavefront, takes the shapes with more than 16 groups or 16 selected experts.
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
