@@ -56,6 +56,33 @@ __device__ __forceinline__ float wave_max_f32(float v)
     return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), 63));
 }
 
+// Wavefront-wide sum, the same value in every lane, with the additions of the xor butterfly (partners 1, 2, 4, 8, 16, 32
+// lanes away, in that order) but without its six dependent permutes through LDS.  After the first two steps (quad
+// permutes) a quad's lanes hold the same value, so mirroring a half row pairs every lane with a lane that holds what
+// its xor-4 partner holds; likewise the row mirror for xor 8; the two swaps exchange whole rows and half-waves.  a + b
+// is b + a, so every lane adds the same two numbers as in the butterfly: the result is the butterfly's, bit for bit.
+template <int CTRL>
+__device__ __forceinline__ float dpp_perm_f32(float v)
+{
+    return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xf, 0xf, false));
+}
+__device__ __forceinline__ float wave_sum_butterfly(float v)
+{
+    v += dpp_perm_f32<0xB1>(v);  // quad_perm [1, 0, 3, 2]
+    v += dpp_perm_f32<0x4E>(v);  // quad_perm [2, 3, 0, 1]
+    v += dpp_perm_f32<0x141>(v); // row_half_mirror
+    v += dpp_perm_f32<0x140>(v); // row_mirror
+    {
+        const auto sw = __builtin_amdgcn_permlane16_swap(__builtin_bit_cast(unsigned, v), __builtin_bit_cast(unsigned, v), false, false);
+        v = __builtin_bit_cast(float, (unsigned)sw[0]) + __builtin_bit_cast(float, (unsigned)sw[1]);
+    }
+    {
+        const auto sw = __builtin_amdgcn_permlane32_swap(__builtin_bit_cast(unsigned, v), __builtin_bit_cast(unsigned, v), false, false);
+        v = __builtin_bit_cast(float, (unsigned)sw[0]) + __builtin_bit_cast(float, (unsigned)sw[1]);
+    }
+    return v;
+}
+
 // Two fp32 -> one dword holding two bf16 (round to nearest even), low half = a.
 __device__ __forceinline__ uint32_t pack_bf16x2(float a, float b)
 {

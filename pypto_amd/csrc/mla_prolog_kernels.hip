@@ -309,12 +309,7 @@ __global__ __launch_bounds__(256) void mla_qb16_epilogue_kernel(MlaPrologArgs a)
 }
 
 // ------------------------------------------------------------------------------------------------ norms, quantisation, cache
-__device__ __forceinline__ float wave_sum(float v)
-{
-#pragma unroll
-    for (int d = 1; d < 64; d <<= 1) v += __shfl_xor(v, d);
-    return v;
-}
+__device__ __forceinline__ float wave_sum(float v) { return wave_sum_butterfly(v); }
 __device__ __forceinline__ float wave_max(float v) { return wave_max_f32(v); }
 
 // one workgroup of 256 lanes per token

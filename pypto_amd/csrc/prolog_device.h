@@ -439,8 +439,7 @@ constexpr int PROLOG_BIG_T = 128;   // token count from which the query product 
 // ------------------------------------------------------------------------------------------------ key path, weights
 __device__ __forceinline__ float block_sum128(float v, float* red)
 {
-#pragma unroll
-    for (int d = 1; d < 64; d <<= 1) v += __shfl_xor(v, d);
+    v = wave_sum_butterfly(v);
     __syncthreads();
     if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = v;
     __syncthreads();
