@@ -262,15 +262,38 @@ __global__ __launch_bounds__(128) void gqa_combine_kernel(GqaArgs a)
     const int nvalid = (cur + a.chunk - 1) / a.chunk;
     const float* pm = a.part_ml + head_row * a.nsplit * 2;
     const float* po = a.part_o + head_row * a.nsplit * GD + d0;
+    // eight chunks' loads in flight at a time (a chunk past the last valid one re-reads the last and is dropped): the
+    // additions keep the order of the chunks
+    constexpr int G = 8;
     float M = -INFINITY;
-    for (int s = 0; s < nvalid; ++s) M = fmaxf(M, pm[2 * s]);
+    for (int s0 = 0; s0 < nvalid; s0 += G) {
+        float m[G];
+#pragma unroll
+        for (int j = 0; j < G; ++j) m[j] = pm[2 * min(s0 + j, nvalid - 1)];
+#pragma unroll
+        for (int j = 0; j < G; ++j) M = fmaxf(M, m[j]);
+    }
     float L = 0.f;
     f32x4 acc = {0.f, 0.f, 0.f, 0.f};
     if (M > -INFINITY) {
-        for (int s = 0; s < nvalid; ++s) {
-            const float wgt = exp2f(pm[2 * s] - M);
-            L += wgt * pm[2 * s + 1];
-            acc += *reinterpret_cast<const f32x4*>(po + (int64_t)s * GD) * wgt;
+        for (int s0 = 0; s0 < nvalid; s0 += G) {
+            f32x4 v[G];
+            float m[G], l[G];
+#pragma unroll
+            for (int j = 0; j < G; ++j) {
+                const int s = min(s0 + j, nvalid - 1);
+                m[j] = pm[2 * s];
+                l[j] = pm[2 * s + 1];
+                v[j] = *reinterpret_cast<const f32x4*>(po + (int64_t)s * GD);
+            }
+#pragma unroll
+            for (int j = 0; j < G; ++j) {
+                if (s0 + j < nvalid) {
+                    const float wgt = exp2f(m[j] - M);
+                    L += wgt * l[j];
+                    acc += v[j] * wgt;
+                }
+            }
         }
     }
     const float inv = L > 0.f ? 1.f / L : 0.f;
