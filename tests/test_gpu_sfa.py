@@ -85,7 +85,7 @@ def test_bf16_cache(cuda):
     full_check(run_sfa(case, cuda), case, "bf16 cache")
 
 
-@pytest.mark.parametrize("nq", [16, 48, 64, 96, 128])
+@pytest.mark.parametrize("nq", [16, 48, 64, 96, 128, 200])
 def test_head_counts(cuda, nq):
     case = osfa.make_case(2, nq, 1, [2500, 40], topk=512, seed=nq, dist="bench", softmax_scale=192 ** -0.5)
     full_check(run_sfa(case, cuda), case, f"nq={nq}")
