@@ -4,15 +4,17 @@ Plays the role of the reference's call path ``JitCallableWrapper.__call__`` ->
 ``LaunchKernelTorch`` (python/pypto/frontend/parser/entry.py:296-365,518-583,638-662 and
 python/src/bindings/runtime.cpp:625-723): split positional/keyword arguments into tensors and
 scalars, check that every tensor is a contiguous torch.Tensor on one device, allocate the workspace
-through the torch allocator and launch asynchronously on the caller's current stream.  PyTorch is
-used for device memory and streams only; all compute is in the HIP library.
+through the torch allocator and launch asynchronously on the caller's current stream.  The checks, the
+descriptor list and the launch are C++ (csrc/host_binding.cpp, a pybind11 module over the C ABI);
+this file holds the scalar-parameter blocks, the call convention of the operators and a ctypes
+binding of the same C ABI for tests and measurement hooks.  PyTorch is used for device memory and
+streams only; all compute is in the HIP library.
 """
 import ctypes
 import functools
 import os
 import struct
 import threading
-import weakref
 
 import torch
 
@@ -21,7 +23,8 @@ from .error import FeError, PyptoError, PyptoRtError
 # PYPTO_AMD_LIBRARY names another build of the library (e.g. the host-sanitizer build of pypto_amd.build)
 _LIB_PATH = os.environ.get("PYPTO_AMD_LIBRARY") or os.path.join(os.path.dirname(os.path.abspath(__file__)), "libpypto_amd.so")
 _lib = None
-_lib_lock = threading.Lock()
+_lib_lock = threading.RLock()
+ABI_VERSION = 2  # include/pypto_amd.h: every launch ends in (workspace, workspace_bytes, hip_stream, sync)
 
 
 class TensorDesc(ctypes.Structure):
@@ -124,6 +127,10 @@ def load_library():
         lib.pto_last_error.restype = ctypes.c_char_p
         lib.pto_last_error.argtypes = []
         lib.pto_abi_version.restype = ctypes.c_int
+        if lib.pto_abi_version() != ABI_VERSION:
+            raise PyptoRtError(RuntimeError(
+                f"{_LIB_PATH} has ABI version {lib.pto_abi_version()}, this package needs {ABI_VERSION}: rebuild it "
+                f"with `python -m pypto_amd.build`"))
         _lib = lib
     return _lib
 
@@ -151,164 +158,72 @@ def describe(tensors):
     return (TensorDesc * n).from_buffer(buf)
 
 
-def _check_and_describe(tensors):
-    """The checks of the reference's binding (every operand a dense torch.Tensor, all on one HIP device) and the
-    descriptor array, in one pass over the tensors: this is the host's cost of a call, and it shows for the operators
-    whose kernels take a few tens of microseconds."""
-    n = len(tensors)
-    buf = bytearray(_DESC.size * n)
-    off = 0
-    dev = None
-    for idx, t in enumerate(tensors):
-        if type(t) is not torch.Tensor:
-            if not isinstance(t, torch.Tensor):
-                raise FeError(RuntimeError(f"Input {idx + 1} (index {idx}) must be a torch.Tensor, got {t.__class__}"))
-            if type(t).__name__ == "DTensor":
-                raise FeError(RuntimeError(f"Input {idx + 1} (index {idx}) must not be a DTensor, got {t.__class__}"))
-        if not t.is_contiguous():
-            raise FeError(RuntimeError("not all tensors are contiguous"))
-        d = t.device
-        if dev is None:
-            dev = d
-        elif d != dev:
-            raise FeError(RuntimeError(f"all tensors must be on the same device, got {dev} and {d}"))
-        code = _DTYPE_CODE.get(t.dtype)
-        if code is None:
-            raise ValueError(f"unsupported tensor dtype {t.dtype}")
-        shape = t.shape
-        r = len(shape)
-        if r > 8:
-            raise ValueError("tensors of more than 8 dimensions are not supported")
-        _DESC.pack_into(buf, off, t.data_ptr() if t.numel() else 0, code, r, *shape, *_PAD[r])
-        off += _DESC.size
-    if dev.type != "cuda":
-        raise FeError(RuntimeError(f"tensors must be on a HIP device (torch device type 'cuda'), got {dev}"))
-    descs = (TensorDesc * n).from_buffer(buf)
-    descs._buf = buf  # (the planned path rewrites addresses in place)
-    return dev, descs
+_host_mod = None
 
 
-_fns = {}
+def load_host():
+    """The pybind11 layer (pypto_amd/_host.so, built by ``python -m pypto_amd.build``): the product's call path from
+    torch tensors to the C ABI.  There is no fallback: without it every operator call fails."""
+    global _host_mod
+    if _host_mod is not None:
+        return _host_mod
+    load_library()  # the C ABI library first: a clear message when it is the one that is missing
+    with _lib_lock:
+        if _host_mod is None:
+            try:
+                from . import _host
+            except ImportError as e:
+                raise PyptoRtError(RuntimeError(
+                    f"pypto_amd._host is missing or does not load ({e}): build it with `python -m pypto_amd.build`")) from None
+            if _host.ABI_VERSION != ABI_VERSION:
+                raise PyptoRtError(RuntimeError(
+                    f"pypto_amd._host was built against ABI version {_host.ABI_VERSION}, this package needs "
+                    f"{ABI_VERSION}: rebuild with `python -m pypto_amd.build`"))
+            for op, ptype in _OPS.items():
+                if _host.PARAM_BYTES[op] != ctypes.sizeof(ptype):
+                    raise PyptoRtError(RuntimeError(f"parameter block of '{op}' differs between Python and pypto_amd._host"))
+            addr = lambda f: ctypes.cast(f, ctypes.c_void_p).value
+            _host.bind({op: (addr(getattr(_lib, f"pto_{op}_workspace")), addr(getattr(_lib, f"pto_{op}_launch")))
+                        for op in _OPS}, addr(_lib.pto_last_error))
+            _host_mod = _host
+    return _host_mod
 
 
-def _entry_points(op):
-    fns = _fns.get(op)
-    if fns is None:
-        lib = load_library()
-        fns = _fns[op] = (getattr(lib, f"pto_{op}_workspace"), getattr(lib, f"pto_{op}_launch"))
-    return fns
-
-
-def _launch_on_current_device(dev, launch_fn, descs, n, params_ref, ws_bytes):
-    ws = torch.empty(ws_bytes, dtype=torch.uint8, device=dev) if ws_bytes else None
-    return launch_fn(descs, n, params_ref, ws.data_ptr() if ws is not None else None, ws_bytes,
-                     torch.cuda.current_stream(dev).cuda_stream, 0)
-
-
-class _Plan:
-    """What a call leaves behind for the next call of the same operator on the same thread: the checked descriptor
-    array and the workspace size.  The reference keeps a compiled kernel module per (operator, argument shapes) and
-    skips compilation on a hit (python/pypto/frontend/parser/entry.py:613-636, python/src/bindings/runtime.cpp:430-523);
-    what there is to skip here is the validation of the tensor list and the workspace query."""
-    __slots__ = ("refs", "shapes", "ptrs", "buf", "descs", "n", "params", "params_ref", "ws_bytes", "dev", "current")
-
-
-_tls = threading.local()
-_PTR = struct.Struct("P")
-
-
-def _check_one(idx, t, dev):
-    """The per-tensor checks of _check_and_describe for one operand of a planned call; returns its dtype code."""
-    if type(t) is not torch.Tensor:
-        if not isinstance(t, torch.Tensor):
-            raise FeError(RuntimeError(f"Input {idx + 1} (index {idx}) must be a torch.Tensor, got {t.__class__}"))
-        if type(t).__name__ == "DTensor":
-            raise FeError(RuntimeError(f"Input {idx + 1} (index {idx}) must not be a DTensor, got {t.__class__}"))
-    if not t.is_contiguous():
-        raise FeError(RuntimeError("not all tensors are contiguous"))
-    if t.device != dev:
-        raise FeError(RuntimeError(f"all tensors must be on the same device, got {dev} and {t.device}"))
-    code = _DTYPE_CODE.get(t.dtype)
-    if code is None:
-        raise ValueError(f"unsupported tensor dtype {t.dtype}")
-    if len(t.shape) > 8:
-        raise ValueError("tensors of more than 8 dimensions are not supported")
-    return code
-
-
-def _refresh(plan, tensors, params, ws_fn):
-    """Brings the plan up to date with this call, operand by operand: an operand that is the very object of the planned
-    call, unchanged in shape and layout, only has its address looked at (storage can be reallocated under a live
-    tensor); any other operand - another layer's weights, a new activation - is checked and described afresh.  The
-    workspace is sized again only if a shape or the scalar parameters changed.  False: plan from scratch."""
-    if plan.n != len(tensors):
-        return False
-    resize = False
-    pb = bytes(params)
-    if pb != plan.params:
-        plan.params = pb
-        plan.params_ref = ctypes.byref(params.__class__.from_buffer_copy(pb))
-        resize = True
-    refs, shapes, ptrs, buf, dev = plan.refs, plan.shapes, plan.ptrs, plan.buf, plan.dev
-    i = 0
-    for t in tensors:
-        if refs[i]() is t and t.shape == shapes[i] and t.is_contiguous():
-            p = t.data_ptr() if ptrs[i] else 0  # (an empty tensor's descriptor carries a null address)
-            if p != ptrs[i]:
-                _PTR.pack_into(buf, i * _DESC.size, p)
-                ptrs[i] = p
-        else:
-            code = _check_one(i, t, dev)
-            shape = t.shape
-            r = len(shape)
-            p = t.data_ptr() if t.numel() else 0
-            _DESC.pack_into(buf, i * _DESC.size, p, code, r, *shape, *_PAD[r])
-            resize = resize or shape != shapes[i]
-            refs[i], shapes[i], ptrs[i] = weakref.ref(t), shape, p
-        i += 1
-    if resize:
-        plan.ws_bytes = ws_fn(plan.descs, plan.n, plan.params_ref)
-    return True
+_op_ids = {}
 
 
 def launch(op, tensors, params):
-    """Validate, size the workspace, launch on the current stream of the tensors' device.  A repeated call of an
-    operator takes the planned path (_refresh)."""
-    plans = getattr(_tls, "plans", None)
-    if plans is None:
-        plans = _tls.plans = {}
-    ws_fn, launch_fn = _entry_points(op)
-    plan = plans.get(op)
+    """Validate, size the workspace, launch on the current stream of the tensors' device: one call into the pybind11
+    layer (csrc/host_binding.cpp), which checks the operands the way the reference's binding does
+    (python/src/bindings/torch_tensor_converter.cpp:91-214), fills the descriptor list and calls the C ABI."""
+    op_id = _op_ids.get(op)
+    if op_id is None:
+        op_id = _op_ids[op] = load_host().OPS[op]
     try:
-        hit = plan is not None and _refresh(plan, tensors, params, ws_fn)
-    except Exception:
-        plans.pop(op, None)  # the buffer may be half rewritten
-        raise
-    if not hit:
-        dev, descs = _check_and_describe(tensors)
-        plan = _Plan()
-        plan.n = len(tensors)
-        plan.refs = [weakref.ref(t) for t in tensors]
-        plan.shapes = [t.shape for t in tensors]
-        plan.ptrs = [t.data_ptr() if t.numel() else 0 for t in tensors]
-        plan.descs = descs
-        plan.buf = descs._buf
-        plan.params = bytes(params)
-        plan.params_ref = ctypes.byref(params.__class__.from_buffer_copy(plan.params))
-        plan.ws_bytes = ws_fn(descs, plan.n, plan.params_ref)
-        plan.dev = dev
-        plan.current = dev.index is None
-        plans[op] = plan
-    dev = plan.dev
-    if plan.current or dev.index == torch.cuda.current_device():
-        rc = _launch_on_current_device(dev, launch_fn, plan.descs, plan.n, plan.params_ref, plan.ws_bytes)
-    else:
-        with torch.cuda.device(dev):
-            rc = _launch_on_current_device(dev, launch_fn, plan.descs, plan.n, plan.params_ref, plan.ws_bytes)
+        _host_mod.launch(op_id, tensors, bytes(params))
+    except _host_mod.BindingError as e:
+        raise FeError(RuntimeError(str(e))) from None
+
+
+def launch_ctypes(op, tensors, params, workspace=None, stream=None, sync=0):
+    """The same call through ctypes, every step spelled out: for tests of the C ABI and for callers that bring their own
+    workspace or stream (``workspace``: a uint8 tensor of at least the size the workspace query returns)."""
+    lib = load_library()
+    ws_fn, launch_fn = getattr(lib, f"pto_{op}_workspace"), getattr(lib, f"pto_{op}_launch")
+    descs = describe(tensors)
+    n = len(tensors)
+    dev = tensors[0].device
+    pref = ctypes.byref(params)
+    ws_bytes = ws_fn(descs, n, pref)
+    with torch.cuda.device(dev):
+        if workspace is None and ws_bytes:
+            workspace = torch.empty(ws_bytes, dtype=torch.uint8, device=dev)
+        s = torch.cuda.current_stream(dev).cuda_stream if stream is None else stream
+        rc = launch_fn(descs, n, pref, workspace.data_ptr() if workspace is not None else None,
+                       workspace.numel() if workspace is not None else 0, s, sync)
     if rc != 0:
-        plans.pop(op, None)
-        msg = _lib.pto_last_error().decode()
-        raise _STATUS_EXC.get(rc, RuntimeError)(msg)
+        raise _STATUS_EXC.get(rc, RuntimeError)(lib.pto_last_error().decode())
+    return ws_bytes
 
 
 def operator(n_tensors, scalar_names):

@@ -1,6 +1,7 @@
 """Builds libpypto_amd.so (HIP kernels + C ABI) for gfx950, in-tree, with hipcc.
 
-    python -m pypto_amd.build            # compile
+    python -m pypto_amd.build            # compile the library, then the pybind11 layer on top of it (_host.so)
+    python -m pypto_amd.build --host     # the pybind11 layer only
     python -m pypto_amd.build --verbose  # also print register / LDS usage per kernel
     python -m pypto_amd.build --sanitize # host code with AddressSanitizer and UndefinedBehaviorSanitizer, into
                                          # libpypto_amd_san.so: for the boundary's validation paths on a machine
@@ -42,6 +43,32 @@ def build(verbose=False):
     return LIB_PATH
 
 
+HOST_PATH = os.path.join(HERE, "_host.so")
+
+
+def build_host():
+    """The pybind11 layer (csrc/host_binding.cpp -> pypto_amd/_host.so): host C++ only, compiled with g++ against the
+    torch headers and linked to torch's HIP stream / allocator libraries; the C entry points of libpypto_amd.so are handed
+    to it by address at load time (pypto_amd/_runtime.py), so it does not link against the library."""
+    import sysconfig
+    import torch
+    from torch.utils import cpp_extension as ce
+    torch_lib = ce.library_paths()[0]
+    cxx = os.environ.get("CXX", "g++")
+    cmd = [cxx, "-O2", "-std=c++17", "-fPIC", "-shared", "-fvisibility=hidden", "-Wno-deprecated-declarations",
+           "-D__HIP_PLATFORM_AMD__=1", "-DUSE_ROCM=1", "-DTORCH_EXTENSION_NAME=_host", "-DTORCH_API_INCLUDE_EXTENSION_H",
+           f"-D_GLIBCXX_USE_CXX11_ABI={int(torch._C._GLIBCXX_USE_CXX11_ABI)}"]
+    for inc in ce.include_paths() + [sysconfig.get_paths()["include"], "/opt/rocm/include", INCLUDE]:
+        cmd += ["-isystem" if "torch" in inc or "rocm" in inc else "-I", inc]
+    cmd += [os.path.join(CSRC, "host_binding.cpp"), "-o", HOST_PATH,
+            "-L", torch_lib, "-lc10", "-lc10_hip", "-ltorch_cpu", "-ltorch_hip", "-ltorch",
+            "-ltorch_python", f"-Wl,-rpath,{torch_lib}"]
+    res = subprocess.run(cmd, capture_output=True, text=True)
+    if res.returncode != 0:
+        raise RuntimeError("host binding build failed:\n" + res.stderr)
+    return HOST_PATH
+
+
 SAN_LIB_PATH = os.path.join(HERE, "libpypto_amd_san.so")
 
 
@@ -70,4 +97,10 @@ def sanitizer_runtime():
 
 
 if __name__ == "__main__":
-    print(build_sanitized() if "--sanitize" in sys.argv else build(verbose="--verbose" in sys.argv))
+    if "--sanitize" in sys.argv:
+        print(build_sanitized())
+    elif "--host" in sys.argv:
+        print(build_host())
+    else:
+        print(build(verbose="--verbose" in sys.argv))
+        print(build_host())

@@ -18,5 +18,5 @@ def cuda():
     if not torch.cuda.is_available():
         pytest.skip("no GPU visible")
     from pypto_amd import _runtime
-    _runtime.load_library()  # fails loudly when the HIP library is missing
+    _runtime.load_host()  # fails loudly when the HIP library or the pybind11 layer is missing
     return torch.device("cuda:0")
