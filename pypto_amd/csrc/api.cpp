@@ -1056,7 +1056,7 @@ const char* pto_kernel_name(int kernel_id)
                                   "sfa_combine_kernel", "indexer_select_kernel", "select_experts_kernel",
                                   "gqa_decode_kernel", "gqa_combine_kernel", "apq_norm_kernel", "prolog_qx_kernel", "apq_gemm_kernel",
                                   "prolog_k_kernel", "mla_xa_kernel", "mla_norm_kernel", "mla_qb_kernel",
-                                  "mla_wuk_kernel", "apq_head_kernel", "paged_gather_kernel", "indexer_zero_kernel"};
+                                  "mla_wuk_kernel", "apq_head_kernel", "paged_gather_kernel"};
     return kernel_id >= 0 && kernel_id < pto::KID_COUNT ? names[kernel_id] : "";
 }
 

@@ -15,12 +15,14 @@
 // the fp16 rounding are 4 VALU operations per (head, key), and the weighted head sum is a second MFMA
 // (v_mfma_f32_16x16x32_f16: row 0 of A holds w_scale, B is the fp16 tile just produced; every product of two
 // fp16 values is exact in fp32, so this is the golden's fp32 sum up to the order of additions).  Scores go to
-// a dense fp32 row per query token, and the top 11 bits of their order-preserving keys into a 2048-bin
-// histogram per query token (LDS per workgroup, flushed with global atomics).
+// a dense fp32 row per query token, and their order-preserving keys into a 256-bin histogram in LDS (score_bin:
+// quarter octaves).  Every workgroup owns a 2048-key span of its sequence and leaves its histogram in a slot of
+// its own in the workspace (16-bit counts): plain stores, nothing to clear beforehand and no global atomics.
 //
-// indexer_select_kernel: every workgroup scans the histogram for the bin B that holds the k-th largest key,
-// then files its 4096 scores: bins above B are winners, bin B goes to a tie list (both lists in the
-// workspace, appended with one global atomic per workgroup).
+// indexer_select_kernel: every workgroup adds up the spans' histograms of its query token, finds the bin B that
+// holds the k-th largest key, and files its 4096 scores: bins above B are winners, bin B goes to a tie list (both
+// lists in the workspace, appended with one global atomic per workgroup; the counters are cleared by the score
+// kernel).
 //
 // indexer_topk_kernel: one workgroup per query token takes the winners, picks the missing krem entries out of
 // the tie list by radix-selecting on the 64-bit words (key << 32 | ~index) (so equal keys resolve to the
@@ -37,15 +39,95 @@ constexpr int D = 128;          // index head dim
 constexpr int CHUNK = 512;      // keys per pass of a workgroup of the score kernel (8 groups of 16 per wavefront)
 constexpr int PASSES = 4;       // passes per workgroup (amortise the Q / w_scale set-up)
 constexpr int MAX_K = 2048;     // top-k capacity
-constexpr int NBINS = 2048;     // histogram over the top 11 key bits
+constexpr int NBINS = 2048;     // digit bins of the radix select and of the final ordering (11 bits)
+constexpr int SBINS = 256;      // bins of the selection histogram (score_bin)
 constexpr int SEL_CHUNK = 4096; // scores per workgroup of the select kernel
 constexpr int TIE_CAP = 8192;   // capacity of the per-row tie list
 
 __device__ __forceinline__ float f16_bits_to_f32(uint16_t h) { return (float)__builtin_bit_cast(_Float16, h); }
 __device__ __forceinline__ uint32_t score_key(float f) { return f32_to_ordered(f + 0.0f); } // -0 -> +0
+// Bin of a score key in the selection histogram, non-decreasing in the key: quarter octaves (sign, exponent, two
+// mantissa bits - the top 11 key bits) of the magnitudes 2^-20 .. 2^12, 128 bins for either sign; smaller and larger
+// magnitudes fall into the first and last bin of their sign.  Keys of one interior bin share their top 11 bits.
+__device__ __forceinline__ uint32_t score_bin(uint32_t key)
+{
+    constexpr int LO = (127 - 20) * 4; // exponent field and two mantissa bits of 2^-20
+    const int t = (int)(key >> 21);
+    return t >= 1024 ? 128u + (uint32_t)min(max(t - 1024 - LO, 0), 127) : (uint32_t)min(max(t - (1023 - LO - 127), 0), 127);
+}
+__device__ __forceinline__ bool score_bin_is_interior(uint32_t bin) { return (bin & 127u) != 0u && (bin & 127u) != 127u; }
+// Smallest and largest key of a bin (the first and last bin of a sign reach to the end of the sign's keys).
+__device__ __forceinline__ void score_bin_range(uint32_t bin, uint32_t& lo, uint32_t& hi)
+{
+    constexpr int LO = (127 - 20) * 4;
+    const uint32_t j = bin & 127u;
+    const uint32_t t = bin >= 128u ? 1024u + LO + j : j + (1023u - LO - 127u);
+    lo = j == 0u ? (bin & 128u) << 24 : t << 21;
+    hi = j == 127u ? ((bin & 128u) << 24) | 0x7fffffffu : (t << 21) | 0x1fffffu;
+}
+
 __device__ __forceinline__ uint64_t make_cand(uint32_t key, int idx)
 {
     return ((uint64_t)key << 32) | (uint32_t)(0xffffffffu - (uint32_t)idx);
+}
+
+// One step of a wavefront scan in the vector unit's own lane network (no trip through LDS): the value of the lane
+// CTRL names (row_shr:n = 0x110 + n within a row of 16 lanes, row_bcast15 = 0x142 / row_bcast31 = 0x143 across rows,
+// limited to the rows of ROW_MASK), IDENT where there is no such lane.
+template <int CTRL, int ROW_MASK>
+__device__ __forceinline__ uint32_t dpp_from(uint32_t v, uint32_t ident)
+{
+    return (uint32_t)__builtin_amdgcn_update_dpp((int)ident, (int)v, CTRL, ROW_MASK, 0xf, false);
+}
+
+// wavefront-wide inclusive prefix sum: lane l gets v[0] + .. + v[l]
+__device__ __forceinline__ uint32_t wave_prefix_sum(uint32_t v)
+{
+    v += dpp_from<0x111, 0xf>(v, 0u);
+    v += dpp_from<0x112, 0xf>(v, 0u);
+    v += dpp_from<0x114, 0xf>(v, 0u);
+    v += dpp_from<0x118, 0xf>(v, 0u);
+    v += dpp_from<0x142, 0xa>(v, 0u); // rows 1 and 3 add the totals of rows 0 and 2
+    v += dpp_from<0x143, 0xc>(v, 0u); // rows 2 and 3 add the total of rows 0 and 1
+    return v;
+}
+
+// wavefront-wide minimum / maximum, the same value in every lane
+__device__ __forceinline__ uint32_t wave_min(uint32_t v)
+{
+    v = min(v, dpp_from<0x111, 0xf>(v, 0xffffffffu));
+    v = min(v, dpp_from<0x112, 0xf>(v, 0xffffffffu));
+    v = min(v, dpp_from<0x114, 0xf>(v, 0xffffffffu));
+    v = min(v, dpp_from<0x118, 0xf>(v, 0xffffffffu));
+    v = min(v, dpp_from<0x142, 0xa>(v, 0xffffffffu));
+    v = min(v, dpp_from<0x143, 0xc>(v, 0xffffffffu));
+    return (uint32_t)__builtin_amdgcn_readlane((int)v, 63);
+}
+
+__device__ __forceinline__ uint32_t wave_max(uint32_t v)
+{
+    v = max(v, dpp_from<0x111, 0xf>(v, 0u));
+    v = max(v, dpp_from<0x112, 0xf>(v, 0u));
+    v = max(v, dpp_from<0x114, 0xf>(v, 0u));
+    v = max(v, dpp_from<0x118, 0xf>(v, 0u));
+    v = max(v, dpp_from<0x142, 0xa>(v, 0u));
+    v = max(v, dpp_from<0x143, 0xc>(v, 0u));
+    return (uint32_t)__builtin_amdgcn_readlane((int)v, 63);
+}
+
+// The workgroup's histograms (S1 query tokens, one 2048-key span) go to its own slots, as 16-bit counts (at most 2048
+// each), two per lane.  The span-0 workgroup also clears the select kernel's list counters of its query tokens.  256 lanes.
+template <int S1>
+__device__ __forceinline__ void flush_span_hist(const IndexerArgs& a, const uint32_t (*hist)[SBINS], int row0, int span, int tid)
+{
+    if (tid < SBINS / 2) {
+#pragma unroll
+        for (int s = 0; s < S1; ++s) {
+            const int64_t slot = (int64_t)(row0 + s) * a.pchunks + span;
+            reinterpret_cast<uint32_t*>(a.span_hist + slot * SBINS)[tid] = hist[s][2 * tid] | (hist[s][2 * tid + 1] << 16);
+        }
+    }
+    if (span == 0 && tid < 4 * S1) a.counters[(int64_t)row0 * 4 + tid] = 0u;
 }
 
 // S1 query tokens of one sequence share every key fragment.
@@ -53,7 +135,7 @@ __device__ __forceinline__ uint64_t make_cand(uint32_t key, int idx)
 template <int S1, bool POW2>
 __global__ __launch_bounds__(256) void indexer_score_kernel(IndexerArgs a)
 {
-    __shared__ uint32_t hist[S1][NBINS];
+    __shared__ __align__(16) uint32_t hist[S1][SBINS];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int l16 = lane & 15, g = lane >> 4;
     const int bi = blockIdx.y;
@@ -62,7 +144,7 @@ __global__ __launch_bounds__(256) void indexer_score_kernel(IndexerArgs a)
     if (blockIdx.x * (CHUNK * PASSES) >= L) return;
     const int row0 = bi * a.s1 + sgrp * S1;
 
-    for (int i = tid; i < S1 * NBINS; i += 256) (&hist[0][0])[i] = 0;
+    for (int i = tid; i < S1 * SBINS; i += 256) (&hist[0][0])[i] = 0;
 
     // int8 A fragments: head hb*16 + l16, bytes 64*ks + 16*g .. +15
     i32x4 qf[S1][4][2];
@@ -145,16 +227,13 @@ __global__ __launch_bounds__(256) void indexer_score_kernel(IndexerArgs a)
             if (ok && g == 0) {
                 const float sc = sum[0] * (present[j] ? f16_bits_to_f32(ksb[j]) : 0.f);
                 a.scores[(int64_t)(row0 + s) * a.score_stride + tok] = sc;
-                if (tok < eff) atomicAdd(&hist[s][score_key(sc) >> 21], 1u);
+                if (tok < eff) atomicAdd(&hist[s][score_bin(score_key(sc))], 1u);
             }
         }
     }
     } // pass
     __syncthreads();
-    for (int i = tid; i < S1 * NBINS; i += 256) {
-        const uint32_t c = (&hist[0][0])[i];
-        if (c) atomicAdd(a.hist + (int64_t)(row0 + i / NBINS) * NBINS + (i % NBINS), c);
-    }
+    flush_span_hist<S1>(a, hist, row0, (int)blockIdx.x, tid);
 }
 
 // relu(a) * 2^-11 and relu(b) * 2^-11, each rounded once to fp16, packed (a in the low half).  The int32 sums arrive
@@ -181,29 +260,37 @@ __device__ __forceinline__ uint32_t relu_scale_pack(int a, int b)
 // scores of a key group and lane group g keeps those of key group g - after four key groups lane l holds the score of
 // key l of the 64, next to that key's scale (loaded with one 128-byte instruction per 64 keys).
 constexpr int PPASSES = 4; // passes (of 512 keys) per workgroup of the paged kernel
+constexpr int SPAN = CHUNK * PPASSES; // keys per workgroup of either score kernel: one histogram slot
+static_assert(SPAN == CHUNK * PASSES, "both score kernels own spans of the same size");
 template <int S1>
 __global__ __launch_bounds__(256, S1 == 1 ? 3 : 2) void indexer_score_paged_kernel(IndexerArgs a)
 {
     constexpr int NBUF = 2; // half-pass buffers: NBUF-1 halves ahead (deeper prefetch measured no faster)
     constexpr int NHALF = 2 * PPASSES;
-    __shared__ uint32_t hist[S1][NBINS];
+    __shared__ __align__(16) uint32_t hist[S1][SBINS];
     __shared__ __align__(16) float s_sc[S1][CHUNK * PPASSES]; // the workgroup's scores, written out in one burst at the end
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int l16 = lane & 15, g = lane >> 4;
     const int sgrp = blockIdx.z;
     const int bs = a.block_size;
-    // The (sequence, 2048-key span) of this workgroup: by its place in the grid, or - when the span list exists - entry
-    // w of the list, w its place in launch order.  The list entry is fetched together with the sequence length and the
-    // page-table entries of the grid place; only if it names another span (ragged lengths) are those fetched again.
+    // The (sequence, 2048-key span) of this workgroup: by its place in the grid when every sequence fills its spans.
+    // With ragged lengths the workgroups that have work should be the first ones of the launch order, so that they
+    // spread evenly over the CUs: workgroup w (its place in launch order, sequence-major) takes the w-th span that
+    // holds keys.  Every wavefront finds it on its own from the sequence lengths (lane l holds sequences l, l + 64, ..;
+    // a wavefront prefix sum of the spans per sequence), which are fetched together with the page-table entries of the
+    // grid place; only if the span is another one (ragged lengths) are those fetched again.  Batches beyond
+    // SCAN_SEQS sequences keep the grid place.
     // Lane p takes the page-table entry of pass p and the sequence's first entry, and picks once the length is known:
     // it then holds the first cache row of pass p (-1: unmapped page); a pass past the end re-reads the sequence's
     // first page and is discarded.
     int bi = blockIdx.y, span = blockIdx.x;
     const uint32_t w = blockIdx.x + gridDim.x * blockIdx.y;
-    const bool listed = a.span_list != nullptr;
-    // (unconditional loads - from the lengths when there is no list - so that they travel with the ones below)
-    const uint32_t* lp = listed ? a.span_list : reinterpret_cast<const uint32_t*>(a.act_seq);
-    const uint32_t lp_count = lp[0], lp_item = lp[listed ? 1 + min(w, (uint32_t)SPAN_LIST_CAP - 1) : 0];
+    constexpr int SCAN_SEQS = 256;
+    const bool balanced = a.b <= SCAN_SEQS;
+    int lens[SCAN_SEQS / 64];
+    // (unconditional loads, so that they travel with the ones below)
+#pragma unroll
+    for (int j = 0; j < SCAN_SEQS / 64; ++j) lens[j] = a.act_seq[min(lane + 64 * j, a.b - 1)];
     int pg_mine, pg_first, L, mytok;
     auto fetch = [&]() {
         mytok = span * (CHUNK * PPASSES) + wave * 128 + (lane < PPASSES ? lane : 0) * CHUNK;
@@ -213,11 +300,26 @@ __global__ __launch_bounds__(256, S1 == 1 ? 3 : 2) void indexer_score_paged_kern
         L = min(a.act_seq[bi], a.max_ctx); // keys past the page table's reach do not exist
     };
     fetch();
-    if (listed) {
-        if (w >= lp_count) return;
-        if (lp_item != (((uint32_t)bi << 10) | (uint32_t)span)) {
-            bi = (int)(lp_item >> 10);
-            span = (int)(lp_item & 1023u);
+    if (balanced) {
+        uint32_t base = 0;
+        int fseq = -1, fspan = 0;
+#pragma unroll
+        for (int j = 0; j < SCAN_SEQS / 64; ++j) {
+            const int len = min(lens[j], a.max_ctx);
+            const uint32_t cnt = (lane + 64 * j < a.b && len > 0) ? (uint32_t)((len + CHUNK * PPASSES - 1) / (CHUNK * PPASSES)) : 0u;
+            const uint32_t incl = wave_prefix_sum(cnt), excl = incl - cnt;
+            const uint64_t hit = __ballot(w >= base + excl && w < base + incl); // at most one lane, in one round
+            if (hit != 0ull && fseq < 0) {
+                const int l = __builtin_ctzll(hit);
+                fseq = 64 * j + l;
+                fspan = (int)(w - base - (uint32_t)__builtin_amdgcn_readlane((int)excl, l));
+            }
+            base += (uint32_t)__builtin_amdgcn_readlane((int)incl, 63);
+        }
+        if (fseq < 0) return; // more workgroups than spans with keys
+        if (fseq != bi || fspan != span) {
+            bi = fseq;
+            span = fspan;
             fetch();
         }
     }
@@ -278,7 +380,7 @@ __global__ __launch_bounds__(256, S1 == 1 ? 3 : 2) void indexer_score_paged_kern
             const f16x4 wlo = *reinterpret_cast<const f16x4*>(a.weights + h), whi = *reinterpret_cast<const f16x4*>(a.weights + h + 16);
             wa[s][mm] = __builtin_shufflevector(qlo * wlo, qhi * whi, 0, 1, 2, 3, 4, 5, 6, 7);
         }
-    for (int i = tid; i < S1 * NBINS; i += 256) (&hist[0][0])[i] = 0;
+    for (int i = tid; i < S1 * SBINS; i += 256) (&hist[0][0])[i] = 0;
     __syncthreads();
 
     auto compute_half = [&](int hh, int buf) {
@@ -311,7 +413,7 @@ __global__ __launch_bounds__(256, S1 == 1 ? 3 : 2) void indexer_score_paged_kern
             const float sc = res[s] * ks;
             s_sc[s][tok - span * (CHUNK * PPASSES)] = sc;
             const int eff = L - (a.s1 - 1 - (sgrp * S1 + s));
-            if (tok < eff) atomicAdd(&hist[s][score_key(sc) >> 21], 1u);
+            if (tok < eff) atomicAdd(&hist[s][score_bin(score_key(sc))], 1u);
         }
     };
 
@@ -339,60 +441,13 @@ __global__ __launch_bounds__(256, S1 == 1 ? 3 : 2) void indexer_score_paged_kern
         for (int i = 0; i < CHUNK * PPASSES / 1024; ++i)
             *reinterpret_cast<f32x4*>(dst + 4 * (tid + 256 * i)) = *reinterpret_cast<const f32x4*>(&s_sc[s][4 * (tid + 256 * i)]);
     }
-    for (int i = tid; i < S1 * NBINS; i += 256) {
-        const uint32_t c = (&hist[0][0])[i];
-        if (c) atomicAdd(a.hist + (int64_t)(row0 + i / NBINS) * NBINS + (i % NBINS), c);
-    }
+    flush_span_hist<S1>(a, hist, row0, span, tid);
 }
 
 __global__ void indexer_fill_kernel(int32_t* p, int n, int32_t v)
 {
     const int i = blockIdx.x * blockDim.x + threadIdx.x;
     if (i < n) p[i] = v;
-}
-
-// One step of a wavefront scan in the vector unit's own lane network (no trip through LDS): the value of the lane
-// CTRL names (row_shr:n = 0x110 + n within a row of 16 lanes, row_bcast15 = 0x142 / row_bcast31 = 0x143 across rows,
-// limited to the rows of ROW_MASK), IDENT where there is no such lane.
-template <int CTRL, int ROW_MASK>
-__device__ __forceinline__ uint32_t dpp_from(uint32_t v, uint32_t ident)
-{
-    return (uint32_t)__builtin_amdgcn_update_dpp((int)ident, (int)v, CTRL, ROW_MASK, 0xf, false);
-}
-
-// wavefront-wide inclusive prefix sum: lane l gets v[0] + .. + v[l]
-__device__ __forceinline__ uint32_t wave_prefix_sum(uint32_t v)
-{
-    v += dpp_from<0x111, 0xf>(v, 0u);
-    v += dpp_from<0x112, 0xf>(v, 0u);
-    v += dpp_from<0x114, 0xf>(v, 0u);
-    v += dpp_from<0x118, 0xf>(v, 0u);
-    v += dpp_from<0x142, 0xa>(v, 0u); // rows 1 and 3 add the totals of rows 0 and 2
-    v += dpp_from<0x143, 0xc>(v, 0u); // rows 2 and 3 add the total of rows 0 and 1
-    return v;
-}
-
-// wavefront-wide minimum / maximum, the same value in every lane
-__device__ __forceinline__ uint32_t wave_min(uint32_t v)
-{
-    v = min(v, dpp_from<0x111, 0xf>(v, 0xffffffffu));
-    v = min(v, dpp_from<0x112, 0xf>(v, 0xffffffffu));
-    v = min(v, dpp_from<0x114, 0xf>(v, 0xffffffffu));
-    v = min(v, dpp_from<0x118, 0xf>(v, 0xffffffffu));
-    v = min(v, dpp_from<0x142, 0xa>(v, 0xffffffffu));
-    v = min(v, dpp_from<0x143, 0xc>(v, 0xffffffffu));
-    return (uint32_t)__builtin_amdgcn_readlane((int)v, 63);
-}
-
-__device__ __forceinline__ uint32_t wave_max(uint32_t v)
-{
-    v = max(v, dpp_from<0x111, 0xf>(v, 0u));
-    v = max(v, dpp_from<0x112, 0xf>(v, 0u));
-    v = max(v, dpp_from<0x114, 0xf>(v, 0u));
-    v = max(v, dpp_from<0x118, 0xf>(v, 0u));
-    v = max(v, dpp_from<0x142, 0xa>(v, 0u));
-    v = max(v, dpp_from<0x143, 0xc>(v, 0u));
-    return (uint32_t)__builtin_amdgcn_readlane((int)v, 63);
 }
 
 // block-wide inclusive suffix sum (lane t gets sum of v[t .. nthreads-1]); tmp holds one word per wavefront
@@ -414,39 +469,6 @@ __device__ __forceinline__ uint32_t block_suffix_sum(uint32_t v, uint32_t* tmp)
     return v + add;
 }
 
-// Clears the histograms and counters; its first workgroup also lists the 2048-key spans that hold keys, in launch
-// order of the score kernel's grid (sequence-major): span_list[0] = their number, span_list[1 + i] = sequence << 10 | span.
-// The score kernel's workgroup i takes entry i, so that with ragged lengths the workgroups that have work are the
-// first ones of the launch order and spread evenly over the CUs (when every sequence fills its spans the list is the
-// identity and changes nothing).  256 lanes per workgroup.
-__global__ __launch_bounds__(256) void indexer_zero_kernel(uint32_t* p, int n, const int32_t* act_seq, int b, int pchunks,
-                                                           int max_ctx, uint32_t* span_list)
-{
-    const int i = blockIdx.x * blockDim.x + threadIdx.x;
-    if (i < n) p[i] = 0u;
-    if (blockIdx.x != 0 || span_list == nullptr) return;
-    __shared__ uint32_t tmp[4];
-    __shared__ uint32_t s_total;
-    const int tid = threadIdx.x;
-    uint32_t base_off = 0;
-    for (int base = 0; base < b; base += 256) {
-        const int seq = base + tid;
-        uint32_t cnt = 0;
-        if (seq < b) {
-            const int L = min(act_seq[seq], max_ctx);
-            cnt = L > 0 ? (uint32_t)min((L + CHUNK * PPASSES - 1) / (CHUNK * PPASSES), pchunks) : 0u;
-        }
-        const uint32_t suffix = block_suffix_sum<4>(cnt, tmp); // sum over lanes tid .. 255
-        if (tid == 0) s_total = suffix;
-        __syncthreads();
-        const uint32_t off = base_off + (s_total - suffix); // spans of the sequences before this one
-        for (uint32_t j = 0; j < cnt; ++j) span_list[1 + off + j] = ((uint32_t)seq << 10) | j;
-        base_off += s_total;
-        __syncthreads();
-    }
-    if (tid == 0) span_list[0] = base_off;
-}
-
 // Valid length of query token `row`'s score row: the sequence's length, cut to what the page table can address
 // (the score kernels write no score beyond that), less the query tokens that come after this one.
 __device__ __forceinline__ int row_length(const int32_t* act_seq, int row, int s1, int max_ctx)
@@ -460,37 +482,77 @@ __global__ __launch_bounds__(256) void indexer_select_kernel(IndexerArgs a)
 {
     __shared__ uint32_t tmp[4];
     __shared__ uint32_t s_bin, s_base_gt, s_base_tie;
+    __shared__ __align__(16) uint32_t s_hist[4][SBINS];
     const int tid = threadIdx.x, row = blockIdx.y;
     const int i_begin = blockIdx.x * SEL_CHUNK;
-    // everything this workgroup reads is requested at once - the row's length, its histogram (lane t owns bins
-    // 8t .. 8t+7) and the workgroup's 16 scores per lane (addresses clamped to the padded row) - one round trip, not three
-    const uint32_t* hist = a.hist + (int64_t)row * NBINS;
-    const u32x4 ha = *reinterpret_cast<const u32x4*>(hist + 8 * tid);
-    const u32x4 hb = *reinterpret_cast<const u32x4*>(hist + 8 * tid + 4);
+    // everything this workgroup reads is requested at once - the row's length, the histograms of the first GROUP spans
+    // and the workgroup's 16 scores per lane (addresses clamped to the padded row) - one round trip.  The histograms
+    // are read as they lie in memory, 16 bytes per lane: lane l takes bins 8 (l % 32) .. + 7 of spans l / 32,
+    // l / 32 + 8, ..  A slot of a span without keys was never written: it is requested all the same (workspace
+    // memory) and left out of the sum once the length is known.
+    constexpr int GROUP = 32;
+    const int sg = tid >> 5, oct = tid & 31;
+    const uint16_t* sh = a.span_hist + (int64_t)row * a.pchunks * SBINS + 8 * oct;
+    u32x4 cv[GROUP / 8];
+#pragma unroll
+    for (int j = 0; j < GROUP / 8; ++j) cv[j] = *reinterpret_cast<const u32x4*>(sh + (int64_t)min(sg + 8 * j, a.pchunks - 1) * SBINS);
     const float* x = a.scores + (int64_t)row * a.score_stride;
     f32x4 v[4];
 #pragma unroll
     for (int j = 0; j < 4; ++j) v[j] = *reinterpret_cast<const f32x4*>(x + min(i_begin + 4 * (j * 256 + tid), a.score_stride - 4));
-    const int n = row_length(a.act_seq, row, a.s1, a.max_ctx);
-    if (i_begin >= n) return;
+    const int bi = row / a.s1;
+    const int len = min(a.act_seq[bi], a.max_ctx);
+    const int n = max(len - (a.s1 - 1 - (row - bi * a.s1)), 0);
+    // (a workgroup past the row's end leaves further down, behind the first use of what was requested above: an exit
+    // here would let the compiler move those requests behind the wait for the length - two round trips instead of one)
+    const int nsp = min((len + SPAN - 1) / SPAN, a.pchunks); // spans whose workgroup ran
     if (tid == 0) s_bin = 0xffffffffu; // n <= k: no threshold bin, everything is a winner
 
-    // bin of the k-th largest key
-    const uint32_t h[8] = {ha[0], ha[1], ha[2], ha[3], hb[0], hb[1], hb[2], hb[3]};
-    uint32_t own = 0;
+    uint32_t acc[8] = {0u, 0u, 0u, 0u, 0u, 0u, 0u, 0u};
+    for (int g0 = 0; g0 < nsp; g0 += GROUP) { // (one trip but for contexts beyond GROUP spans; block-uniform)
+        if (g0 > 0) {
 #pragma unroll
-    for (int j = 0; j < 8; ++j) own += h[j];
-    uint32_t above = block_suffix_sum<4>(own, tmp) - own; // elements in bins > 8t+7
+            for (int j = 0; j < GROUP / 8; ++j)
+                cv[j] = *reinterpret_cast<const u32x4*>(sh + (int64_t)min(g0 + sg + 8 * j, a.pchunks - 1) * SBINS);
+        }
+#pragma unroll
+        for (int j = 0; j < GROUP / 8; ++j) {
+            const bool in = g0 + sg + 8 * j < nsp;
+#pragma unroll
+            for (int c = 0; c < 4; ++c) {
+                acc[2 * c] += in ? cv[j][c] & 0xffffu : 0u;
+                acc[2 * c + 1] += in ? cv[j][c] >> 16 : 0u;
+            }
+        }
+    }
+    // the two span groups of a wavefront (lanes l and l + 32 hold the same bins), then the four wavefronts through LDS
+#pragma unroll
+    for (int c = 0; c < 8; ++c) {
+        const auto sw = __builtin_amdgcn_permlane32_swap(acc[c], acc[c], false, false);
+        acc[c] = (uint32_t)sw[0] + (uint32_t)sw[1];
+    }
+    if ((tid & 32) == 0) {
+        uint32_t* dst = &s_hist[tid >> 6][8 * oct];
+        *reinterpret_cast<u32x4*>(dst) = u32x4{acc[0], acc[1], acc[2], acc[3]};
+        *reinterpret_cast<u32x4*>(dst + 4) = u32x4{acc[4], acc[5], acc[6], acc[7]};
+    }
+    __syncthreads();
+    if (i_begin >= n) return;
+    // bin of the k-th largest key: lane t owns bin t
+    const uint32_t own = s_hist[0][tid] + s_hist[1][tid] + s_hist[2][tid] + s_hist[3][tid];
     const uint32_t k = (uint32_t)a.k;
-#pragma unroll
-    for (int j = 7; j >= 0; --j) {
-        if (above < k && k <= above + h[j]) s_bin = 8 * tid + j;
-        above += h[j];
+    {
+        const uint32_t above = block_suffix_sum<4>(own, tmp) - own; // elements in the bins above
+        if (above < k && k <= above + own) s_bin = (uint32_t)tid;
     }
     __syncthreads();
     const uint32_t bin = s_bin;
 
-    // file this workgroup's scores: 16 per lane
+    // file this workgroup's scores: 16 per lane.  A score's side of the threshold bin is read off its key: winners lie
+    // above the bin's largest key, ties between its smallest and largest.  Without a threshold bin every key is a winner.
+    uint32_t key_lo = 0u, key_hi = 0u;
+    const bool all_win = bin == 0xffffffffu;
+    if (!all_win) score_bin_range(bin, key_lo, key_hi);
     uint32_t key[16];
     uint32_t c_gt = 0, c_tie = 0;
 #pragma unroll
@@ -500,10 +562,9 @@ __global__ __launch_bounds__(256) void indexer_select_kernel(IndexerArgs a)
             const int i = i_begin + 4 * (j * 256 + tid) + c;
             const uint32_t u = score_key(v[j][c]);
             key[4 * j + c] = u;
-            const uint32_t b = u >> 21;
             const bool in = i < n;
-            c_gt += in && (bin == 0xffffffffu || b > bin) ? 1u : 0u;
-            c_tie += in && b == bin ? 1u : 0u;
+            c_gt += in && (all_win || u > key_hi) ? 1u : 0u;
+            c_tie += in && !all_win && u >= key_lo && u <= key_hi ? 1u : 0u;
         }
     const uint32_t packed = block_suffix_sum<4>(c_gt | (c_tie << 16), tmp);
     if (tid == 0) {
@@ -521,15 +582,14 @@ __global__ __launch_bounds__(256) void indexer_select_kernel(IndexerArgs a)
 #pragma unroll
         for (int c = 0; c < 4; ++c) {
             const int i = i_begin + 4 * (j * 256 + tid) + c;
-            if (i >= n) continue;
-            const uint32_t u = key[4 * j + c], b = u >> 21;
-            if (bin == 0xffffffffu || b > bin) {
-                if (p_gt < MAX_K) winners[p_gt] = make_cand(u, i);
-                ++p_gt;
-            } else if (b == bin) {
-                if (p_tie < TIE_CAP) ties[p_tie] = make_cand(u, i);
-                ++p_tie;
-            }
+            const uint32_t u = key[4 * j + c];
+            const bool in = i < n;
+            const bool gt = in && (all_win || u > key_hi), tie = in && !all_win && u >= key_lo && u <= key_hi;
+            // (one store per element, to whichever list takes it)
+            uint64_t* dst = gt ? winners + p_gt : ties + p_tie;
+            if ((gt && p_gt < MAX_K) || (tie && p_tie < TIE_CAP)) *dst = make_cand(u, i);
+            p_gt += gt ? 1u : 0u;
+            p_tie += tie ? 1u : 0u;
         }
 }
 
@@ -703,8 +763,10 @@ __global__ __launch_bounds__(1024) void indexer_topk_kernel(IndexerArgs a)
     const uint64_t t0 = tsrc[tid], t1 = tsrc[tid + 1024];
     const int n = row_length(a.act_seq, row, a.s1, a.max_ctx);
     const int k = a.k;
-    const uint32_t n_gt = min(a.counters[(int64_t)row * 4], (uint32_t)MAX_K);
-    const uint32_t n_tie = a.counters[(int64_t)row * 4 + 1];
+    // (the counters of a query token are cleared by its sequence's first score workgroup: a sequence without keys has none)
+    const uint32_t c_gt = a.counters[(int64_t)row * 4], c_tie = a.counters[(int64_t)row * 4 + 1];
+    const uint32_t n_gt = n > 0 ? min(c_gt, (uint32_t)MAX_K) : 0u;
+    const uint32_t n_tie = n > 0 ? c_tie : 0u;
     const uint32_t need = (uint32_t)min(n, k) - min(n_gt, (uint32_t)min(n, k));
 
     cand[tid] = tid < (int)n_gt ? w0 : 0ull;
@@ -719,7 +781,7 @@ __global__ __launch_bounds__(1024) void indexer_topk_kernel(IndexerArgs a)
     };
 
     if (need > 0 && n_tie <= TIE_CAP) {
-        // the usual case: the tie list (one histogram bin) fits in LDS; its words share the top 11 bits
+        // the usual case: the tie list (one histogram bin) fits in LDS
         if (n_tie > 2048) { // block-uniform
             for (int i = tid + 2048; i < (int)n_tie; i += 1024) tie[i] = tsrc[i];
             __syncthreads();
@@ -727,7 +789,10 @@ __global__ __launch_bounds__(1024) void indexer_topk_kernel(IndexerArgs a)
         auto each = [&](auto&& f) {
             for (int i = tid; i < (int)n_tie; i += 1024) f(tie[i]);
         };
-        radix_select64(each, emit, need, 53, hist, tmp, &s_bin, &s_krem, &s_cnt);
+        // the ties of an interior bin share their top 11 key bits; those of a first or last bin (magnitudes outside the
+        // histogram's range) need not
+        const int top = score_bin_is_interior(score_bin((uint32_t)(tie[0] >> 32))) ? 53 : 64;
+        radix_select64(each, emit, need, top, hist, tmp, &s_bin, &s_krem, &s_cnt);
     } else if (need > 0) {
         // overflowed tie list: select over the whole row instead (winners are found again, so start empty)
         if (tid == 0) s_out = 0;
@@ -825,28 +890,31 @@ hipError_t topk_launch(const float* x, float* values, int32_t* indices, int64_t 
     return hipGetLastError();
 }
 
-// workspace: scores [t, stride] f32 | hist [t, 2048] u32 | counters [t, 4] u32 | winners [t, 2048] u64 | ties [t, 8192] u64
+// workspace: scores [t, stride] f32 | span_hist [t, spans, 256] u16 | counters [t, 4] u32 | winners [t, 2048] u64 |
+// ties [t, 8192] u64; spans = stride / 2048
 static uint64_t align256(uint64_t x) { return (x + 255) & ~(uint64_t)255; }
 
 uint64_t indexer_workspace_bytes(int t, int stride)
 {
-    return align256((uint64_t)t * stride * 4) + align256((uint64_t)t * (NBINS + 4) * 4) +
-           align256((uint64_t)t * (MAX_K + TIE_CAP) * 8) + (1 + SPAN_LIST_CAP) * 4;
+    const uint64_t spans = (uint64_t)stride / SPAN;
+    return align256((uint64_t)t * stride * 4) + align256((uint64_t)t * spans * SBINS * 2) + align256((uint64_t)t * 4 * 4) +
+           align256((uint64_t)t * (MAX_K + TIE_CAP) * 8);
 }
 
 void indexer_bind_workspace(IndexerArgs& a, void* ws)
 {
     const int t = a.b * a.s1;
+    const uint64_t spans = (uint64_t)a.score_stride / SPAN;
     uint8_t* p = static_cast<uint8_t*>(ws);
     a.scores = reinterpret_cast<float*>(p);
     p += align256((uint64_t)t * a.score_stride * 4);
-    a.hist = reinterpret_cast<uint32_t*>(p);
-    a.counters = a.hist + (uint64_t)t * NBINS;
-    p += align256((uint64_t)t * (NBINS + 4) * 4);
+    a.span_hist = reinterpret_cast<uint16_t*>(p);
+    p += align256((uint64_t)t * spans * SBINS * 2);
+    a.counters = reinterpret_cast<uint32_t*>(p);
+    p += align256((uint64_t)t * 4 * 4);
     a.winners = reinterpret_cast<uint64_t*>(p);
     a.ties = a.winners + (uint64_t)t * MAX_K;
-    p += align256((uint64_t)t * (MAX_K + TIE_CAP) * 8);
-    a.span_list = reinterpret_cast<uint32_t*>(p); // the launch drops it when the grid does not fit
+    a.pchunks = (int32_t)spans;
 }
 
 hipError_t indexer_launch(const IndexerArgs& a, hipStream_t stream)
@@ -859,18 +927,11 @@ hipError_t indexer_launch(const IndexerArgs& a, hipStream_t stream)
         hipLaunchKernelGGL(indexer_fill_kernel, dim3((n + 255) / 256), dim3(256), 0, stream, a.topk_res, n, -1);
         return hipGetLastError();
     }
-    const int chunks = (max_ctx + CHUNK * PASSES - 1) / (CHUNK * PASSES);
-    const int pchunks = (max_ctx + CHUNK * PPASSES - 1) / (CHUNK * PPASSES);
-    const int nzero = t * (NBINS + 4);
+    // one workgroup per 2048-key span the page table can address (a.pchunks slots per query token hold at least as many)
+    const int chunks = (max_ctx + SPAN - 1) / SPAN;
+    const int pchunks = chunks;
     IndexerArgs args = a;
     args.max_ctx = max_ctx;
-    const bool paged = a.block_size % 128 == 0;
-    if (!paged || (int64_t)a.b * pchunks > SPAN_LIST_CAP || pchunks > 1024) args.span_list = nullptr;
-    {
-        ScopedKernelTimer tm(KID_INDEXER_ZERO, stream);
-        hipLaunchKernelGGL(indexer_zero_kernel, dim3((nzero + 255) / 256), dim3(256), 0, stream, a.hist, nzero, a.act_seq, a.b,
-                           pchunks, max_ctx, args.span_list);
-    }
     {
         ScopedKernelTimer tm(KID_INDEXER_SCORE, stream);
         const bool pow2 = (a.block_size & (a.block_size - 1)) == 0;

@@ -48,18 +48,16 @@ struct IndexerArgs {
     const int32_t* block_table;  // [b, bt_stride]
     int32_t* topk_res;           // [t, k]
     float* scores;               // workspace [t, score_stride]
-    uint32_t* hist;              // workspace [t, 2048]: histogram of the top 11 bits of the score keys
-    uint32_t* counters;          // workspace [t, 4]: winners, ties
+    uint16_t* span_hist;         // workspace [t, pchunks, 256]: per 2048-key span, histogram of the score keys (quarter octaves)
+    uint32_t* counters;          // workspace [t, 4]: winners, ties (cleared by the score kernel)
     uint64_t* winners;           // workspace [t, 2048]
     uint64_t* ties;              // workspace [t, 8192]
-    uint32_t* span_list;         // workspace [1 + SPAN_LIST_CAP]: count, then (sequence << 10 | span) of every 2048-key span
-                                 // that holds keys; nullptr when the grid is too large for the list
     int64_t n_blocks;
     int32_t b, s1, nh, block_size, bt_stride, k, score_stride;
     int32_t max_ctx; // set by indexer_launch: bt_stride * block_size, the longest sequence the page table can address
+    int32_t pchunks; // set by indexer_bind_workspace: histogram slots (2048-key spans) per query token = score_stride / 2048
 };
 
-constexpr int SPAN_LIST_CAP = 16384;
 uint64_t indexer_workspace_bytes(int t, int score_stride);
 void indexer_bind_workspace(IndexerArgs& a, void* workspace);
 hipError_t indexer_launch(const IndexerArgs& a, hipStream_t stream);

@@ -5,7 +5,7 @@
 
 namespace pto {
 
-enum KernelId { KID_INDEXER_SCORE = 0, KID_INDEXER_TOPK = 1, KID_SFA_DECODE = 2, KID_SFA_COMBINE = 3, KID_INDEXER_SELECT = 4, KID_SELECT_EXPERTS = 5, KID_GQA_DECODE = 6, KID_GQA_COMBINE = 7, KID_APQ_NORM = 8, KID_PROLOG_Q = 9, KID_APQ_GEMM = 10, KID_PROLOG_K = 11, KID_MLA_XA = 12, KID_MLA_NORM = 13, KID_MLA_QB = 14, KID_MLA_WUK = 15, KID_APQ_HEAD = 16, KID_PAGED_GATHER = 17, KID_INDEXER_ZERO = 18, KID_COUNT = 19 };
+enum KernelId { KID_INDEXER_SCORE = 0, KID_INDEXER_TOPK = 1, KID_SFA_DECODE = 2, KID_SFA_COMBINE = 3, KID_INDEXER_SELECT = 4, KID_SELECT_EXPERTS = 5, KID_GQA_DECODE = 6, KID_GQA_COMBINE = 7, KID_APQ_NORM = 8, KID_PROLOG_Q = 9, KID_APQ_GEMM = 10, KID_PROLOG_K = 11, KID_MLA_XA = 12, KID_MLA_NORM = 13, KID_MLA_QB = 14, KID_MLA_WUK = 15, KID_APQ_HEAD = 16, KID_PAGED_GATHER = 17, KID_COUNT = 18 };
 
 bool timing_enabled();
 void timing_set(bool on);
