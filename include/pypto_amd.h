@@ -48,7 +48,7 @@ enum PtoStatus {
     PTO_ERR_WORKSPACE = -5, /* workspace missing or too small */
     PTO_ERR_NULL = -6,      /* null device address */
     PTO_ERR_HIP = -7,       /* the HIP runtime reported an error on launch */
-    PTO_ERR_ALIGN = -8      /* a device address is not aligned as the operator needs (16 bytes; paged_gather: one element) */
+    PTO_ERR_ALIGN = -8      /* a device address is not aligned as the operator needs (16 bytes; paged_gather and topk: one element) */
 };
 
 /* Scalar arguments of sparse_flash_attention_quant_* / sparse_attention_antiquant_*

@@ -906,9 +906,11 @@ static int topk_launch_async(const PtoTensorDesc* ts, uint32_t n, const PtoTopkP
     if (ts == nullptr || n != 3) return fail(PTO_ERR_ARG_COUNT, "%s: expected 3 tensors, got %u", op, n);
     if (p == nullptr) return fail(PTO_ERR_PARAM, "%s: params is null", op);
     int rc;
-    if ((rc = check_tensor(op, ts[0], "input", PTO_DT_FP32, 2))) return rc;
-    if ((rc = check_tensor(op, ts[1], "values", PTO_DT_FP32, 2))) return rc;
-    if ((rc = check_tensor(op, ts[2], "indices", PTO_DT_INT32, 2))) return rc;
+    // (the kernel reads and writes single elements: element alignment is all it asks for, so a view that starts at any
+    // row of a tensor is a valid operand)
+    if ((rc = check_tensor(op, ts[0], "input", PTO_DT_FP32, 2, 4))) return rc;
+    if ((rc = check_tensor(op, ts[1], "values", PTO_DT_FP32, 2, 4))) return rc;
+    if ((rc = check_tensor(op, ts[2], "indices", PTO_DT_INT32, 2, 4))) return rc;
     const int64_t rows = ts[0].shape[0], len = ts[0].shape[1];
     if (ts[1].shape[0] != rows || ts[2].shape[0] != rows || ts[1].shape[1] != p->k || ts[2].shape[1] != p->k)
         return fail(PTO_ERR_SHAPE, "%s: values and indices must be [%lld, %d]", op, (long long)rows, p->k);

@@ -154,6 +154,38 @@ def test_forced_kv_splits_agree(cuda):
         assert count_violations(o, outs[0], 2e-3, 2.0 ** -5) == 0
 
 
+@pytest.mark.parametrize("packed", [False, True])
+@pytest.mark.parametrize("splits", [1, 8])
+def test_page_table_too_wide_for_lds(cuda, packed, splits):
+    """A page-table row that does not fit beside the kernel's other LDS arrays (4096 columns, the unused ones -1) is read
+    from global memory entry by entry instead of from an LDS copy.  Configuration 1's shape through the three-tensor
+    entry and the packed-row entry, at 1 and 8 forced KV splits: bit-equal to the same call with the table cut to
+    the columns in use (the LDS-copy path), and within the bars of the oracle.  Semantics of the unused columns:
+    models/deepseek_v32_exp/deepseekv32_sparse_flash_attention_quant.py:220-233."""
+    from pypto_amd import _runtime
+    case = osfa.make_case(1, 16, 1, [4096], topk=256, seed=7, dist="bench", softmax_scale=192 ** -0.5)
+    narrow = case["block_table"]
+    wide = torch.full((narrow.shape[0], 4096), -1, dtype=torch.int32)
+    wide[:, :narrow.shape[1]] = narrow
+    dev = cuda
+    q = case["q"]
+    head = [q[..., :512].reshape(-1, 512).contiguous().to(dev), q[..., 512:].reshape(-1, 64).contiguous().to(dev)]
+    if packed:
+        cache = [osfa.pack_cache_rows(case["kn"], case["kr"], case["kn_scales"]).to(dev)]
+    else:
+        cache = [case["kn"].to(dev), case["kr"].to(dev), case["kn_scales"].to(dev)]
+    tail = [case["topk_indices"].to(dev)]
+    act = torch.tensor(case["act_seq"], dtype=torch.int32, device=dev)
+    outs = []
+    for table in (narrow, wide):
+        out = torch.zeros((16, 512) if packed else (1, 1, 16, 512), dtype=torch.bfloat16, device=dev)
+        p = _runtime.SfaParams(16, 1, case["softmax_scale"], 256, 128, table.shape[1], splits)
+        _runtime.launch_ctypes("sfa_antiquant" if packed else "sfa_quant", head + cache + tail + [table.to(dev), act, out], p, sync=1)
+        outs.append(out.cpu().reshape(1, 1, 16, 512))
+    assert torch.equal(outs[0], outs[1]), "the table read from global memory must give the bits of the LDS copy"
+    full_check(outs[1], case, f"wide page table, packed={packed}, {splits} split(s)")
+
+
 def test_full_size_config5(cuda):
     # benchmark configuration 5: b=32, 128 heads, context lengths U[16384, 65536], top-2048, bench distribution
     g = torch.Generator().manual_seed(55)

@@ -58,6 +58,19 @@ def test_ties_zero_signs_and_whole_rows(cuda):
     check(torch.rand((6, 17), generator=g), 3, 0, False, cuda)     # the first dimension
 
 
+def test_row_slices_that_start_off_a_16_byte_boundary(cuda):
+    # x[1:] of rows of 3 floats starts 12 bytes into the allocation and is contiguous: a legal operand as it is
+    from pypto_amd.op import topk
+    g = torch.Generator().manual_seed(9)
+    x = torch.rand((5, 3), generator=g)
+    xd = x.to(cuda)
+    view = xd[1:]
+    assert view.is_contiguous() and view.data_ptr() % 16 != 0
+    vals, idx = topk(view, 2)
+    gv, gi = otopk.topk_rows(x[1:], 2, True)
+    assert torch.equal(idx.cpu(), gi) and torch.equal(vals.cpu(), gv)
+
+
 def test_long_rows_go_through_the_radix_select(cuda):
     g = torch.Generator().manual_seed(6)
     x = torch.randn((3, 131072), generator=g)

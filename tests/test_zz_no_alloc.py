@@ -11,6 +11,9 @@ import pytest
 import torch
 
 from oracle import sfa as osfa
+from oracle.compare import count_violations
+
+from _cases import sfa_golden
 
 pytestmark = pytest.mark.gpu
 
@@ -52,6 +55,8 @@ def test_no_alloc_entry_matches_the_workspace_entry_twice(cuda):
         want, got = both_entries(case, cuda)
         assert torch.isfinite(got.float()).all()
         assert torch.equal(got, want)
+        # and on its own against the oracle, to the attention tests' bar (every element within 1e-2 + 2e-2 |golden|)
+        assert count_violations(got, sfa_golden(case), 1e-2, 2e-2) == 0
 
 
 def test_no_alloc_entry_rejects_what_does_not_fit(cuda):
