@@ -25,19 +25,25 @@ sys.path.insert(0, ROOT)
 HBM_PEAK_GBS = 8000.0
 MFMA_BF16_PEAK_TFLOPS = 2500.0
 
-# HBM bytes per launch (read + written) from rocprofv3 FETCH_SIZE x 2.000 and WRITE_SIZE x 1.000, the factors being what
-# the same counters read for a 256 MiB-in / 256 MiB-out elementwise kernel (--calibrate-copy); measured on the default
-# workload only (batch 32, s1 1, ctx 65536, three cache tensors) and reported for that workload only.
-MEASURED_TRAFFIC_BYTES = {
-    "indexer_score_kernel": 275.6e6 + 8.9e6,
-    "sfa_decode_kernel": 55.9e6 + 35.1e6,
-    "sfa_combine_kernel": 34.7e6 + 4.2e6,
-    "indexer_select_kernel": 10.6e6 + 0.8e6,
-    "indexer_topk_kernel": 1.2e6 + 0.3e6,
-}
-# same counters and factors on the default shapes of --workload gqa and --workload paged_gather
-GQA_TRAFFIC_BYTES = 5150.7e6 + 65.8e6
-PAGED_GATHER_TRAFFIC_BYTES = 51.4e6 + 43.0e6
+def profile_traffic(name):
+    """HBM bytes per launch (read + written) of every kernel in the table of profiles/<name>: rocprofv3 FETCH_SIZE and
+    WRITE_SIZE per dispatch, each scaled by what the same counter reads for a plain elementwise kernel of known size
+    (the file says how it was made; --calibrate-copy puts that kernel into a counter run).  The figures belong to the
+    exact workload the file names and are reported for that workload only.  {} when the file is not there."""
+    path = os.path.join(ROOT, "profiles", name)
+    out, in_table = {}, False
+    if not os.path.exists(path):
+        return out
+    for line in open(path):
+        cols = line.split()
+        if cols[:2] == ["kernel", "FETCH_SIZE"]:
+            in_table = True
+        elif in_table:
+            if len(cols) < 5 or not cols[1].isdigit():
+                break
+            # columns: kernel, FETCH_SIZE KiB, read MB, WRITE_SIZE KiB, written MB; the kernel as bench.py names it
+            out[cols[0].split("<")[0].replace("_paged", "")] = (float(cols[2]) + float(cols[4])) * 1e6
+    return out
 
 
 def parse():
@@ -53,6 +59,8 @@ def parse():
     ap.add_argument("--cpu-seqs", type=int, default=8, help="sequences of the workload timed on the CPU oracle")
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--packed", action="store_true", help="use the packed 656-byte-row attention entry point")
+    ap.add_argument("--fp32-scales", action="store_true",
+                    help="indexer query / key scales as fp32 tensors (the default is fp16, the reference operator's signature)")
     ap.add_argument("--workload", choices=["v32", "gqa", "select_experts", "indexer_prolog", "mla_prolog", "mla_indexer_prolog", "decode_layer", "attention_pre_quant", "sfa_prefill", "paged_gather"], default="v32",
                     help="v32 (default): the headline DeepSeek-V3.2 indexer + sparse attention decode step; gqa: GLM-4.5 "
                          "paged GQA decode (batch 64, 96/8 heads, contexts U[4096, 32768]); select_experts: GLM-4.5 "
@@ -72,9 +80,10 @@ def parse():
     return ap.parse_args()
 
 
-def make_workload(torch, dev, b, ctx, s1, nbuf, seed=0, ctx_min=0):
+def make_workload(torch, dev, b, ctx, s1, nbuf, seed=0, ctx_min=0, idx_scale_dtype=None):
     g = torch.Generator(device=dev).manual_seed(seed)
     bs = 128
+    sdt = idx_scale_dtype or torch.float16  # fp16: the reference operator's signature; fp32: --fp32-scales
     pages_per_seq = (ctx + bs - 1) // bs
     n_pages = b * pages_per_seq
     n_rows = n_pages * bs
@@ -84,7 +93,7 @@ def make_workload(torch, dev, b, ctx, s1, nbuf, seed=0, ctx_min=0):
     for _ in range(nbuf):
         sets.append({
             "idx_k": torch.randint(-127, 128, (n_pages, bs, 1, 128), generator=g, device=dev, dtype=torch.int8),
-            "idx_ks": (0.005 + 0.015 * torch.rand((n_pages, bs, 1), generator=g, device=dev)).to(torch.float16),
+            "idx_ks": (0.005 + 0.015 * torch.rand((n_pages, bs, 1), generator=g, device=dev)).to(sdt),
             "kn": torch.randint(-127, 128, (n_rows, 512), generator=g, device=dev, dtype=torch.int8),
             "kr": torch.randn((n_rows, 64), generator=g, device=dev).to(torch.bfloat16),
             "ks": (0.005 + 0.015 * torch.rand((n_rows, 4), generator=g, device=dev)).float(),
@@ -92,7 +101,7 @@ def make_workload(torch, dev, b, ctx, s1, nbuf, seed=0, ctx_min=0):
     w = {
         "b": b, "s1": s1, "ctx": ctx, "bs": bs, "pages_per_seq": pages_per_seq, "table": table, "sets": sets,
         "idx_q": torch.randint(-127, 128, (t, 64, 128), generator=g, device=dev, dtype=torch.int8),
-        "idx_qs": (0.005 + 0.015 * torch.rand((t, 64), generator=g, device=dev)).to(torch.float16),
+        "idx_qs": (0.005 + 0.015 * torch.rand((t, 64), generator=g, device=dev)).to(sdt),
         "idx_w": (torch.randn((t, 64), generator=g, device=dev) / 8).to(torch.float16),
         "q_nope": torch.randn((t * 128, 512), generator=g, device=dev).to(torch.bfloat16),
         "q_rope": torch.randn((t * 128, 64), generator=g, device=dev).to(torch.bfloat16),
@@ -215,7 +224,7 @@ def bench_gqa(args, torch, lib, dev):
         "config": {"workload": f"paged GQA decode attention, batch {b}, {nq}/{nkv} heads x {d}, bf16 KV, block {bs}, "
                                f"{tokens} cached tokens in total"},
         "roofline": {"kernel": "gqa_decode_kernel", "bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS,
-                     "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": GQA_TRAFFIC_BYTES,
+                     "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": profile_traffic("bench_gqa_b64_hbm_traffic.txt").get("gqa_decode_kernel"),
                      "traffic_unit": "bytes per launch (rocprofv3 FETCH_SIZE + WRITE_SIZE, calibrated)",
                      "work_per_launch": work, "us_per_launch": round(us, 2)},
         "kernels": [{"kernel": n, "us": round(u, 2)} for n, u in kernels.items()], "cpu_baseline": None,
@@ -554,7 +563,7 @@ def bench_paged_gather(args, torch, lib, dev):
                                f"pages of {bs}, rows of {hidden} bytes"},
         "roofline": {"kernel": "paged_gather_kernel", "bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS,
                      "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4),
-                     "traffic": PAGED_GATHER_TRAFFIC_BYTES if (b, args.ctx) == (32, 65536) else None,
+                     "traffic": profile_traffic("bench_paged_gather_b32_k2048_hbm_traffic.txt").get("paged_gather_kernel") if (b, args.ctx) == (32, 65536) else None,
                      "traffic_unit": "bytes per launch (rocprofv3 FETCH_SIZE + WRITE_SIZE, calibrated)",
                      "work_per_launch": work, "us_per_launch": round(us, 2)},
         "kernels": [{"kernel": n, "us": round(u, 2)} for n, u in kernels.items()], "cpu_baseline": cpu,
@@ -661,7 +670,9 @@ def main():
     b, ctx, s1 = args.batch, args.ctx, args.s1
     scale = 192 ** -0.5
     nbuf = 3
-    w = make_workload(torch, dev, b, ctx, s1, nbuf, ctx_min=args.ctx_min)
+    w = make_workload(torch, dev, b, ctx, s1, nbuf, ctx_min=args.ctx_min,
+                      idx_scale_dtype=torch.float32 if args.fp32_scales else None)
+    ks_bytes = 4 if args.fp32_scales else 2
     lengths = w["act"].tolist()
     if args.packed:
         for s in w["sets"]:
@@ -746,7 +757,7 @@ def main():
 
     t = b * s1
     # algorithmic traffic / work per launch, summed over the sequences' lengths
-    score_bytes = sum(L * 128 + L * 2 + (L + 127) // 128 * 4 for L in lengths) + t * (64 * 128 + 64 * 2 + 64 * 2)
+    score_bytes = sum(L * 128 + L * ks_bytes + (L + 127) // 128 * 4 for L in lengths) + t * (64 * 128 + 64 * ks_bytes + 64 * 2)
     topk_bytes = t * 2048 * 4
     curs = [min(max(L - s1 + 1 + i, 0), 2048) for L in lengths for i in range(s1)]
     sfa_bytes = sum(cur * 656 for cur in curs) + t * (128 * 576 * 2 + 128 * 512 * 2 + 2048 * 4)
@@ -773,7 +784,7 @@ def main():
     default_workload = (b, ctx, s1, args.packed, args.ctx_min) == (32, 65536, 1, False, 0)
     roofline = {"kernel": dom["kernel"], "bound": dom["bound"], "achieved": dom["achieved"], "peak": dom["peak"],
                 "unit": dom["unit"], "frac": dom["frac"],
-                "traffic": MEASURED_TRAFFIC_BYTES.get(dom["kernel"]) if default_workload else None,
+                "traffic": profile_traffic("bench_b32_ctx64k_hbm_traffic.txt").get(dom["kernel"]) if default_workload else None,
                 "traffic_unit": "bytes per launch (rocprofv3 FETCH_SIZE + WRITE_SIZE, calibrated)",
                 "work_per_launch": info[dom["kernel"]]["work"], "us_per_launch": dom["us"]}
     sfa_row = next((r for r in per_kernel if r["kernel"] == "sfa_decode_kernel"), None)

@@ -123,13 +123,16 @@ int pto_sfa_antiquant_launch(const PtoTensorDesc* tensors, uint32_t n_tensors, c
  * lightning_indexer_decode (models/deepseek_v32_exp/lightning_indexer_quant_impl.py:226-238).
  * tensors[8], in order:
  *   0 idx_query       [t, 64, 128]            INT8
- *   1 idx_query_scale [t, 64]                 FP16
+ *   1 idx_query_scale [t, 64]                 FP16 (FP32: see below)
  *   2 idx_key_cache   [blocks, block_size, 1, 128] INT8
- *   3 idx_key_scale   [blocks, block_size, 1] FP16
+ *   3 idx_key_scale   [blocks, block_size, 1] FP16 (FP32: see below)
  *   4 idx_weight      [t, 64]                 FP16
  *   5 act_seq_key     [b]                     INT32
  *   6 block_table     [b, max_blocks]         INT32
  *   7 topk_res        [t, 1, selected_count]  INT32 (output; -1 beyond a token's valid length)
+ * The reference's operator takes fp16 scales.  Both scale tensors may instead be FP32 (per-token scales kept in fp32):
+ * then the per-head factor is fp16(idx_query_scale * fp32(idx_weight)) - the golden's fp16 rounding point, taken from the
+ * fp32 product - and idx_key_scale enters the final fp32 product unrounded; one FP16 and one FP32 scale tensor is an error.
  */
 uint64_t pto_lightning_indexer_workspace(const PtoTensorDesc* tensors, uint32_t n_tensors,
                                          const PtoIndexerParams* params);

@@ -9,6 +9,11 @@ its data generators (same file, :46-175).  Arithmetic the golden fixes:
   score[n]     = ( sum_h fp32(w_scale[h]) * fp32(y[h, n]) ) * fp32(k_scale[n])     fp32 (:238-241)
   top-k        = torch.topk over score[:eff_seq], eff_seq = act - (s1 - 1 - i); -1 fills unused slots (:244-261)
 
+fp32-scale variant (the benchmark's configuration with fp32 per-token scales; the reference's operator takes fp16):
+q_scale and k_scale may be fp32 tensors.  Then w_scale[h] = fp16(fp32(q_scale[h] * fp32(weight[h]))) and k_scale
+enters the last product as it is; everything else is unchanged.  With fp32 scales that hold fp16 values the two
+variants give the same bits.
+
 Every product in the head sum is exact in fp32 (11-bit x 11-bit significands);
 only the order of the 64 fp32 additions is left to the BLAS that torch calls,
 so scores are defined up to fp32 summation order.  ``scores_exact`` gives the
@@ -27,7 +32,13 @@ SCORE_SHIFT = 1.0 / 2048.0
 
 
 def w_scale_of(q_scale, weights):
-    """[t,nh] fp16 x [t,nh] fp16 -> fp16 product (one rounding)."""
+    """[t,nh] fp16 x [t,nh] fp16 -> fp16 product (one rounding).
+
+    fp32-scale variant (not in the reference, whose operator takes fp16 scales only): an fp32 q_scale is multiplied
+    with the fp16 weight in fp32 and the product is rounded to fp16 - the golden's rounding point, reached from the
+    fp32 product instead of the exact one (two roundings where the 35-bit product does not fit fp32's 24 bits)."""
+    if q_scale.dtype == torch.float32:
+        return (q_scale * weights.to(torch.float32)).to(torch.float16)
     return (q_scale.to(torch.float16) * weights.to(torch.float16)).to(torch.float16)
 
 
@@ -99,10 +110,11 @@ def scatter_to_cache(k_bsd, block_table, n_blocks, block_size):
 
 
 def make_case(b, s1, act_seq, nh=64, d=128, block_size=128, selected_count=2048, seed=0, dist="bench",
-              spare_pages=0):
+              spare_pages=0, scale_dtype=torch.float16):
     """Synthetic indexer inputs with the reference's tensor signature.
 
-    dist="bench":  q/k int8 U{-127..127}, scales fp16 ~U(0.005,0.02), weights fp16 ~N(0,1)/8.
+    dist="bench":  q/k int8 U{-127..127}, scales ~U(0.005,0.02) in scale_dtype (fp16: the reference's operator;
+                   fp32: the benchmark's configuration as written), weights fp16 ~N(0,1)/8.
     dist="driver": the reference driver's recipe - randn cast to int8, scale = absmax/127
                    in fp16 (floored at 1e-3), requantised; weights fp16 ~N(0,1).
     """
@@ -114,8 +126,8 @@ def make_case(b, s1, act_seq, nh=64, d=128, block_size=128, selected_count=2048,
     if dist == "bench":
         query = torch.randint(-127, 128, (t, nh, d), generator=g, dtype=torch.int8)
         key_cache = torch.randint(-127, 128, (n_blocks, block_size, 1, d), generator=g, dtype=torch.int8)
-        q_scale = (0.005 + 0.015 * torch.rand((t, nh), generator=g)).to(torch.float16)
-        k_scale = (0.005 + 0.015 * torch.rand((n_blocks, block_size, 1), generator=g)).to(torch.float16)
+        q_scale = (0.005 + 0.015 * torch.rand((t, nh), generator=g)).to(scale_dtype)
+        k_scale = (0.005 + 0.015 * torch.rand((n_blocks, block_size, 1), generator=g)).to(scale_dtype)
         weights = (torch.randn((t, nh), generator=g) / 8).to(torch.float16)
     else:
         s2 = max(act)

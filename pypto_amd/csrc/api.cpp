@@ -214,9 +214,12 @@ int plan_indexer(const PtoTensorDesc* ts, uint32_t n, const PtoIndexerParams* p,
     if (p == nullptr) return fail(PTO_ERR_PARAM, "%s: params is null", op);
     int rc;
     if ((rc = check_tensor(op, ts[0], "idx_query", PTO_DT_INT8, 3))) return rc;
-    if ((rc = check_tensor(op, ts[1], "idx_query_scale", PTO_DT_FP16, 2))) return rc;
+    // the scales are fp16 (the reference's signature) or both fp32 (per-token scales kept in fp32)
+    const bool scales_f32 = ts[1].dataType == PTO_DT_FP32;
+    const int scale_dt = scales_f32 ? PTO_DT_FP32 : PTO_DT_FP16;
+    if ((rc = check_tensor(op, ts[1], "idx_query_scale", scale_dt, 2))) return rc;
     if ((rc = check_tensor(op, ts[2], "idx_key_cache", PTO_DT_INT8, 4))) return rc;
-    if ((rc = check_tensor(op, ts[3], "idx_key_scale", PTO_DT_FP16, 3))) return rc;
+    if ((rc = check_tensor(op, ts[3], "idx_key_scale", scale_dt, 3))) return rc;
     if ((rc = check_tensor(op, ts[4], "idx_weight", PTO_DT_FP16, 2))) return rc;
     if ((rc = check_tensor(op, ts[5], "act_seq_key", PTO_DT_INT32, 1))) return rc;
     if ((rc = check_tensor(op, ts[6], "block_table", PTO_DT_INT32, 2))) return rc;
@@ -241,9 +244,10 @@ int plan_indexer(const PtoTensorDesc* ts, uint32_t n, const PtoIndexerParams* p,
     if (max_ctx > (1 << 20) || blocks * bs > 0x7fffffff || t > 65535) return fail(PTO_ERR_SHAPE, "%s: problem too large", op);
     pto::IndexerArgs& a = plan->args;
     a.q = static_cast<const int8_t*>(ts[0].addr);
-    a.q_scale = static_cast<const uint16_t*>(ts[1].addr);
+    a.q_scale = ts[1].addr;
+    a.scales_f32 = scales_f32;
     a.k_cache = static_cast<const int8_t*>(ts[2].addr);
-    a.k_scale = static_cast<const uint16_t*>(ts[3].addr);
+    a.k_scale = ts[3].addr;
     a.weights = static_cast<const uint16_t*>(ts[4].addr);
     a.act_seq = static_cast<const int32_t*>(ts[5].addr);
     a.block_table = static_cast<const int32_t*>(ts[6].addr);

@@ -45,6 +45,20 @@ constexpr int SEL_CHUNK = 4096; // scores per workgroup of the select kernel
 constexpr int TIE_CAP = 8192;   // capacity of the per-row tie list
 
 __device__ __forceinline__ float f16_bits_to_f32(uint16_t h) { return (float)__builtin_bit_cast(_Float16, h); }
+// A scale as it lies in memory (fp16 bits, or fp32 in the fp32-scale variant) and as the fp32 factor it stands for.
+template <bool F32> struct ScaleOf { typedef uint16_t raw; static __device__ __forceinline__ float f32(raw v) { return f16_bits_to_f32(v); } };
+template <> struct ScaleOf<true> { typedef float raw; static __device__ __forceinline__ float f32(raw v) { return v; } };
+// w_scale = q_scale * weight rounded once to fp16: the fp16 product of two fp16 values, or - fp32 scales - the fp32
+// product of the scale and the widened weight
+template <bool F32>
+__device__ __forceinline__ _Float16 w_scale_of(const void* q_scale, const uint16_t* weights, int64_t h)
+{
+    const _Float16 w = __builtin_bit_cast(_Float16, weights[h]);
+    if constexpr (F32)
+        return (_Float16)(static_cast<const float*>(q_scale)[h] * (float)w);
+    else
+        return (_Float16)(__builtin_bit_cast(_Float16, static_cast<const uint16_t*>(q_scale)[h]) * w);
+}
 __device__ __forceinline__ uint32_t score_key(float f) { return f32_to_ordered(f + 0.0f); } // -0 -> +0
 // Bin of a score key in the selection histogram, non-decreasing in the key: quarter octaves (sign, exponent, two
 // mantissa bits - the top 11 key bits) of the magnitudes 2^-20 .. 2^12, 128 bins for either sign; smaller and larger
@@ -132,7 +146,7 @@ __device__ __forceinline__ void flush_span_hist(const IndexerArgs& a, const uint
 
 // S1 query tokens of one sequence share every key fragment.
 // POW2: block_size is a power of two (page index by shift instead of an integer division per key).
-template <int S1, bool POW2>
+template <int S1, bool POW2, bool F32>
 __global__ __launch_bounds__(256) void indexer_score_kernel(IndexerArgs a)
 {
     __shared__ __align__(16) uint32_t hist[S1][SBINS];
@@ -164,9 +178,7 @@ __global__ __launch_bounds__(256) void indexer_score_kernel(IndexerArgs a)
 #pragma unroll
             for (int e = 0; e < 8; ++e) {
                 const int64_t h = (int64_t)(row0 + s) * a.nh + 32 * mm + 16 * (e >> 2) + 4 * g + (e & 3);
-                const _Float16 qs = __builtin_bit_cast(_Float16, a.q_scale[h]);
-                const _Float16 w = __builtin_bit_cast(_Float16, a.weights[h]);
-                wa[s][mm][e] = l16 == 0 ? (_Float16)(qs * w) : (_Float16)0.f; // one fp16 rounding
+                wa[s][mm][e] = l16 == 0 ? w_scale_of<F32>(a.q_scale, a.weights, h) : (_Float16)0.f; // one fp16 rounding
             }
     }
     __syncthreads(); // histogram zeroed
@@ -195,13 +207,13 @@ __global__ __launch_bounds__(256) void indexer_score_kernel(IndexerArgs a)
         krow[j] = present[j] ? (int64_t)page[j] * bs + in_page : 0;
     }
     i32x4 kf0[STEPS], kf1[STEPS];
-    uint16_t ksb[STEPS];
+    typename ScaleOf<F32>::raw ksb[STEPS];
 #pragma unroll
     for (int j = 0; j < STEPS; ++j) {
         const int8_t* kp = a.k_cache + krow[j] * D + 16 * g;
         kf0[j] = *reinterpret_cast<const i32x4*>(kp);
         kf1[j] = *reinterpret_cast<const i32x4*>(kp + 64);
-        ksb[j] = a.k_scale[krow[j]];
+        ksb[j] = static_cast<const typename ScaleOf<F32>::raw*>(a.k_scale)[krow[j]];
     }
 #pragma unroll
     for (int j = 0; j < STEPS; ++j) {
@@ -225,7 +237,7 @@ __global__ __launch_bounds__(256) void indexer_score_kernel(IndexerArgs a)
             // row 0 of the result: register 0 of lanes 0..15, one key each
             const int eff = L - (a.s1 - 1 - (sgrp * S1 + s));
             if (ok && g == 0) {
-                const float sc = sum[0] * (present[j] ? f16_bits_to_f32(ksb[j]) : 0.f);
+                const float sc = sum[0] * (present[j] ? ScaleOf<F32>::f32(ksb[j]) : 0.f);
                 a.scores[(int64_t)(row0 + s) * a.score_stride + tok] = sc;
                 if (tok < eff) atomicAdd(&hist[s][score_bin(score_key(sc))], 1u);
             }
@@ -262,7 +274,7 @@ __device__ __forceinline__ uint32_t relu_scale_pack(int a, int b)
 constexpr int PPASSES = 4; // passes (of 512 keys) per workgroup of the paged kernel
 constexpr int SPAN = CHUNK * PPASSES; // keys per workgroup of either score kernel: one histogram slot
 static_assert(SPAN == CHUNK * PASSES, "both score kernels own spans of the same size");
-template <int S1>
+template <int S1, bool F32>
 __global__ __launch_bounds__(256, S1 == 1 ? 3 : 2) void indexer_score_paged_kernel(IndexerArgs a)
 {
     constexpr int NBUF = 2; // half-pass buffers: NBUF-1 halves ahead (deeper prefetch measured no faster)
@@ -339,7 +351,7 @@ __global__ __launch_bounds__(256, S1 == 1 ? 3 : 2) void indexer_score_paged_kern
     };
 
     i32x4 kf[NBUF][4][2];
-    uint16_t ksc[NBUF][2]; // [buffer][unused for odd halves]: the scales of a pass travel with its first half
+    typename ScaleOf<F32>::raw ksc[NBUF][2]; // [buffer][unused for odd halves]: the scales of a pass travel with its first half
     auto load_half = [&](int hh, int buf) {
         const int64_t r = pass_row(hh >> 1);
         const int64_t rb = r < 0 ? 0 : r;
@@ -349,7 +361,7 @@ __global__ __launch_bounds__(256, S1 == 1 ? 3 : 2) void indexer_score_paged_kern
             kf[buf][jj][0] = *reinterpret_cast<const i32x4*>(kp + jj * 16 * D);
             kf[buf][jj][1] = *reinterpret_cast<const i32x4*>(kp + jj * 16 * D + 64);
         }
-        ksc[buf][0] = a.k_scale[rb + 64 * (hh & 1) + lane];
+        ksc[buf][0] = static_cast<const typename ScaleOf<F32>::raw*>(a.k_scale)[rb + 64 * (hh & 1) + lane];
     };
     // The key loads go out first; the query and its scales follow them (memory operations complete in order, and the
     // first MFMA needs all of them).  Every memory operation from here on is unconditional, so that the number in
@@ -376,9 +388,20 @@ __global__ __launch_bounds__(256, S1 == 1 ? 3 : 2) void indexer_score_paged_kern
         for (int mm = 0; mm < 2; ++mm) {
             typedef _Float16 f16x4 __attribute__((ext_vector_type(4)));
             const int64_t h = (int64_t)(row0 + s) * a.nh + 32 * mm + 4 * g;
-            const f16x4 qlo = *reinterpret_cast<const f16x4*>(a.q_scale + h), qhi = *reinterpret_cast<const f16x4*>(a.q_scale + h + 16);
             const f16x4 wlo = *reinterpret_cast<const f16x4*>(a.weights + h), whi = *reinterpret_cast<const f16x4*>(a.weights + h + 16);
-            wa[s][mm] = __builtin_shufflevector(qlo * wlo, qhi * whi, 0, 1, 2, 3, 4, 5, 6, 7);
+            if constexpr (F32) {
+                const f32x4 qlo = *reinterpret_cast<const f32x4*>(static_cast<const float*>(a.q_scale) + h);
+                const f32x4 qhi = *reinterpret_cast<const f32x4*>(static_cast<const float*>(a.q_scale) + h + 16);
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    wa[s][mm][e] = (_Float16)(qlo[e] * (float)wlo[e]);
+                    wa[s][mm][4 + e] = (_Float16)(qhi[e] * (float)whi[e]);
+                }
+            } else {
+                const uint16_t* qs = static_cast<const uint16_t*>(a.q_scale);
+                const f16x4 qlo = *reinterpret_cast<const f16x4*>(qs + h), qhi = *reinterpret_cast<const f16x4*>(qs + h + 16);
+                wa[s][mm] = __builtin_shufflevector(qlo * wlo, qhi * whi, 0, 1, 2, 3, 4, 5, 6, 7);
+            }
         }
     for (int i = tid; i < S1 * SBINS; i += 256) (&hist[0][0])[i] = 0;
     __syncthreads();
@@ -407,7 +430,7 @@ __global__ __launch_bounds__(256, S1 == 1 ? 3 : 2) void indexer_score_paged_kern
             }
         }
         const int tok = wtok + (hh >> 1) * CHUNK + 64 * (hh & 1) + lane;
-        const float ks = pass_row(hh >> 1) >= 0 ? f16_bits_to_f32(ksc[buf][0]) : 0.f;
+        const float ks = pass_row(hh >> 1) >= 0 ? ScaleOf<F32>::f32(ksc[buf][0]) : 0.f;
 #pragma unroll
         for (int s = 0; s < S1; ++s) {
             const float sc = res[s] * ks;
@@ -935,17 +958,17 @@ hipError_t indexer_launch(const IndexerArgs& a, hipStream_t stream)
     {
         ScopedKernelTimer tm(KID_INDEXER_SCORE, stream);
         const bool pow2 = (a.block_size & (a.block_size - 1)) == 0;
+        const bool s2 = a.s1 % 2 == 0, f32 = a.scales_f32;
         if (a.block_size % 128 == 0) {
-            if (a.s1 % 2 == 0)
-                hipLaunchKernelGGL(indexer_score_paged_kernel<2>, dim3(pchunks, a.b, a.s1 / 2), dim3(256), 0, stream, args);
-            else
-                hipLaunchKernelGGL(indexer_score_paged_kernel<1>, dim3(pchunks, a.b, a.s1), dim3(256), 0, stream, args);
-        } else if (a.s1 % 2 == 0) {
-            auto kern = pow2 ? indexer_score_kernel<2, true> : indexer_score_kernel<2, false>;
-            hipLaunchKernelGGL(kern, dim3(chunks, a.b, a.s1 / 2), dim3(256), 0, stream, args);
+            auto kern = s2 ? (f32 ? indexer_score_paged_kernel<2, true> : indexer_score_paged_kernel<2, false>)
+                           : (f32 ? indexer_score_paged_kernel<1, true> : indexer_score_paged_kernel<1, false>);
+            hipLaunchKernelGGL(kern, dim3(pchunks, a.b, s2 ? a.s1 / 2 : a.s1), dim3(256), 0, stream, args);
         } else {
-            auto kern = pow2 ? indexer_score_kernel<1, true> : indexer_score_kernel<1, false>;
-            hipLaunchKernelGGL(kern, dim3(chunks, a.b, a.s1), dim3(256), 0, stream, args);
+            auto kern = s2 ? (pow2 ? (f32 ? indexer_score_kernel<2, true, true> : indexer_score_kernel<2, true, false>)
+                                   : (f32 ? indexer_score_kernel<2, false, true> : indexer_score_kernel<2, false, false>))
+                           : (pow2 ? (f32 ? indexer_score_kernel<1, true, true> : indexer_score_kernel<1, true, false>)
+                                   : (f32 ? indexer_score_kernel<1, false, true> : indexer_score_kernel<1, false, false>));
+            hipLaunchKernelGGL(kern, dim3(chunks, a.b, s2 ? a.s1 / 2 : a.s1), dim3(256), 0, stream, args);
         }
     }
     hipError_t e = hipGetLastError();

@@ -40,9 +40,9 @@ hipError_t sfa_static_scratch(void** ptr);
 // ---------------------------------------------------------------- lightning indexer
 struct IndexerArgs {
     const int8_t* q;             // [t, nh, 128]
-    const uint16_t* q_scale;     // [t, nh] fp16
+    const void* q_scale;         // [t, nh] fp16, or fp32 when scales_f32
     const int8_t* k_cache;       // [blocks*bs, 128]
-    const uint16_t* k_scale;     // [blocks*bs] fp16
+    const void* k_scale;         // [blocks*bs] fp16, or fp32 when scales_f32
     const uint16_t* weights;     // [t, nh] fp16
     const int32_t* act_seq;      // [b]
     const int32_t* block_table;  // [b, bt_stride]
@@ -55,6 +55,7 @@ struct IndexerArgs {
     int64_t n_blocks;
     int32_t b, s1, nh, block_size, bt_stride, k, score_stride;
     int32_t max_ctx; // set by indexer_launch: bt_stride * block_size, the longest sequence the page table can address
+    bool scales_f32; // q_scale and k_scale are fp32: w_scale = fp16(q_scale * fp32(weight)), k_scale enters the score as it is
     int32_t pchunks; // set by indexer_bind_workspace: histogram slots (2048-key spans) per query token = score_stride / 2048
 };
 

@@ -25,6 +25,8 @@ class LightningIndexerConfigs:
 def lightning_indexer_decode(idx_query, idx_query_scale, idx_key_cache, idx_key_scale, idx_weight, act_seq_key,
                              block_table, topk_res, unroll_list, configs, selected_count):
     """topk_res[t, 1, selected_count] <- indices of the selected_count best-scoring cached tokens of each
-    query token (best first, -1 beyond the token's valid length)."""
+    query token (best first, -1 beyond the token's valid length).  The scales are fp16 as in the reference, or both
+    fp32 (per-token scales kept in fp32; then the per-head factor is fp16(idx_query_scale * fp32(idx_weight)) and
+    idx_key_scale multiplies the head sum unrounded)."""
     launch("lightning_indexer", [idx_query, idx_query_scale, idx_key_cache, idx_key_scale, idx_weight, act_seq_key,
                                  block_table, topk_res], IndexerParams(int(selected_count)))

@@ -60,6 +60,18 @@ def test_small_edge_lengths(cuda):
     check_topk(case, run_indexer(case, cuda))
 
 
+def test_fp32_scales(cuda):
+    """Benchmark configuration 3 as written - fp32 per-token scales - through the same entry point: both score kernels
+    (128-token pages and a page size that is not a multiple of 128), one and two query tokens per sequence."""
+    for b, s1, act, bs, seed in ((3, 1, [9000, 2049, 300], 128, 61), (2, 2, [5000, 77], 128, 62), (2, 1, [3000, 500], 48, 63)):
+        case = oi.make_case(b, s1, act, block_size=bs, seed=seed, scale_dtype=torch.float32)
+        check_topk(case, run_indexer(case, cuda))
+    # one fp16 and one fp32 scale tensor is neither form
+    from pypto_amd.error import FeError
+    with pytest.raises(FeError, match="idx_key_scale"):
+        run_indexer(dict(case, k_scale=case["k_scale"].half()), cuda)
+
+
 def test_mtp_two_query_tokens(cuda):
     case = oi.make_case(4, 2, [5000, 971, 2049, 300], seed=4, dist="driver")
     check_topk(case, run_indexer(case, cuda))

@@ -100,3 +100,30 @@ def test_driver_style_case_respects_quantisation_ranges():
                                c["block_table"], 2, 2048)
     assert out.shape == (4, 1, 2048) and (out[0, 0, 299:] == -1).all() and (out[1, 0, 300:] == -1).all()
     assert sorted(out[1, 0, :300].tolist()) == list(range(300))
+
+
+def test_fp32_scale_variant():
+    """The fp32-scale variant (scales kept in fp32; not in the reference, whose operator takes fp16): with fp32 tensors
+    that hold fp16 values it gives the bits of the fp16 form (every product it forms is then the same number); with
+    general fp32 scales w_scale is the fp32 product rounded to fp16 by hand, and the score follows the formula in
+    float64 to fp32 accuracy."""
+    case = oi.make_case(2, 2, [300, 77], seed=9)
+    args = lambda c: (c["query"], c["q_scale"], c["key_cache"], c["k_scale"], c["weights"], c["act_seq"], c["block_table"], c["s1"])  # noqa: E731
+    as32 = dict(case, q_scale=case["q_scale"].float(), k_scale=case["k_scale"].float())
+    assert torch.equal(oi.scores(*args(as32)), oi.scores(*args(case)))
+    c32 = oi.make_case(2, 2, [300, 77], seed=9, scale_dtype=torch.float32)
+    assert c32["q_scale"].dtype == torch.float32 and not torch.equal(c32["q_scale"], c32["q_scale"].half().float())
+    ws = oi.w_scale_of(c32["q_scale"], c32["weights"])
+    prod32 = (c32["q_scale"].double() * c32["weights"].double()).float()   # the fp32 product (one rounding of the exact one)
+    assert torch.equal(ws.double(), torch.from_numpy(f16_rne(prod32.double().numpy())))
+    # the formula end to end in float64 from the same w_scale, page by page through the table
+    sc = oi.scores(*args(c32))
+    t, nh, d = c32["query"].shape
+    for r in range(t):
+        bi = r // 2
+        for tok in (0, 1, min(130, c32["act_seq"][bi] - 1), c32["act_seq"][bi] - 1):
+            page, off = int(c32["block_table"][bi, tok // 128]), tok % 128
+            dot = (c32["query"][r].long() @ c32["key_cache"][page, off, 0].long()).clamp(min=0)
+            y = torch.from_numpy(f16_rne((dot.double() / 2048).numpy()))
+            want = float((ws[r].double() * y).sum() * c32["k_scale"][page, off, 0].double())
+            assert abs(float(sc[r, tok]) - want) <= 1e-5 * max(abs(want), 1e-6)
