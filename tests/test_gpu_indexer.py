@@ -72,6 +72,25 @@ def test_fp32_scales(cuda):
         run_indexer(dict(case, k_scale=case["k_scale"].half()), cuda)
 
 
+def test_scores_outside_the_histogram_range(cuda):
+    """The selection histogram resolves magnitudes 2^-20 .. 2^12; smaller and larger scores share the first and last bin
+    of their sign, whose keys do not share a bit prefix.  fp32 scales put whole rows out of range: tiny scores (the
+    threshold bin is a first bin - once with a tie list that fits LDS, once with one that overflows into the pass over
+    the whole row), huge scores (a last bin), and a mix of tiny, ordinary and huge ones in one row."""
+    for act, qmul, kmul, seed in (([5000, 2300], 1e-5, 1e-5, 71), ([40000], 1e-5, 1e-5, 72), ([9000, 4000], 1e3, 1e3, 73)):
+        case = oi.make_case(len(act), 1, act, seed=seed, scale_dtype=torch.float32)
+        case["q_scale"] = case["q_scale"] * qmul
+        case["k_scale"] = case["k_scale"] * kmul
+        sc = indexer_scores(case, exact=True)
+        big = sc.abs().max()
+        assert (big < 2.0 ** -20) if qmul < 1 else (big > 2.0 ** 12)
+        check_topk(case, run_indexer(case, cuda))
+    case = oi.make_case(2, 2, [7000, 3000], seed=74, scale_dtype=torch.float32)
+    g = torch.Generator().manual_seed(74)
+    case["k_scale"] = case["k_scale"] * torch.tensor([1e-9, 1.0, 1e7])[torch.randint(0, 3, case["k_scale"].shape, generator=g)]
+    check_topk(case, run_indexer(case, cuda))
+
+
 def test_mtp_two_query_tokens(cuda):
     case = oi.make_case(4, 2, [5000, 971, 2049, 300], seed=4, dist="driver")
     check_topk(case, run_indexer(case, cuda))
