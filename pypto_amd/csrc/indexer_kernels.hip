@@ -48,6 +48,15 @@ __device__ __forceinline__ float f16_bits_to_f32(uint16_t h) { return (float)__b
 // A scale as it lies in memory (fp16 bits, or fp32 in the fp32-scale variant) and as the fp32 factor it stands for.
 template <bool F32> struct ScaleOf { typedef uint16_t raw; static __device__ __forceinline__ float f32(raw v) { return f16_bits_to_f32(v); } };
 template <> struct ScaleOf<true> { typedef float raw; static __device__ __forceinline__ float f32(raw v) { return v; } };
+// fp16(fp32(a * b)): the product is rounded to fp32 first and that value to fp16, as the golden's tensor operations do.
+// (The compiler would otherwise fuse the multiplication and the conversion into one mixed-precision instruction that
+// rounds the exact product once - a different fp16 value about once in 8000 products.)
+__device__ __forceinline__ _Float16 round_f32_product_to_f16(float a, float b)
+{
+    float p = a * b;
+    asm volatile("" : "+v"(p));
+    return (_Float16)p;
+}
 // w_scale = q_scale * weight rounded once to fp16: the fp16 product of two fp16 values, or - fp32 scales - the fp32
 // product of the scale and the widened weight
 template <bool F32>
@@ -55,7 +64,7 @@ __device__ __forceinline__ _Float16 w_scale_of(const void* q_scale, const uint16
 {
     const _Float16 w = __builtin_bit_cast(_Float16, weights[h]);
     if constexpr (F32)
-        return (_Float16)(static_cast<const float*>(q_scale)[h] * (float)w);
+        return round_f32_product_to_f16(static_cast<const float*>(q_scale)[h], (float)w);
     else
         return (_Float16)(__builtin_bit_cast(_Float16, static_cast<const uint16_t*>(q_scale)[h]) * w);
 }
@@ -394,8 +403,8 @@ __global__ __launch_bounds__(256, S1 == 1 ? 3 : 2) void indexer_score_paged_kern
                 const f32x4 qhi = *reinterpret_cast<const f32x4*>(static_cast<const float*>(a.q_scale) + h + 16);
 #pragma unroll
                 for (int e = 0; e < 4; ++e) {
-                    wa[s][mm][e] = (_Float16)(qlo[e] * (float)wlo[e]);
-                    wa[s][mm][4 + e] = (_Float16)(qhi[e] * (float)whi[e]);
+                    wa[s][mm][e] = round_f32_product_to_f16(qlo[e], (float)wlo[e]);
+                    wa[s][mm][4 + e] = round_f32_product_to_f16(qhi[e], (float)whi[e]);
                 }
             } else {
                 const uint16_t* qs = static_cast<const uint16_t*>(a.q_scale);

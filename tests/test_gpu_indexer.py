@@ -72,6 +72,26 @@ def test_fp32_scales(cuda):
         run_indexer(dict(case, k_scale=case["k_scale"].half()), cuda)
 
 
+def test_fp32_scale_products_round_twice_like_the_golden(cuda):
+    """fp16(fp32(scale * weight)) rounds twice; a fused multiply-convert would round the exact product once and land on
+    another fp16 value about once in 8000 products.  Every (token, head) here is such a pair (found by search), so a
+    kernel that rounds once gets every per-head factor wrong by an ulp and fails the ordering check."""
+    g = torch.Generator().manual_seed(81)
+    a = (0.005 + 0.015 * torch.rand(8000000, generator=g)).float()
+    w = (torch.randn(8000000, generator=g) / 8).half()
+    twice = (a * w.float()).half()
+    # (numpy rounds float64 to float16 in one step; torch goes through float32)
+    once = torch.from_numpy((a.double().numpy() * w.double().numpy()).astype("float16"))
+    hit = (twice != once).nonzero().flatten()
+    assert hit.numel() >= 4 * 64
+    for bs in (128, 48):
+        case = oi.make_case(2, 2, [3000, 500], block_size=bs, seed=82, scale_dtype=torch.float32)
+        case["q_scale"] = a[hit[:256]].reshape(4, 64).clone()
+        case["weights"] = w[hit[:256]].reshape(4, 64).clone()
+        assert not torch.equal(oi.w_scale_of(case["q_scale"], case["weights"]), once[hit[:256]].reshape(4, 64))
+        check_topk(case, run_indexer(case, cuda))
+
+
 def test_scores_outside_the_histogram_range(cuda):
     """The selection histogram resolves magnitudes 2^-20 .. 2^12; smaller and larger scores share the first and last bin
     of their sign, whose keys do not share a bit prefix.  fp32 scales put whole rows out of range: tiny scores (the
