@@ -64,9 +64,11 @@ def install_guards(monkeypatch):
                 t.copy_(view)
         log.append((op, int(n)))
 
+    # (the operator modules first: one imported while _runtime.launch is swapped would bind the swapped function for good)
+    modules = [importlib.import_module(name) for name in MODULES]
     monkeypatch.setattr(_runtime, "launch", launch)
-    for name in MODULES:
-        monkeypatch.setattr(importlib.import_module(name), "launch", launch)
+    for m in modules:
+        monkeypatch.setattr(m, "launch", launch)
     return log
 
 
