@@ -19,14 +19,18 @@ def cur_seq_of(act, s1, j):
     return max(int(act) - (s1 - 1 - j), 0)
 
 
-def attention_flash(q, k_cache, v_cache, block_table, act_seqs, softmax_scale):
-    """q [t, nq, d] bf16; k_cache / v_cache [blocks, bs, nkv, d] bf16 -> [t, nq, d] bf16 (zeros where nothing is attended)."""
+def attention_flash(q, k_cache, v_cache, block_table, act_seqs, softmax_scale, tile=None):
+    """q [t, nq, d] bf16; k_cache / v_cache [blocks, bs, nkv, d] bf16 -> [t, nq, d] bf16 (zeros where nothing is attended).
+    ``tile``: tokens per tile; None is the reference's choice, one tile per cache page.  (Another tile size is the same
+    algorithm with its roundings of P~ taken relative to other maxima: tests use it as a yardstick of what the
+    algorithm's accuracy is when the tile is not the page.)"""
     t, nq, d = q.shape
     _, bs, nkv, _ = k_cache.shape
     b = len(act_seqs)
     s1 = t // b
     g = nq // nkv
     out = torch.zeros_like(q)
+    step = bs if tile is None else int(tile)
     for bi in range(b):
         for j in range(s1):
             cur = cur_seq_of(act_seqs[bi], s1, j)
@@ -34,11 +38,17 @@ def attention_flash(q, k_cache, v_cache, block_table, act_seqs, softmax_scale):
                 continue
             qi = q[bi * s1 + j].view(nkv, g, d).float()
             m = l = o = None
-            for p in range(math.ceil(cur / bs)):
-                blk = int(block_table[bi, p])
-                n = min(bs, cur - p * bs)
-                kj = k_cache[blk, :n].permute(1, 0, 2).float()                       # [nkv, n, d]
-                vj = v_cache[blk, :n].permute(1, 0, 2).float()
+            for p in range(math.ceil(cur / step)):
+                n = min(step, cur - p * step)
+                if tile is None:
+                    blk = int(block_table[bi, p])
+                    kj = k_cache[blk, :n].permute(1, 0, 2).float()                   # [nkv, n, d]
+                    vj = v_cache[blk, :n].permute(1, 0, 2).float()
+                else:
+                    pos = torch.arange(p * step, p * step + n)
+                    rows = block_table[bi, pos // bs].long() * bs + pos % bs
+                    kj = k_cache.reshape(-1, nkv, d)[rows].permute(1, 0, 2).float()
+                    vj = v_cache.reshape(-1, nkv, d)[rows].permute(1, 0, 2).float()
                 s = torch.matmul(qi, kj.transpose(1, 2)) * softmax_scale              # :1436-1437
                 mt = s.max(dim=-1, keepdim=True).values                              # :1438
                 pt = torch.exp(s - mt)                                               # :1439-1440

@@ -129,7 +129,7 @@ def test_topk(cuda, guarded):
 
 
 def test_paged_gather(cuda, guarded):
-    from pypto_amd.experimental import gather_in_ub
+    from pypto_amd.experimental import gather_in_l1, gather_in_ub
     from oracle import paged
     g = torch.Generator().manual_seed(7)
     # row widths that take the 16-, 4-, 2- and 1-byte copy paths, index counts that end inside a 32-row workgroup
@@ -139,8 +139,10 @@ def test_paged_gather(cuda, guarded):
         src = torch.randint(-100, 100, (n, hidden), generator=g).to(dtype)
         page = torch.randperm(nblk, generator=g).to(torch.int32).reshape(1, nblk)
         idx = torch.randint(0, n, (1, k), generator=g, dtype=torch.int32)
-        view = src.to(cuda)[:, :size] if size != hidden else src.to(cuda)
-        out = gather_in_ub(view, idx.to(cuda), page.to(cuda), bs, -2).cpu()
+        if size != hidden:   # the first `size` columns of every row
+            out = gather_in_l1(src.to(cuda), idx.to(cuda), page.to(cuda), bs, size).cpu()
+        else:
+            out = gather_in_ub(src.to(cuda), idx.to(cuda), page.to(cuda), bs, -2).cpu()
         want = paged.paged_gather(src, idx[0], page[0], bs)[:, :size]
         assert torch.equal(out.view(torch.uint8), want.contiguous().view(torch.uint8))
     assert len(guarded) == 4

@@ -37,6 +37,19 @@ def run(case, dev):
             "k_scale_cache": out.k_scale.cpu(), "weights": out.weights.cpu()}
 
 
+WEIGHTS_REL = 2.0 ** -7 + 2.0 ** -11
+
+
+def weights_allowance(case):
+    """What the summation order of x @ w_proj (h fp32 terms) may move a weight by, in the weight's units: a weight is
+    that sum times 1 / sqrt(heads * 128), and where the terms cancel the sum carries an absolute error of a few units in
+    the last place of the terms' magnitudes, whatever the order - 8 * 2^-24 * sum |x_i| |w_i| is a generous bound for
+    the blocked orders of either side.  Both the kernel and the golden sit within it of the exact sum, so twice that."""
+    n = case["w_qb"].shape[1] // case["hadamard_q"].shape[0]
+    mag = case["x"].double().abs() @ case["w_proj"].double().abs()
+    return (2 * 8 * 2.0 ** -24 * mag * (n * case["hadamard_q"].shape[0]) ** -0.5).float()
+
+
 def check(case, got):
     gold = op.indexer_prolog(case)
     rows = case["k_cache_index"]
@@ -46,17 +59,19 @@ def check(case, got):
         assert diff.max() <= 1, f"{name}: off by {int(diff.max())}"
         assert (diff == 0).float().mean() >= 0.98, f"{name}: {(diff != 0).float().mean():.4f} of the values differ"
 
-    def scales(a, b, name, min_equal):
+    def scales(a, b, name, min_equal, atol=1e-8, rel=2.0 ** -7):
         a, b = a.float().flatten(), b.float().flatten()
         assert torch.isfinite(a).all(), name
-        assert ((a - b).abs() <= 2.0 ** -7 * b.abs() + 1e-8).all(), f"{name}: {float(((a - b).abs() / b.abs()).max())}"
+        assert ((a - b).abs() <= rel * b.abs() + atol).all(), f"{name}: {float(((a - b).abs() / b.abs()).max())}"
         assert (a == b).float().mean() >= min_equal, f"{name}: only {(a == b).float().mean():.3f} bit-equal"
 
     ints(got["q_int8"], gold["q_int8"], "q_int8")
     scales(got["q_scale"], gold["q_scale"], "q_scale", 0.90)
     ints(got["k_cache"].view(-1, 128)[rows], gold["k_cache"].view(-1, 128)[rows], "k_int8")
     scales(got["k_scale_cache"].view(-1)[rows], gold["k_scale_cache"].view(-1)[rows], "k_scale", 0.80)
-    scales(got["weights"], gold["weights"], "weights", 0.98)
+    # (a weight is the bf16 rounding of the sum, scaled and rounded to fp16: a sum that rounds the other way moves it by
+    # one bf16 step, 2^-7 of the value at the bottom of a binade, and the two fp16 roundings add half an fp16 step each)
+    scales(got["weights"], gold["weights"], "weights", 0.98, atol=weights_allowance(case).flatten(), rel=WEIGHTS_REL)
     # nothing but the indexed rows of the caches may change
     keep = torch.ones(case["k_cache"].shape[0] * case["k_cache"].shape[1], dtype=torch.bool)
     keep[rows] = False

@@ -14,6 +14,8 @@ import pytest
 import torch
 
 from oracle import mla_prolog as op
+from test_gpu_indexer_prolog import WEIGHTS_REL, weights_allowance
+from test_gpu_mla_prolog import check_rope_cache
 
 pytestmark = pytest.mark.gpu
 EPS = 1e-5
@@ -89,28 +91,34 @@ def check_against_oracle(mla_case, idx_case, got):
             f"{name}: {int((ratio > 1).sum())} values out of tolerance, worst {float(ratio.max())} x"
 
     ints(got["kv_cache"].view(-1, 512)[rows], gm["kv_cache"].view(-1, 512)[rows], "kv_cache", 1, 0.98)
-    close(got["k_scale_cache"].view(-1, 4)[rows], gm["k_scale_cache"].view(-1, 4)[rows], "k_scale_cache")
+    close(got["k_scale_cache"].view(-1, 4)[rows], gm["k_scale_cache"].view(-1, 4)[rows], "k_scale_cache", rel=2.0 ** -6)  # see test_gpu_mla_prolog
     close(got["q_nope"], gm["q_nope"], "q_nope", 0.0078125, 0.005, outliers=1e-3)   # see test_gpu_mla_prolog
     close(got["q_rope"], gm["q_rope"], "q_rope", 0.0078125, 0.005, outliers=1e-3)
-    close(got["kr_cache"].view(-1, 64)[rows], gm["kr_cache"].view(-1, 64)[rows], "kr_cache", 0.0078125, 1e-4)
+    check_rope_cache(mla_case, got["kr_cache"], gm["kr_cache"], EPS)   # see test_gpu_mla_prolog
     ints(got["q_int8"], gi["q_int8"], "q_int8", 2, 0.95)
-    close(got["q_scale"], gi["q_scale"], "q_scale")
+    # (the golden's index queries come from the golden's q_norm, the product's from its own: a q_norm value that rounded
+    # the other way shifts the 128 values of a head a little, on top of the one bf16 step their own rounding can move,
+    # which is why q_int8 gets 2 above; a query scale follows the largest of them, so two bf16 steps here.  The tight
+    # check of this stage is that the fused call gives the bits of the separate calls, whose index prolog is tested
+    # against the oracle from one and the same q_norm.)
+    close(got["q_scale"], gi["q_scale"], "q_scale", rel=2.0 ** -6)
     ints(got["k_cache"].view(-1, 128)[rows], gi["k_cache"].view(-1, 128)[rows], "idx k_int8", 1, 0.98)
     close(got["idx_k_scale_cache"].view(-1)[rows], gi["k_scale_cache"].view(-1)[rows], "idx k_scale")
-    close(got["weights"], gi["weights"], "weights", atol=2e-6)
+    close(got["weights"], gi["weights"], "weights", rel=WEIGHTS_REL, atol=weights_allowance(idx_case).flatten())
 
 
-def same_as_separate(fused, sep):
+def same_as_separate(fused, sep, idx_case):
     for k, v in fused.items():
         if k in ("k_cache", "idx_k_scale_cache", "weights"):
             continue
         assert torch.equal(v, sep[k]), f"{k}: fused and separate calls differ"
     assert (fused["k_cache"].int() - sep["k_cache"].int()).abs().max() <= 1
     assert (fused["k_cache"] == sep["k_cache"]).float().mean() >= 0.999
-    for k in ("idx_k_scale_cache", "weights"):
-        a, b = fused[k].float(), sep[k].float()
-        # weights near zero are sums that cancel: there the summation order shows at the fp32 level of the 7168 terms
-        assert ((a - b).abs() <= 2.0 ** -7 * b.abs() + 2e-6).all(), k
+    a, b = fused["idx_k_scale_cache"].float(), sep["idx_k_scale_cache"].float()
+    assert ((a - b).abs() <= 2.0 ** -7 * b.abs() + 1e-8).all(), "idx_k_scale_cache"
+    # weights near zero are sums that cancel: there the summation order shows at the fp32 level of the h terms
+    a, b = fused["weights"].float(), sep["weights"].float()
+    assert ((a - b).abs() <= WEIGHTS_REL * b.abs() + weights_allowance(idx_case)).all(), "weights"
 
 
 def test_reference_case_b4_s2_fused_equals_separate_and_oracle(cuda):
@@ -118,7 +126,7 @@ def test_reference_case_b4_s2_fused_equals_separate_and_oracle(cuda):
     mla_case, idx_case = op.make_fused_case(4, 2, 1024, seed=21)
     fused = run_fused(mla_case, idx_case, cuda)
     sep = run_separate(mla_case, idx_case, cuda)
-    same_as_separate(fused, sep)
+    same_as_separate(fused, sep, idx_case)
     check_against_oracle(mla_case, idx_case, fused)
 
 
@@ -126,7 +134,7 @@ def test_prefill_entry_ragged_tiles_small_sizes(cuda):
     mla_case, idx_case = op.make_fused_case(37, 1, 300, seed=22, n_idx=64, h=512, q_lora_rank=256, n=4)
     fused = run_fused(mla_case, idx_case, cuda, entry="mla_indexer_prolog_quant_p")
     sep = run_separate(mla_case, idx_case, cuda)
-    same_as_separate(fused, sep)
+    same_as_separate(fused, sep, idx_case)
     check_against_oracle(mla_case, idx_case, fused)
 
 
@@ -138,7 +146,7 @@ def test_prefill_sizes_fused_equals_separate_and_oracle(cuda):
         mla_case, idx_case = op.make_fused_case(b, 1, 300, seed=seed, n_idx=64, h=1280, q_lora_rank=256, n=4)
         fused = run_fused(mla_case, idx_case, cuda, entry="mla_indexer_prolog_quant_p")
         sep = run_separate(mla_case, idx_case, cuda)
-        same_as_separate(fused, sep)
+        same_as_separate(fused, sep, idx_case)
         check_against_oracle(mla_case, idx_case, fused)
 
 

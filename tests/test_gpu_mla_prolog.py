@@ -5,12 +5,18 @@ atol 0.005, the int8 tensors (q_norm, kv_cache) with an absolute tolerance of 1,
 atol 2.5e-5 and the rope cache with rtol 0.0078125 / atol 1e-4.  Every stage here reproduces the operator's rounding
 points; what differs from the oracle is the summation order of the fp32 matmuls and of the RmsNorm sums, which now and
 then moves a value across a bf16 rounding boundary.  So, against the oracle evaluated with the operator's epsilons:
-int8 values within 1 everywhere and equal in at least 98 % of the places; scales within one bf16 step (2^-7 relative)
-and bit-equal in most rows.  A flipped q_norm value moves the 24576 products of its token by up to one int8 step of
+int8 values within 1 everywhere and equal in at least 98 % of the places; scales within two bf16 steps (2^-6
+relative: a scale follows the largest value of its row, which is a bf16 rounding of the product carried through the
+norm's own bf16 rounding - either can fall the other way) and bit-equal in most rows.  A flipped q_norm value moves the 24576 products of its token by up to one int8 step of
 that token, which takes a few of that token's q_nope values out of the tight tolerance - the reference's comparator
 allows 0.5 % of such outliers (utils/compare.py:16, max_error_ratio); here at most 0.1 % of the elements and none
 beyond 3 x the tolerance.  The downstream stages are also checked on their own: from the product's own q_norm /
 q_norm_scale the oracle's q_nope and q_rope must be met with no outlier at all.
+
+The rope cache (check_rope_cache): a rope key is a cos + b sin of two bf16 roundings of x @ w_kr.  A rounding that fell
+the other way moves a (or b) by one bf16 step and the key by that step times |cos| (|sin|); when the two terms cancel
+that is more than 2^-7 of the result.  So: every key within the reference's tolerance plus that move (computed from
+the oracle's own a and b), and at most 0.1 % of them outside the plain tolerance.
 """
 import pytest
 import torch
@@ -19,6 +25,27 @@ from oracle import mla_prolog as op
 
 pytestmark = pytest.mark.gpu
 EPS = 1e-5
+
+
+def bf16_step(v):
+    """Distance between neighbouring bf16 values at |v| (8 significant bits)."""
+    return torch.exp2(torch.floor(torch.log2(v.float().abs().clamp(min=2.0 ** -126))) - 7)
+
+
+def check_rope_cache(case, got_cache, gold_cache, eps=EPS, min_equal=0.95):
+    rows = case["cache_index"]   # (one cache row per token: make_case draws distinct positions)
+    a, b = got_cache.view(-1, 64)[rows].float(), gold_cache.view(-1, 64)[rows].float()
+    assert torch.isfinite(a).all(), "kr_cache"
+    t = a.shape[0]
+    pre = op.intermediates(case, eps, eps)["kv"][:, 512:].float()   # the bf16 products, before the rotary embedding
+    pre = pre.reshape(t, 32, 2).permute(0, 2, 1).reshape(t, 64)      # pairs (2i, 2i+1) -> positions (i, 32+i)
+    move = bf16_step(pre) * case["cos"].float().abs() + bf16_step(op.rotate_half(pre)) * case["sin"].float().abs()
+    tol = 1e-4 + 0.0078125 * b.abs()
+    err = (a - b).abs()
+    worst = float((err / (tol + move)).max())
+    assert worst <= 1, f"kr_cache: {worst} x the tolerance plus one flipped rounding of x @ w_kr"
+    assert (err > tol).float().mean() <= 1e-3, f"kr_cache: {int((err > tol).sum())} of {err.numel()} values outside the plain tolerance"
+    assert (a == b).float().mean() >= min_equal, f"kr_cache: only {(a == b).float().mean():.3f} bit-equal"
 
 
 def run(case, dev, entry="mla_prolog_quant_d", eps=EPS):
@@ -53,7 +80,7 @@ def check(case, got, eps=EPS):
     def scales(a, b, name, min_equal):
         a, b = a.float().flatten(), b.float().flatten()
         assert torch.isfinite(a).all(), name
-        assert ((a - b).abs() <= 2.0 ** -7 * b.abs() + 1e-8).all(), f"{name}: {float(((a - b).abs() / b.abs()).max())}"
+        assert ((a - b).abs() <= 2.0 ** -6 * b.abs() + 1e-8).all(), f"{name}: {float(((a - b).abs() / b.abs()).max())}"
         assert (a == b).float().mean() >= min_equal, f"{name}: only {(a == b).float().mean():.3f} bit-equal"
 
     def floats(a, b, name, rtol, atol, min_equal, outliers=0.0):
@@ -73,7 +100,7 @@ def check(case, got, eps=EPS):
     floats(got["q_rope"], tail_rope, "q_rope from the product's q_norm", 0.0078125, 0.005, 0.99)
     ints(got["kv_cache"].view(-1, 512)[rows], gold["kv_cache"].view(-1, 512)[rows], "kv_cache")
     scales(got["k_scale_cache"].view(-1, 4)[rows], gold["k_scale_cache"].view(-1, 4)[rows], "k_scale_cache", 0.80)
-    floats(got["kr_cache"].view(-1, 64)[rows], gold["kr_cache"].view(-1, 64)[rows], "kr_cache", 0.0078125, 1e-4, 0.95)
+    check_rope_cache(case, got["kr_cache"], gold["kr_cache"], eps)
     # nothing but the indexed rows of the caches may change
     keep = torch.ones(case["kv_cache"].shape[0] * case["kv_cache"].shape[1], dtype=torch.bool)
     keep[rows] = False
@@ -128,8 +155,9 @@ def check_bf16_form(case, got, eps=EPS, outliers=0.0):
     """bf16 form (the reference's tolerances, :686-694: q_norm, kv, kr rtol 2^-7 / atol 1e-4; q_nope, q_rope rtol 2^-7 /
     atol 5e-3): everything within those everywhere, and bit-equal in at least 98 % of the places - the difference is
     the summation order of x @ w, which now and then moves a bf16 rounding.  `outliers`: the fraction of values that may
-    sit up to 1.5 x outside (a flipped rounding of q_a that the norm's own rounding carries to a second bf16 step; the
-    reference's comparator lets 0.5 % of the values be anywhere)."""
+    sit up to 2 x outside (a flipped rounding of the product that the norm's own rounding carries to a second bf16 step:
+    two steps are at most 2^-6 of the value, twice the relative tolerance; the reference's comparator lets 0.5 % of the
+    values be anywhere)."""
     gold = op.mla_prolog(case, eps, eps)
     rows = case["cache_index"]
 
@@ -137,7 +165,7 @@ def check_bf16_form(case, got, eps=EPS, outliers=0.0):
         a, b = a.float(), b.float()
         assert torch.isfinite(a).all(), name
         ratio = (a - b).abs() / (atol + rtol * b.abs())
-        assert (ratio > 1).float().mean() <= outliers and ratio.max() <= (1.5 if outliers else 1), \
+        assert (ratio > 1).float().mean() <= outliers and ratio.max() <= (2 if outliers else 1), \
             f"{name}: worst {float(ratio.max())} x the tolerance, {int((ratio > 1).sum())} values outside"
         assert (a == b).float().mean() >= min_equal, f"{name}: only {(a == b).float().mean():.3f} bit-equal"
 
@@ -157,7 +185,7 @@ def check_bf16_form(case, got, eps=EPS, outliers=0.0):
     floats(got["q_nope"], tail_nope, "q_nope from the product's q_norm", 0.0078125, 0.005, 0.99)
     floats(got["q_rope"], tail_rope, "q_rope from the product's q_norm", 0.0078125, 0.005, 0.99)
     floats(got["kv_cache"].view(-1, 512)[rows], gold["kv_cache"].view(-1, 512)[rows], "kv_cache", 0.0078125, 1e-4)
-    floats(got["kr_cache"].view(-1, 64)[rows], gold["kr_cache"].view(-1, 64)[rows], "kr_cache", 0.0078125, 1e-4, 0.95)
+    check_rope_cache(case, got["kr_cache"], gold["kr_cache"], eps)
     keep = torch.ones(case["kv_cache"].shape[0] * case["kv_cache"].shape[1], dtype=torch.bool)
     keep[rows] = False
     assert torch.equal(got["kv_cache"].view(-1, 512)[keep], case["kv_cache"].view(-1, 512)[keep])

@@ -15,6 +15,17 @@ def test_flash_matches_fp64_within_bf16():
     assert torch.equal(o[5].view(2, 6, 128), c["v"][blk, 0].unsqueeze(1).expand(2, 6, 128))
 
 
+def test_tile_argument_regroups_the_same_rows():
+    """tile = page size walks the page table by positions instead of by pages: the same rows, so the same bits; one tile
+    per sequence is plain softmax attention with one bf16 rounding of P~."""
+    c = gqa.make_case(2, 2, 4, 2, [150, 33], seed=4, block_size=32)
+    args = (c["q"], c["k"], c["v"], c["block_table"], c["act_seq"], c["softmax_scale"])
+    assert torch.equal(gqa.attention_flash(*args, tile=32), gqa.attention_flash(*args))
+    whole = gqa.attention_flash(*args, tile=150)
+    r = gqa.attention_fp64(*args)
+    assert (whole.double() - r).abs().max() < 2.0 ** -7 * r.abs().max() + 1e-3
+
+
 def test_zero_query_gives_the_mean_of_v():
     c = gqa.make_case(1, 1, 8, 2, [200], seed=2, block_size=32, dist="uniform")
     q = torch.zeros_like(c["q"])
