@@ -122,9 +122,8 @@ int bind_workspace(const char* op, SfaPlan* plan, void* ws, uint64_t ws_bytes)
         return fail(PTO_ERR_WORKSPACE, "%s: workspace of %llu bytes required, got %llu", op,
                     (unsigned long long)plan->ws_bytes, (unsigned long long)(ws ? ws_bytes : 0));
     pto::SfaArgs& a = plan->args;
-    const uint64_t rows = (uint64_t)a.b * a.s1 * a.nsplit * a.nq;
     a.part_o = static_cast<_Float16*>(ws);
-    a.part_ml = reinterpret_cast<float*>(a.part_o + rows * 512);
+    a.part_ml = reinterpret_cast<float*>(static_cast<char*>(ws) + pto::sfa_partials_bytes(a.b * a.s1, a.nq, a.nsplit));
     return PTO_OK;
 }
 

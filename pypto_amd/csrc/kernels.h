@@ -20,7 +20,7 @@ struct SfaArgs {
     const int32_t* block_table; // [b, bt_stride]
     const int32_t* act_seq;     // [b]
     void* out;                  // [t*nq, 512] bf16
-    _Float16* part_o;           // [t, nsplit, nq, 512] fp16: each split's output normalised by its own sum (nsplit > 1)
+    _Float16* part_o;           // [t, nsplit, head groups, 128 x 512] fp16 in the accumulators' fragment order: each split's output normalised by its own sum (nsplit > 1)
     float* part_ml;             // [t, nsplit, nq, 2]  fp32 (running max in log2 units, sum)
     int32_t b, s1, nq, topk, topk_stride, block_size, bt_stride, nsplit;
     int32_t split_cap; // set by sfa_launch: capacity (tokens) of the per-split LDS arrays
@@ -31,6 +31,7 @@ struct SfaArgs {
 
 int sfa_pick_splits(int t, int nq, int topk);
 uint64_t sfa_workspace_bytes(int t, int nq, int nsplit);
+uint64_t sfa_partials_bytes(int t, int nq, int nsplit); // the fp16 partials at the front of that workspace; (m, l) follow
 hipError_t sfa_launch(const SfaArgs& a, hipStream_t stream);
 // Device address, on the current device, of the library's own scratch array of SFA_STATIC_SCRATCH_BYTES bytes (looked up
 // once per device).  Every call on a GPU shares that GPU's array.

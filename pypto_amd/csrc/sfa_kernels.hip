@@ -28,11 +28,11 @@
 // the rate), and two waves issuing vector work fill the vector port (one wave alone issues at about half its rate);
 // running the phases of two wave groups one barrier interval apart was measured and is slower.
 //
-// KV splits write their output normalised by their own sum as fp16 plus (m, l); sfa_combine_kernel merges them.
+// KV splits write their output normalised by their own sum as fp16, in the accumulators' fragment order, plus (m, l);
+// sfa_combine_kernel merges them and turns the result into rows.
 #include "common.h"
 #include "kernels.h"
 #include "timing.h"
-#include <type_traits>
 
 namespace pto {
 namespace {
@@ -632,14 +632,9 @@ __device__ __forceinline__ void sfa_wave(const SfaArgs& a, uint8_t* smem, uint32
         }
     }
 
-    // Epilogue.  The softmax waves publish the row sums (in a part of LDS the staging area below does not reach); then
-    // every wave normalises its O^T blocks, rounds them to the output's 16-bit type and stages them in LDS as
-    // [head][512] rows of 1024 bytes (everything below OUT_LSUM_OFF is free now), and all 512 lanes copy the rows out,
-    // a wavefront writing one whole row per instruction.  Register r of o[i][hb] holds dim
-    // 32*(4*dq + i) + 8*(r/4) + 4*hl + r%4 of head 64*hh + 32*hb + l32: four consecutive dims, and the other half-wave
-    // holds the four next to them.  v_permlane32_swap pairs them up - the lower half-wave ends up with the 8 dims of
-    // block g = 2 gp, the upper one with those of block 2 gp + 1 - so that a lane stores 16 bytes; the 16-byte chunks
-    // of a row are XOR-swizzled with the head so that the 8 lanes of a b128 access hit distinct banks.
+    // Epilogue.  The softmax waves publish the row sums (in a part of LDS the staging area below does not reach) and every
+    // wave normalises its O^T blocks.  Register r of o[i][hb] holds dim 32*(4*dq + i) + 8*(r/4) + 4*hl + r%4 of head
+    // 64*hh + 32*hb + l32: four consecutive dims, and the other half-wave holds the four next to them.
     float* lsum = reinterpret_cast<float*>(smem + OUT_LSUM_OFF);
     if (KH == 0) {
         const float l_tot = l_run + __shfl_xor(l_run, 32);
@@ -651,12 +646,41 @@ __device__ __forceinline__ void sfa_wave(const SfaArgs& a, uint8_t* smem, uint32
         }
     }
     __syncthreads(); // row sums published; nobody reads a tile, P~ or parked Q any more
-    const bool final_out = a.nsplit == 1; // bf16 output; otherwise the split's share, normalised by its own sum, in fp16:
-                                          // |value| <= max |V| and 2^-11 relative rounding, a quarter of the final bf16
-                                          // rounding, half the bytes of fp32 for this kernel to write and the merge to read
-    // (one copy of the staging code per output type: a test of the type inside it ends up as a branch per value pair)
-    auto stage_out = [&](auto as_final) {
-        constexpr bool FINAL = decltype(as_final)::value;
+    if (a.nsplit > 1) {
+        // A split's share, normalised by its own sum, in fp16 (|value| <= max |V| and 2^-11 relative rounding, a quarter
+        // of the final bf16 rounding, half the bytes of fp32 for this kernel to write and the merge to read).  It leaves
+        // in fragment order, straight from the accumulators: [token][split][head group][wave 8][hb 2][i 4][half 2]
+        // [lane 64] x 8 fp16 - every store instruction writes 1 KB of consecutive bytes, and nothing is staged.  The
+        // merge kernel reads the same order and does the transposition to rows once, for the output, instead of once
+        // per split here.  (Streaming stores: 34 MB leave the chip's 256 workgroups at once and are read back once.)
+        if (pv_active) {
+            const int wave = tid >> 6;
+            _Float16* wbase = a.part_o + ((((int64_t)tq * a.nsplit + sp) * gridDim.z + hz) * 8 + wave) * 8192 + lane * 8;
+#pragma unroll
+            for (int hb = 0; hb < 2; ++hb) {
+                const float l = lsum[64 * hh + 32 * hb + l32];
+                const float mul = l > 0.f ? 1.f / l : 0.f;
+#pragma unroll
+                for (int i = 0; i < 4; ++i)
+#pragma unroll
+                    for (int h = 0; h < 2; ++h) {
+                        typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
+                        uint32_t w[4];
+#pragma unroll
+                        for (int k = 0; k < 4; ++k)
+                            w[k] = __builtin_bit_cast(uint32_t, f16x2{(_Float16)(o[i][hb][8 * h + 2 * k] * mul), (_Float16)(o[i][hb][8 * h + 2 * k + 1] * mul)});
+                        __builtin_nontemporal_store(u32x4{w[0], w[1], w[2], w[3]}, reinterpret_cast<u32x4*>(wbase + ((hb * 4 + i) * 2 + h) * 512));
+                    }
+            }
+        }
+        return;
+    }
+    // One split: the output itself, bf16 rows.  v_permlane32_swap pairs up the two half-waves' four-dim pieces - the lower
+    // half-wave ends up with the 8 dims of block g = 2 gp, the upper one with those of block 2 gp + 1 - so that a lane
+    // stores 16 bytes; all 128 heads' rows are staged in LDS as [head][512] rows of 1024 bytes (everything below
+    // OUT_LSUM_OFF is free now), the 16-byte chunks of a row XOR-swizzled with the head so that the 8 lanes of a b128
+    // access hit distinct banks, and all 512 lanes copy the rows out, a wavefront writing one whole row per instruction.
+    if (pv_active) {
 #pragma unroll
         for (int hb = 0; hb < 2; ++hb) {
             const int hrow = 64 * hh + 32 * hb + l32;
@@ -671,15 +695,8 @@ __device__ __forceinline__ void sfa_wave(const SfaArgs& a, uint8_t* smem, uint32
 #pragma unroll
                     for (int g = 0; g < 2; ++g)
 #pragma unroll
-                        for (int k = 0; k < 2; ++k) {
-                            const float x = o[i][hb][4 * (2 * gp + g) + 2 * k] * mul, y = o[i][hb][4 * (2 * gp + g) + 2 * k + 1] * mul;
-                            if constexpr (FINAL) {
-                                w[g][k] = pack_bf16x2(x, y);
-                            } else {
-                                typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
-                                w[g][k] = __builtin_bit_cast(uint32_t, f16x2{(_Float16)x, (_Float16)y});
-                            }
-                        }
+                        for (int k = 0; k < 2; ++k)
+                            w[g][k] = pack_bf16x2(o[i][hb][4 * (2 * gp + g) + 2 * k] * mul, o[i][hb][4 * (2 * gp + g) + 2 * k + 1] * mul);
                     // the swap exchanges the upper half-wave of its first operand with the lower half-wave of its second
                     const auto s0 = __builtin_amdgcn_permlane32_swap(w[0][0], w[1][0], false, false);
                     const auto s1 = __builtin_amdgcn_permlane32_swap(w[0][1], w[1][1], false, false);
@@ -687,12 +704,6 @@ __device__ __forceinline__ void sfa_wave(const SfaArgs& a, uint8_t* smem, uint32
                     *reinterpret_cast<u32x4*>(orow + ((c ^ (hrow & 7)) << 4)) = u32x4{(uint32_t)s0[0], (uint32_t)s1[0], (uint32_t)s0[1], (uint32_t)s1[1]};
                 }
         }
-    };
-    if (pv_active) {
-        if (final_out)
-            stage_out(std::true_type{});
-        else
-            stage_out(std::false_type{});
     }
     __syncthreads();
 #pragma unroll 4
@@ -701,15 +712,7 @@ __device__ __forceinline__ void sfa_wave(const SfaArgs& a, uint8_t* smem, uint32
         const int oh = head0 + hrow;
         if (oh >= a.nq) break; // (wave-uniform: a wavefront copies one row)
         const u32x4 v = *reinterpret_cast<const u32x4*>(smem + hrow * OUT_ROW + ((c ^ (hrow & 7)) << 4));
-        if (final_out) {
-            *reinterpret_cast<u32x4*>(reinterpret_cast<uint8_t*>(a.out) + (((int64_t)tq * a.nq + oh) * DN + c * 8) * 2) = v;
-        } else {
-            // (streaming stores: 34 MB leave the chip's 256 workgroups at once and are read back once by the merge;
-            // kept out of the caches they cost this kernel 1.5 us less, and the next step's index cache stream finds
-            // the caches free of them)
-            const int64_t prow = ((int64_t)tq * a.nsplit + sp) * a.nq + oh;
-            __builtin_nontemporal_store(v, reinterpret_cast<u32x4*>(a.part_o + prow * DN + c * 8));
-        }
+        *reinterpret_cast<u32x4*>(reinterpret_cast<uint8_t*>(a.out) + (((int64_t)tq * a.nq + oh) * DN + c * 8) * 2) = v;
     }
 }
 
@@ -742,53 +745,88 @@ __global__ void sfa_zero_kernel(uint32_t* out, int64_t n_words)
 }
 
 // out[row, :] = sum_s (2^(m_s - M) l_s / L) o_s[row, :] with L = sum_s 2^(m_s - M) l_s and o_s the split's normalised
-// output; one wavefront per output row (a lane owns 8 of the 512 values, 16 bytes of every split's fp16 row), four rows
-// per workgroup.  Splits are taken eight at a time, every load of a group requested before any is used (splits past
-// the last are the last again with weight 0).
+// output.  The partials lie in the fragment order the attention kernel's accumulators have (see its epilogue).  One
+// workgroup merges, for one token, what wave wv of the attention workgroups left for head block hb: 32 heads x 128
+// value columns; its wavefront i takes column block i, a lane owning for its head (l32) the four 4-column runs at
+// 32 i + 16 h + 8 g + 4 hl.  Splits are taken eight at a time, every load of a group requested before any is used
+// (splits past the last are the last again with weight 0).  The workgroup then turns its 32 x 128 block through LDS
+// and writes the 256-byte row pieces, 16 lanes a piece.
+constexpr int CROW = 128 * 2 + 16; // LDS row of the merge's transposition: 128 bf16 plus one 16-byte chunk of padding
 __global__ __launch_bounds__(256) void sfa_combine_kernel(const void* __restrict__ part_o_fp16,
                                                           const float* __restrict__ part_ml, void* out, int nq,
-                                                          int nsplit, int n_rows)
+                                                          int nsplit, int hgroups)
 {
+    __shared__ __align__(16) uint8_t tr[32 * CROW];
     const _Float16* part_o = static_cast<const _Float16*>(part_o_fp16); // (a plain pointer type keeps the symbol readable)
-    const int lane = threadIdx.x & 63;
-    const int row = blockIdx.x * 4 + (threadIdx.x >> 6); // tq * nq + head
-    if (row >= n_rows) return;
-    const int tq = row / nq, head = row - tq * nq;
+    const int lane = threadIdx.x & 63, l32 = lane & 31, hl = lane >> 5;
+    const int i = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int task = blockIdx.x; // ((tq * hgroups + hz) * 8 + wv) * 2 + hb
+    const int hb = task & 1, wv = (task >> 1) & 7;
+    const int th = task >> 4, hz = th % hgroups, tq = th / hgroups;
+    const int hh = wv & 1, dq = wv >> 1;
+    const int head_base = hz * HEADS_PER_WG + 64 * hh + 32 * hb;
+    if (head_base >= nq) return; // (a head block past the last head: nothing was written for it)
+    const int headc = min(head_base + l32, nq - 1);
     constexpr int G = 8;
-    float acc[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+    float acc[2][8];
+#pragma unroll
+    for (int x = 0; x < 16; ++x) (&acc[0][0])[x] = 0.f;
     float M = -INFINITY, L = 0.f;
+    const int64_t split_stride = (int64_t)hgroups * 8 * 8192; // fp16 elements between two splits of a token
+    const _Float16* frag0 = part_o + (((int64_t)tq * nsplit * hgroups + hz) * 8 + wv) * 8192 + (hb * 4 + i) * 1024; // (the workgroup's four wavefronts read 8 KB in a row per split)
+    const float* ml0 = part_ml + (int64_t)tq * nsplit * nq * 2;
     for (int s0 = 0; s0 < nsplit; s0 += G) {
-        f16x8 v[G];
+        f16x8 v[G][2];
         float m[G], l[G];
 #pragma unroll
         for (int j = 0; j < G; ++j) {
-            const int64_t prow = ((int64_t)tq * nsplit + min(s0 + j, nsplit - 1)) * nq + head;
-            v[j] = *reinterpret_cast<const f16x8*>(part_o + prow * DN + lane * 8);
-            m[j] = part_ml[prow * 2];
-            l[j] = s0 + j < nsplit ? part_ml[prow * 2 + 1] : 0.f;
+            const int s = min(s0 + j, nsplit - 1);
+            const _Float16* base = frag0 + s * split_stride;
+#pragma unroll
+            for (int h = 0; h < 2; ++h) v[j][h] = __builtin_nontemporal_load(reinterpret_cast<const f16x8*>(base + h * 512 + lane * 8));
+            m[j] = ml0[((int64_t)s * nq + headc) * 2];
+            l[j] = s0 + j < nsplit ? ml0[((int64_t)s * nq + headc) * 2 + 1] : 0.f;
         }
         // the group's maximum joins the running one: what was summed so far is rescaled once per group
         float Mg = M;
 #pragma unroll
         for (int j = 0; j < G; ++j) Mg = l[j] > 0.f ? fmaxf(Mg, m[j]) : Mg;
-        if (Mg == -INFINITY) continue; // nothing attended in these splits
-        const float back = exp2f(M - Mg); // 0 while nothing has been summed (M = -inf)
-        L *= back;
+        if (Mg != -INFINITY) { // (otherwise nothing attended in these splits)
+            if (s0 > 0) {
+                const float back = exp2f(M - Mg); // 0 while nothing has been summed (M = -inf)
+                L *= back;
 #pragma unroll
-        for (int e = 0; e < 8; ++e) acc[e] *= back;
-        M = Mg;
+                for (int x = 0; x < 16; ++x) (&acc[0][0])[x] *= back;
+            }
+            M = Mg;
 #pragma unroll
-        for (int j = 0; j < G; ++j) {
-            const float w = l[j] > 0.f ? exp2f(m[j] - M) * l[j] : 0.f;
-            L += w;
+            for (int j = 0; j < G; ++j) {
+                const float w = l[j] > 0.f ? exp2f(m[j] - M) * l[j] : 0.f;
+                L += w;
 #pragma unroll
-            for (int e = 0; e < 8; ++e) acc[e] += (float)v[j][e] * w;
+                for (int h = 0; h < 2; ++h)
+#pragma unroll
+                    for (int e = 0; e < 8; ++e) acc[h][e] += (float)v[j][h][e] * w;
+            }
         }
     }
     const float inv = L > 0.f ? 1.f / L : 0.f;
-    const u32x4 w = {pack_bf16x2(acc[0] * inv, acc[1] * inv), pack_bf16x2(acc[2] * inv, acc[3] * inv),
-                     pack_bf16x2(acc[4] * inv, acc[5] * inv), pack_bf16x2(acc[6] * inv, acc[7] * inv)};
-    *reinterpret_cast<u32x4*>(reinterpret_cast<uint8_t*>(out) + ((int64_t)row * DN + lane * 8) * 2) = w;
+#pragma unroll
+    for (int h = 0; h < 2; ++h)
+#pragma unroll
+        for (int g = 0; g < 2; ++g) {
+            const float* x = &acc[h][4 * g];
+            const u32x2 w = {pack_bf16x2(x[0] * inv, x[1] * inv), pack_bf16x2(x[2] * inv, x[3] * inv)};
+            *reinterpret_cast<u32x2*>(tr + l32 * CROW + (32 * i + 16 * h + 8 * g + 4 * hl) * 2) = w;
+        }
+    __syncthreads();
+#pragma unroll
+    for (int k = 0; k < 2; ++k) {
+        const int r = 16 * k + (threadIdx.x >> 4), c = threadIdx.x & 15;
+        const u32x4 w = *reinterpret_cast<const u32x4*>(tr + r * CROW + c * 16);
+        if (head_base + r < nq)
+            *reinterpret_cast<u32x4*>(reinterpret_cast<uint8_t*>(out) + (((int64_t)tq * nq + head_base + r) * DN + 128 * dq + 8 * c) * 2) = w;
+    }
 }
 
 int num_cus()
@@ -817,10 +855,17 @@ int sfa_pick_splits(int t, int nq, int topk)
     return n;
 }
 
+uint64_t sfa_partials_bytes(int t, int nq, int nsplit)
+{
+    if (nsplit <= 1) return 0;
+    const int hgroups = (nq + HEADS_PER_WG - 1) / HEADS_PER_WG; // (whole 128-head groups: the partials lie in fragment order)
+    return (uint64_t)t * nsplit * hgroups * HEADS_PER_WG * DN * sizeof(_Float16);
+}
+
 uint64_t sfa_workspace_bytes(int t, int nq, int nsplit)
 {
     if (nsplit <= 1) return 0;
-    return (uint64_t)t * nsplit * nq * (DN * sizeof(_Float16) + 2 * sizeof(float));
+    return sfa_partials_bytes(t, nq, nsplit) + (uint64_t)t * nsplit * nq * 2 * sizeof(float);
 }
 
 // Scratch for callers that cannot allocate (sfa_static_scratch): one array per GPU the library runs on, held until the
@@ -880,9 +925,8 @@ hipError_t sfa_launch(const SfaArgs& a, hipStream_t stream)
     if (e != hipSuccess) return e;
     if (a.nsplit > 1) {
         ScopedKernelTimer tm(KID_SFA_COMBINE, stream);
-        const int n_rows = t * a.nq;
-        hipLaunchKernelGGL(sfa_combine_kernel, dim3((n_rows + 3) / 4), dim3(256), 0, stream, static_cast<const void*>(a.part_o),
-                           a.part_ml, a.out, a.nq, a.nsplit, n_rows);
+        hipLaunchKernelGGL(sfa_combine_kernel, dim3(t * hgroups * 16), dim3(256), 0, stream, static_cast<const void*>(a.part_o),
+                           a.part_ml, a.out, a.nq, a.nsplit, hgroups);
         e = hipGetLastError();
     }
     return e;
