@@ -783,7 +783,7 @@ __global__ __launch_bounds__(256) void sfa_combine_kernel(const void* __restrict
             const int s = min(s0 + j, nsplit - 1);
             const _Float16* base = frag0 + s * split_stride;
 #pragma unroll
-            for (int h = 0; h < 2; ++h) v[j][h] = __builtin_nontemporal_load(reinterpret_cast<const f16x8*>(base + h * 512 + lane * 8));
+            for (int h = 0; h < 2; ++h) v[j][h] = *reinterpret_cast<const f16x8*>(base + h * 512 + lane * 8);
             m[j] = ml0[((int64_t)s * nq + headc) * 2];
             l[j] = s0 + j < nsplit ? ml0[((int64_t)s * nq + headc) * 2 + 1] : 0.f;
         }
