@@ -71,6 +71,10 @@ def parse():
     ap.add_argument("--warm-weights", action="store_true",
                     help="prolog workloads: one copy of the weights, re-read every step (they then partly come out of "
                          "the 256 MB last-level cache); default: rotate enough copies to exceed it")
+    ap.add_argument("--streams", type=int, default=1,
+                    help="v32 workload: launch consecutive steps on this many HIP streams in turn (each with its own "
+                         "outputs), the way a server keeps several micro-batches in flight; the default, 1, is the "
+                         "headline measurement")
     ap.add_argument("--graph", action="store_true",
                     help="replay the step from HIP graphs (one per cache copy) instead of launching it eagerly")
     ap.add_argument("--calibrate-copy", action="store_true",
@@ -684,20 +688,35 @@ def main():
     cfg, tile = LightningIndexerConfigs(), SaTileShapeConfig()
     unroll = [128, 64, 32, 16, 8, 4, 1]
 
-    def step(i):
+    def one_step(i, topk_res, out):
         s = w["sets"][i % nbuf]
         lightning_indexer_decode(w["idx_q"], w["idx_qs"], s["idx_k"], s["idx_ks"], w["idx_w"], w["act"], w["table"],
-                                 w["topk_res"], unroll, cfg, 2048)
-        tk = w["topk_res"].view(b * s1, 2048)
+                                 topk_res, unroll, cfg, 2048)
+        tk = topk_res.view(b * s1, 2048)
         if args.packed:
             sparse_attention_antiquant_d(w["q_nope"], w["q_rope"], s["rows"], tk, w["table"], w["act"],
-                                         w["out"].view(b * s1 * 128, 512), 128, 1, scale, 2048, 128,
+                                         out.view(b * s1 * 128, 512), 128, 1, scale, 2048, 128,
                                          w["pages_per_seq"], tile)
         else:
             sparse_flash_attention_quant_d(w["q_nope"], w["q_rope"], s["kn"], s["kr"], s["ks"], tk, w["table"],
-                                           w["act"], w["out"], 128, 1, scale, 2048, 128, w["pages_per_seq"], tile)
+                                           w["act"], out, 128, 1, scale, 2048, 128, w["pages_per_seq"], tile)
+
+    def step(i):
+        one_step(i, w["topk_res"], w["out"])
 
     eager_step = step
+    if args.streams > 1:
+        if args.graph:
+            print("--streams and --graph do not combine", file=sys.stderr)
+            sys.exit(2)
+        # consecutive steps on different streams, each stream with outputs of its own (the inputs are only read)
+        lanes = [(torch.cuda.Stream(), torch.empty_like(w["topk_res"]), torch.empty_like(w["out"])) for _ in range(args.streams)]
+        torch.cuda.synchronize()
+
+        def step(i):  # noqa: F811
+            st, topk_res, out = lanes[i % args.streams]
+            with torch.cuda.stream(st):
+                one_step(i, topk_res, out)
     if args.graph:
         side = torch.cuda.Stream()
         side.wait_stream(torch.cuda.current_stream())
@@ -739,7 +758,7 @@ def main():
     evs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(n_single)]
     for i, (e0, e1) in enumerate(evs):
         e0.record()
-        step(i)
+        eager_step(i)
         e1.record()
     torch.cuda.synchronize()
     single = sorted(e0.elapsed_time(e1) * 1e3 for e0, e1 in evs)
@@ -824,7 +843,7 @@ def main():
         "value": round(tokens_per_s, 1), "unit": "tokens/s", "n_gpus": 1, "steps": args.steps,
         "warmup": args.warmup, "ms_per_step": round(ms_per_step, 4), "higher_is_better": True, "scaling": "weak",
         "vs_baseline": None, "dtype": "int8+bf16",
-        "data": "synthetic", "launch": "hip graph replay" if args.graph else "eager",
+        "data": "synthetic", "launch": "hip graph replay" if args.graph else "eager" if args.streams == 1 else f"eager, steps in turn on {args.streams} streams",
         "config": {"workload": f"lightning indexer top-2048 + sparse flash attention decode, batch {b}, "
                                f"s1 {s1}, ctx {f'U[{args.ctx_min}, {ctx}]' if args.ctx_min else ctx}, 64x128 int8 index heads, 128 heads x (512 nope + 64 rope), "
                                f"int8 paged MLA cache, block 128, {'packed 656 B rows' if args.packed else 'three cache tensors'}"},
