@@ -41,6 +41,8 @@ constexpr int PASSES = 4;       // passes per workgroup (amortise the Q / w_scal
 constexpr int MAX_K = 2048;     // top-k capacity
 constexpr int NBINS = 2048;     // digit bins of the radix select and of the final ordering (11 bits)
 constexpr int SBINS = 256;      // bins of the selection histogram (score_bin)
+constexpr int SUBBINS = 64;     // second level inside the threshold bin: the next six key bits (tie_sub_bin)
+constexpr int SUB_RANK_CAP = 128; // ties of one second-level step that are ranked by direct comparison (more: digit by digit)
 constexpr int SEL_CHUNK = 4096; // scores per workgroup of the select kernel
 constexpr int TIE_CAP = 8192;   // capacity of the per-row tie list
 
@@ -79,6 +81,8 @@ __device__ __forceinline__ uint32_t score_bin(uint32_t key)
     return t >= 1024 ? 128u + (uint32_t)min(max(t - 1024 - LO, 0), 127) : (uint32_t)min(max(t - (1023 - LO - 127), 0), 127);
 }
 __device__ __forceinline__ bool score_bin_is_interior(uint32_t bin) { return (bin & 127u) != 0u && (bin & 127u) != 127u; }
+// The keys of an interior bin share their top 11 bits; the next six split the bin into 64 equal steps, in key order.
+__device__ __forceinline__ uint32_t tie_sub_bin(uint32_t key) { return (key >> 15) & (SUBBINS - 1u); }
 // Smallest and largest key of a bin (the first and last bin of a sign reach to the end of the sign's keys).
 __device__ __forceinline__ void score_bin_range(uint32_t bin, uint32_t& lo, uint32_t& hi)
 {
@@ -482,6 +486,13 @@ __global__ void indexer_fill_kernel(int32_t* p, int n, int32_t v)
     if (i < n) p[i] = v;
 }
 
+// inclusive suffix sum over a wavefront (lane l gets the sum of v[l .. 63]); all 64 lanes active
+__device__ __forceinline__ uint32_t wave_suffix_sum(uint32_t v)
+{
+    const uint32_t incl = wave_prefix_sum(v);
+    return (uint32_t)__builtin_amdgcn_readlane((int)incl, 63) - incl + v;
+}
+
 // block-wide inclusive suffix sum (lane t gets sum of v[t .. nthreads-1]); tmp holds one word per wavefront
 template <int NWAVES>
 __device__ __forceinline__ uint32_t block_suffix_sum(uint32_t v, uint32_t* tmp)
@@ -821,10 +832,68 @@ __global__ __launch_bounds__(1024) void indexer_topk_kernel(IndexerArgs a)
         auto each = [&](auto&& f) {
             for (int i = tid; i < (int)n_tie; i += 1024) f(tie[i]);
         };
-        // the ties of an interior bin share their top 11 key bits; those of a first or last bin (magnitudes outside the
-        // histogram's range) need not
-        const int top = score_bin_is_interior(score_bin((uint32_t)(tie[0] >> 32))) ? 53 : 64;
-        radix_select64(each, emit, need, top, hist, tmp, &s_bin, &s_krem, &s_cnt);
+        if (score_bin_is_interior(score_bin((uint32_t)(tie[0] >> 32)))) {
+            // The ties of an interior bin share their top 11 key bits.  They are counted by the next six (64 steps in
+            // key order, one LDS counter each); a suffix scan of the 64 counts by one wavefront finds the step that holds
+            // the last wanted tie.  Ties in the steps above it are taken, those inside it (a few dozen) are set aside
+            // and ranked against each other.  (Against a digit of the radix select: 64 counters instead of 2048 to clear
+            // and scan, and no second digit.)
+            uint32_t* subc = hist + NBINS - SUBBINS; // (the far end of hist: its front holds the ties set aside)
+            if (tid < SUBBINS) subc[tid] = 0u;
+            if (tid == 0) { // (overwritten below by the lane whose step it is)
+                s_bin = 0u;
+                s_krem = need;
+                s_cnt = 0xffffffffu;
+                tmp[0] = 0u;
+            }
+            __syncthreads();
+            each([&](uint64_t w) { atomicAdd(&subc[tie_sub_bin((uint32_t)(w >> 32))], 1u); });
+            __syncthreads();
+            if (tid < SUBBINS) {
+                const uint32_t c_sub = subc[tid];
+                const uint32_t above = wave_suffix_sum(c_sub) - c_sub;
+                if (above < need && need <= above + c_sub) {
+                    s_bin = (uint32_t)tid;
+                    s_krem = need - above;
+                    s_cnt = c_sub;
+                }
+            }
+            __syncthreads();
+            const uint32_t sb = s_bin, krem = s_krem, cnt = s_cnt;
+            const bool whole = cnt == krem, small = cnt <= SUB_RANK_CAP;
+            uint64_t* aside = reinterpret_cast<uint64_t*>(hist);
+            each([&](uint64_t w) {
+                const uint32_t d = tie_sub_bin((uint32_t)(w >> 32));
+                if (d > sb || (whole && d == sb))
+                    emit(w);
+                else if (d == sb && small) {
+                    const uint32_t p = atomicAdd(&tmp[0], 1u);
+                    if (p < SUB_RANK_CAP) aside[p] = w;
+                }
+            });
+            __syncthreads();
+            if (!whole && small) {
+                // (words are distinct: the rank of one among the others is the number of larger ones)
+                if (tid < (int)cnt) {
+                    const uint64_t w = aside[tid];
+                    uint32_t larger = 0;
+                    for (uint32_t j = 0; j < cnt; ++j) larger += aside[j] > w ? 1u : 0u;
+                    if (larger < krem) emit(w);
+                }
+            } else if (!whole) {
+                // a crowded step (heavily tied scores): digit by digit over its 15 remaining key bits and the index
+                __syncthreads();
+                auto each_in = [&](auto&& f) {
+                    each([&](uint64_t w) {
+                        if (tie_sub_bin((uint32_t)(w >> 32)) == sb) f(w);
+                    });
+                };
+                radix_select64(each_in, emit, krem, 47, hist, tmp, &s_bin, &s_krem, &s_cnt);
+            }
+        } else {
+            // a first or last bin (magnitudes outside the histogram's range): its keys need not share any bits
+            radix_select64(each, emit, need, 64, hist, tmp, &s_bin, &s_krem, &s_cnt);
+        }
     } else if (need > 0) {
         // overflowed tie list: select over the whole row instead (winners are found again, so start empty)
         if (tid == 0) s_out = 0;
