@@ -49,8 +49,11 @@ def profile_traffic(name):
 def parse():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=50)
-    ap.add_argument("--warmup", type=int, default=10)
+    # (the first hundred or so steps after an idle period run 8-10 % slower than the steady state - clocks and caches
+    # come up - so the defaults warm up for 100 steps and time 500; the whole default run still takes well under a minute
+    # of GPU time)
+    ap.add_argument("--steps", type=int, default=500)
+    ap.add_argument("--warmup", type=int, default=100)
     ap.add_argument("--batch", type=int, default=32)
     ap.add_argument("--ctx", type=int, default=65536)
     ap.add_argument("--s1", type=int, default=1)
