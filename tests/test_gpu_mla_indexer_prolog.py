@@ -15,7 +15,7 @@ import torch
 
 from oracle import mla_prolog as op
 from test_gpu_indexer_prolog import WEIGHTS_REL, weights_allowance
-from test_gpu_mla_prolog import check_rope_cache
+from test_gpu_mla_prolog import FEW, check_rope_cache
 
 pytestmark = pytest.mark.gpu
 EPS = 1e-5
@@ -80,22 +80,26 @@ def check_against_oracle(mla_case, idx_case, got):
 
     def ints(a, b, name, tol, min_equal):
         diff = (a.int() - b.int()).abs()
-        assert diff.max() <= tol, f"{name}: off by {int(diff.max())}"
+        # (a quantisation scale that moved by one bf16 step of the row's largest value moves a quantised value v by
+        # v / 128 steps: in the upper half of the int8 range that is one more step than the value's own rounding)
+        assert (diff <= tol + (b.int().abs() >= 64).int()).all(), f"{name}: off by {int(diff.max())}"
         assert (diff == 0).float().mean() >= min_equal, f"{name}: {(diff != 0).float().mean():.4f} of the values differ"
 
     def close(a, b, name, rel=2.0 ** -7, atol=1e-8, outliers=0.0):
         a, b = a.float().flatten(), b.float().flatten()
         assert torch.isfinite(a).all(), name
         ratio = (a - b).abs() / (rel * b.abs() + atol)
-        assert (ratio > 1).float().mean() <= outliers and ratio.max() <= 3, \
+        assert int((ratio > 1).sum()) <= (max(outliers * ratio.numel(), FEW) if outliers else 0) and ratio.max() <= 3, \
             f"{name}: {int((ratio > 1).sum())} values out of tolerance, worst {float(ratio.max())} x"
 
     ints(got["kv_cache"].view(-1, 512)[rows], gm["kv_cache"].view(-1, 512)[rows], "kv_cache", 1, 0.98)
     close(got["k_scale_cache"].view(-1, 4)[rows], gm["k_scale_cache"].view(-1, 4)[rows], "k_scale_cache", rel=2.0 ** -6)  # see test_gpu_mla_prolog
-    close(got["q_nope"], gm["q_nope"], "q_nope", 0.0078125, 0.005, outliers=1e-3)   # see test_gpu_mla_prolog
-    close(got["q_rope"], gm["q_rope"], "q_rope", 0.0078125, 0.005, outliers=1e-3)
+    close(got["q_nope"], gm["q_nope"], "q_nope", 0.0078125, 0.005, outliers=5e-3)   # see test_gpu_mla_prolog
+    close(got["q_rope"], gm["q_rope"], "q_rope", 0.0078125, 0.005, outliers=5e-3)
     check_rope_cache(mla_case, got["kr_cache"], gm["kr_cache"], EPS)   # see test_gpu_mla_prolog
-    ints(got["q_int8"], gi["q_int8"], "q_int8", 2, 0.95)
+    # (the reference's widened tolerance of 2; with a q_lora_rank of 128 a flipped q_norm value is one of only 128 terms
+    # of a product and moves it by more: 3 there)
+    ints(got["q_int8"], gi["q_int8"], "q_int8", 2 if mla_case["w_dq"].shape[1] >= 256 else 3, 0.95)
     # (the golden's index queries come from the golden's q_norm, the product's from its own: a q_norm value that rounded
     # the other way shifts the 128 values of a head a little, on top of the one bf16 step their own rounding can move,
     # which is why q_int8 gets 2 above; a query scale follows the largest of them, so two bf16 steps here.  The tight
