@@ -748,10 +748,12 @@ __global__ void sfa_zero_kernel(uint32_t* out, int64_t n_words)
 // output.  The partials lie in the fragment order the attention kernel's accumulators have (see its epilogue).  One
 // workgroup merges, for one token, what wave wv of the attention workgroups left for head block hb: 32 heads x 128
 // value columns; its wavefront i takes column block i, a lane owning for its head (l32) the four 4-column runs at
-// 32 i + 16 h + 8 g + 4 hl.  Splits are taken eight at a time, every load of a group requested before any is used
-// (splits past the last are the last again with weight 0).  The workgroup then turns its 32 x 128 block through LDS
+// 32 i + 16 h + 8 g + 4 hl.  Splits are taken G at a time (G = 2, 4 or 8: the smallest that covers the split count,
+// eight for more than eight splits), every load of a group requested before any is used (splits past the last are the
+// last again with weight 0).  The workgroup then turns its 32 x 128 block through LDS
 // and writes the 256-byte row pieces, 16 lanes a piece.
 constexpr int CROW = 128 * 2 + 16; // LDS row of the merge's transposition: 128 bf16 plus one 16-byte chunk of padding
+template <int G>
 __global__ __launch_bounds__(256) void sfa_combine_kernel(const void* __restrict__ part_o_fp16,
                                                           const float* __restrict__ part_ml, void* out, int nq,
                                                           int nsplit, int hgroups)
@@ -767,7 +769,6 @@ __global__ __launch_bounds__(256) void sfa_combine_kernel(const void* __restrict
     const int head_base = hz * HEADS_PER_WG + 64 * hh + 32 * hb;
     if (head_base >= nq) return; // (a head block past the last head: nothing was written for it)
     const int headc = min(head_base + l32, nq - 1);
-    constexpr int G = 8;
     float acc[2][8];
 #pragma unroll
     for (int x = 0; x < 16; ++x) (&acc[0][0])[x] = 0.f;
@@ -925,7 +926,8 @@ hipError_t sfa_launch(const SfaArgs& a, hipStream_t stream)
     if (e != hipSuccess) return e;
     if (a.nsplit > 1) {
         ScopedKernelTimer tm(KID_SFA_COMBINE, stream);
-        hipLaunchKernelGGL(sfa_combine_kernel, dim3(t * hgroups * 16), dim3(256), 0, stream, static_cast<const void*>(a.part_o),
+        auto merge = a.nsplit <= 2 ? sfa_combine_kernel<2> : a.nsplit <= 4 ? sfa_combine_kernel<4> : sfa_combine_kernel<8>;
+        hipLaunchKernelGGL(merge, dim3(t * hgroups * 16), dim3(256), 0, stream, static_cast<const void*>(a.part_o),
                            a.part_ml, a.out, a.nq, a.nsplit, hgroups);
         e = hipGetLastError();
     }
